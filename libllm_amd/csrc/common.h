@@ -1,0 +1,79 @@
+// Shared helpers for the gfx950 kernels: storage types, conversions, wave and block reductions.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#define LLM_DTYPE_F32 0
+#define LLM_DTYPE_BF16 1
+
+#define LLM_OK 0
+#define LLM_ERR_ARG 1        // an argument the kernel refuses (size, dtype, alignment)
+#define LLM_ERR_LAUNCH 2     // the runtime refused the launch
+
+typedef uint16_t bf16_t;     // bfloat16 as raw bits: the upper half of an IEEE float
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+  return __uint_as_float(((uint32_t)v) << 16);
+}
+
+// Round to nearest even; NaN stays NaN.
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+template <typename T> struct Conv;
+template <> struct Conv<float> {
+  static __device__ __forceinline__ float load(const float* p) { return *p; }
+  static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+};
+template <> struct Conv<bf16_t> {
+  static __device__ __forceinline__ float load(const bf16_t* p) { return bf16_to_f32(*p); }
+  static __device__ __forceinline__ void store(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, 64));
+  return v;
+}
+
+// Sum over a block of NT threads (NT a multiple of 64, at most 1024); every thread gets the result.
+// `scratch` needs NT/64 floats of shared memory; the order of additions is fixed.
+template <int NT>
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  v = wave_sum(v);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+#pragma unroll
+  for (int w = 0; w < NT / 64; ++w) total += scratch[w];
+  return total;
+}
+
+template <int NT>
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+  v = wave_max(v);
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = scratch[0];
+#pragma unroll
+  for (int w = 1; w < NT / 64; ++w) total = fmaxf(total, scratch[w]);
+  return total;
+}
+
+static inline int llm_launch_status() {
+  return hipGetLastError() == hipSuccess ? LLM_OK : LLM_ERR_LAUNCH;
+}

@@ -1,0 +1,217 @@
+// Row-wise kernels: embedding gather, residual add + RMS norm, SiLU-mul, bias add, and the fused
+// rotary rotation + cache write.  All arithmetic is float32; storage is float32 or bfloat16.
+#include "common.h"
+
+// ---------------------------------------------------------------------------------- embedding
+// out[m, :] = table[ids[m], :] * scale, written as the float32 residual stream
+// (reference: src/flint/cuda/lookup.cu:30-43).
+template <typename T>
+__global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                             float* __restrict__ out, int H, int V, float scale) {
+  const int m = blockIdx.x;
+  int id = ids[m];
+  if (id < 0 || id >= V) id = 0;   // the host checks ids; never read outside the table
+  const T* row = table + (size_t)id * H;
+  float* dst = out + (size_t)m * H;
+  for (int i = threadIdx.x; i < H; i += blockDim.x) dst[i] = Conv<T>::load(row + i) * scale;
+}
+
+extern "C" int llm_embed(const void* table, int table_dtype, const int* ids, float* out, int M,
+                         int H, int V, float scale, hipStream_t stream) {
+  if (M <= 0) return LLM_OK;
+  if (H <= 0 || V <= 0) return LLM_ERR_ARG;
+  if (table_dtype == LLM_DTYPE_F32)
+    embed_kernel<float><<<M, 256, 0, stream>>>((const float*)table, ids, out, H, V, scale);
+  else if (table_dtype == LLM_DTYPE_BF16)
+    embed_kernel<bf16_t><<<M, 256, 0, stream>>>((const bf16_t*)table, ids, out, H, V, scale);
+  else
+    return LLM_ERR_ARG;
+  return llm_launch_status();
+}
+
+// ---------------------------------------------------------------------------------- add + RMS norm
+// For output row b (input row r = rows ? rows[b] : b):
+//   x = res[r] + delta[r] (stored back into res when delta is given)
+//   out[b] = x * w * 1/sqrt(mean(x^2) + eps)         (src/flint/cuda/rms_norm.cu:45-76)
+template <typename TD, typename TO, int NT>
+__global__ void add_rmsnorm_kernel(float* __restrict__ res, const TD* __restrict__ delta,
+                                   const float* __restrict__ w, float eps, TO* __restrict__ out,
+                                   const int* __restrict__ rows, int H) {
+  __shared__ float scratch[NT / 64];
+  const int b = blockIdx.x;
+  const int r = rows ? rows[b] : b;
+  float* x = res + (size_t)r * H;
+  const TD* d = delta ? delta + (size_t)r * H : nullptr;
+  float ss = 0.f;
+  for (int i = threadIdx.x; i < H; i += NT) {
+    float v = x[i];
+    if (d) {
+      v += Conv<TD>::load(d + i);
+      x[i] = v;
+    }
+    ss += v * v;
+  }
+  ss = block_sum<NT>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+  TO* o = out + (size_t)b * H;
+  for (int i = threadIdx.x; i < H; i += NT) Conv<TO>::store(o + i, x[i] * w[i] * inv);
+}
+
+extern "C" int llm_add_rmsnorm(float* res, const void* delta, int delta_dtype, const float* w,
+                               float eps, void* out, int out_dtype, const int* rows, int n_out,
+                               int H, hipStream_t stream) {
+  if (n_out <= 0) return LLM_OK;
+  if (H <= 0) return LLM_ERR_ARG;
+  constexpr int NT = 256;
+#define LAUNCH(TD, TO) \
+  add_rmsnorm_kernel<TD, TO, NT><<<n_out, NT, 0, stream>>>(res, (const TD*)delta, w, eps, (TO*)out, rows, H)
+  if (delta == nullptr) delta_dtype = out_dtype;
+  if (delta_dtype == LLM_DTYPE_F32 && out_dtype == LLM_DTYPE_F32) LAUNCH(float, float);
+  else if (delta_dtype == LLM_DTYPE_BF16 && out_dtype == LLM_DTYPE_BF16) LAUNCH(bf16_t, bf16_t);
+  else if (delta_dtype == LLM_DTYPE_F32 && out_dtype == LLM_DTYPE_BF16) LAUNCH(float, bf16_t);
+  else if (delta_dtype == LLM_DTYPE_BF16 && out_dtype == LLM_DTYPE_F32) LAUNCH(bf16_t, float);
+  else return LLM_ERR_ARG;
+#undef LAUNCH
+  return llm_launch_status();
+}
+
+// ---------------------------------------------------------------------------------- SiLU-mul
+// out[m, i] = gu[m, i] / (1 + exp(-gu[m, i])) * gu[m, I + i]: the gate is the first half
+// (src/flint/cuda/swiglu.cu:44-49).
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I) {
+  const int m = blockIdx.y;
+  const int i = blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= I) return;
+  const T* row = gu + (size_t)m * 2 * I;
+  const float g = Conv<T>::load(row + i);
+  const float u = Conv<T>::load(row + I + i);
+  Conv<T>::store(out + (size_t)m * I + i, u * g / (1.0f + expf(-g)));
+}
+
+extern "C" int llm_silu_mul(const void* gu, void* out, int dtype, int M, int I, hipStream_t stream) {
+  if (M <= 0) return LLM_OK;
+  if (I <= 0 || M > 65535 * 32) return LLM_ERR_ARG;
+  // grid.y is limited to 65535: fold larger M into several launches
+  for (int m0 = 0; m0 < M; m0 += 65535) {
+    const int mm = (M - m0 < 65535) ? (M - m0) : 65535;
+    dim3 grid((I + 255) / 256, mm);
+    if (dtype == LLM_DTYPE_F32)
+      silu_mul_kernel<float><<<grid, 256, 0, stream>>>((const float*)gu + (size_t)m0 * 2 * I,
+                                                        (float*)out + (size_t)m0 * I, I);
+    else if (dtype == LLM_DTYPE_BF16)
+      silu_mul_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)gu + (size_t)m0 * 2 * I,
+                                                         (bf16_t*)out + (size_t)m0 * I, I);
+    else
+      return LLM_ERR_ARG;
+  }
+  return llm_launch_status();
+}
+
+// ---------------------------------------------------------------------------------- bias add
+template <typename T>
+__global__ void add_bias_kernel(T* __restrict__ x, const float* __restrict__ b, size_t total, int N) {
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (; i < total; i += stride) Conv<T>::store(x + i, Conv<T>::load(x + i) + b[i % N]);
+}
+
+extern "C" int llm_add_bias(void* x, int dtype, const float* b, int M, int N, hipStream_t stream) {
+  if (M <= 0) return LLM_OK;
+  if (N <= 0) return LLM_ERR_ARG;
+  const size_t total = (size_t)M * N;
+  int blocks = (int)((total + 255) / 256);
+  if (blocks > 8192) blocks = 8192;
+  if (dtype == LLM_DTYPE_F32) add_bias_kernel<float><<<blocks, 256, 0, stream>>>((float*)x, b, total, N);
+  else if (dtype == LLM_DTYPE_BF16) add_bias_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)x, b, total, N);
+  else return LLM_ERR_ARG;
+  return llm_launch_status();
+}
+
+// ---------------------------------------------------------------------------------- rotary + cache write
+// One block per token.  Row layout of qkv: [q heads | k heads | v heads], each head_dim wide.
+//   q, k: o[j] = x[j] c - x[j+r/2] s,  o[j+r/2] = x[j+r/2] c + x[j] s  for j < r/2, r = rot_dim
+//         (rotate-half pairing, src/libllm/llama.cc:151-176); dims >= r pass through.
+//   q is rotated in place; k (rotated) and v go to the sequence's page of the cache:
+//   page = table[slot, pos / PAGE], element [page, kv_head, pos % PAGE, d].
+template <typename T, int PAGE>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride, const float* __restrict__ bias,
+                                     int n_heads, int n_kv, int hd, const float* __restrict__ cos_t,
+                                     const float* __restrict__ sin_t, int rot_dim,
+                                     const int* __restrict__ tok_pos, const int* __restrict__ tok_seq,
+                                     const int* __restrict__ seq_slot, const int* __restrict__ table,
+                                     int table_stride, T* __restrict__ k_pages, T* __restrict__ v_pages,
+                                     int write_kv) {
+  const int m = blockIdx.x;
+  const int pos = tok_pos[m];
+  T* row = qkv + (size_t)m * row_stride;
+  const int half = rot_dim / 2;
+  const int pass = hd - rot_dim;                 // dims that do not rotate
+  const int per_head = half + pass;              // work items per rotating head
+  const int n_rot_heads = n_heads + (write_kv ? n_kv : 0);
+  size_t page_base = 0;
+  if (write_kv) {
+    const int slot = seq_slot[tok_seq[m]];
+    const int page = table[(size_t)slot * table_stride + pos / PAGE];
+    page_base = ((size_t)page * n_kv) * PAGE * hd + (size_t)(pos % PAGE) * hd;
+  }
+  const float* c = cos_t + (size_t)pos * half;
+  const float* s = sin_t + (size_t)pos * half;
+  const int rot_items = n_rot_heads * per_head;
+  for (int it = threadIdx.x; it < rot_items; it += blockDim.x) {
+    const int h = it / per_head;
+    const int j = it % per_head;
+    T* x = row + (size_t)h * hd;
+    const float* b = bias ? bias + (size_t)h * hd : nullptr;
+    const bool is_k = h >= n_heads;
+    T* dst = is_k ? k_pages + page_base + (size_t)(h - n_heads) * PAGE * hd : x;
+    if (j < half) {
+      float x1 = Conv<T>::load(x + j), x2 = Conv<T>::load(x + j + half);
+      if (b) { x1 += b[j]; x2 += b[j + half]; }
+      const float cj = c[j], sj = s[j];
+      Conv<T>::store(dst + j, x1 * cj - x2 * sj);
+      Conv<T>::store(dst + j + half, x2 * cj + x1 * sj);
+    } else {
+      const int d = rot_dim + (j - half);
+      float v = Conv<T>::load(x + d);
+      if (b) v += b[d];
+      Conv<T>::store(dst + d, v);
+    }
+  }
+  if (write_kv) {
+    const T* vrow = row + (size_t)(n_heads + n_kv) * hd;
+    const float* b = bias ? bias + (size_t)(n_heads + n_kv) * hd : nullptr;
+    for (int it = threadIdx.x; it < n_kv * hd; it += blockDim.x) {
+      const int h = it / hd, d = it % hd;
+      float v = Conv<T>::load(vrow + it);
+      if (b) v += b[it];
+      Conv<T>::store(v_pages + page_base + (size_t)h * PAGE * hd + d, v);
+    }
+  }
+}
+
+extern "C" int llm_rope_kv_write(void* qkv, int dtype, int row_stride, const float* bias, int n_heads,
+                                 int n_kv, int hd, const float* cos_t, const float* sin_t, int rot_dim,
+                                 const int* tok_pos, const int* tok_seq, const int* seq_slot,
+                                 const int* table, int table_stride, void* k_pages, void* v_pages,
+                                 int page_size, int write_kv, int M, hipStream_t stream) {
+  if (M <= 0) return LLM_OK;
+  if (page_size != 64 || hd <= 0 || n_heads <= 0 || n_kv < 0 || rot_dim < 0 || rot_dim > hd ||
+      (rot_dim & 1))
+    return LLM_ERR_ARG;
+  if (rot_dim > 0 && (cos_t == nullptr || sin_t == nullptr)) return LLM_ERR_ARG;
+  const int width = (n_heads + (write_kv ? 2 * n_kv : 0)) * hd;
+  if (row_stride < width) return LLM_ERR_ARG;
+  if (write_kv && (!k_pages || !v_pages || !table || !seq_slot || !tok_seq)) return LLM_ERR_ARG;
+  if (dtype == LLM_DTYPE_F32)
+    rope_kv_write_kernel<float, 64><<<M, 256, 0, stream>>>(
+        (float*)qkv, row_stride, bias, n_heads, n_kv, hd, cos_t, sin_t, rot_dim, tok_pos, tok_seq,
+        seq_slot, table, table_stride, (float*)k_pages, (float*)v_pages, write_kv);
+  else if (dtype == LLM_DTYPE_BF16)
+    rope_kv_write_kernel<bf16_t, 64><<<M, 256, 0, stream>>>(
+        (bf16_t*)qkv, row_stride, bias, n_heads, n_kv, hd, cos_t, sin_t, rot_dim, tok_pos, tok_seq,
+        seq_slot, table, table_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, write_kv);
+  else
+    return LLM_ERR_ARG;
+  return llm_launch_status();
+}

@@ -1,0 +1,69 @@
+// True 32-bit matrix product C[M,N] = A[M,K] * W[N,K]^T with float32 storage and float32 FMA
+// accumulation in a fixed order over K (no matrix-core reduced-precision mode).  Tiled through
+// shared memory: 64x64 output tile per block of 256 threads, 4x4 outputs per thread.
+#include "common.h"
+
+template <int BM, int BN, int BK>
+__global__ __launch_bounds__(256) void gemm_f32_kernel(const float* __restrict__ A,
+                                                        const float* __restrict__ W,
+                                                        float* __restrict__ C, int M, int N, int K) {
+  __shared__ float As[BK][BM + 4];
+  __shared__ float Ws[BK][BN + 4];
+  const int tid = threadIdx.x;
+  const int tx = tid % 16, ty = tid / 16;
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * BN;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+
+  for (int k0 = 0; k0 < K; k0 += BK) {
+#pragma unroll
+    for (int e = tid; e < BM * BK; e += 256) {
+      const int r = e / BK, c = e % BK;
+      const int gm = m0 + r, gk = k0 + c;
+      As[c][r] = (gm < M && gk < K) ? A[(size_t)gm * K + gk] : 0.f;
+    }
+#pragma unroll
+    for (int e = tid; e < BN * BK; e += 256) {
+      const int r = e / BK, c = e % BK;
+      const int gn = n0 + r, gk = k0 + c;
+      Ws[c][r] = (gn < N && gk < K) ? W[(size_t)gn * K + gk] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int kk = 0; kk < BK; ++kk) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[kk][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = Ws[kk][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int gm = m0 + ty * 4 + i;
+    if (gm >= M) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int gn = n0 + tx * 4 + j;
+      if (gn < N) C[(size_t)gm * N + gn] = acc[i][j];
+    }
+  }
+}
+
+extern "C" int llm_gemm_f32(const float* A, const float* W, float* C, int M, int N, int K,
+                            hipStream_t stream) {
+  if (M <= 0 || N <= 0) return LLM_OK;
+  if (K <= 0) return LLM_ERR_ARG;
+  const int gy = (M + 63) / 64, gx = (N + 63) / 64;
+  if (gy > 65535) return LLM_ERR_ARG;
+  gemm_f32_kernel<64, 64, 16><<<dim3(gx, gy), 256, 0, stream>>>(A, W, C, M, N, K);
+  return llm_launch_status();
+}

@@ -1,0 +1,141 @@
+"""The generation loop above the step function.
+
+The reference generates for one sequence: prefill, then decode token by token, ending when the
+sampled token is a stop token, which is not emitted (src/libllm/generator.cc:140-156).  Here many
+requests are served: they are cut into batches that fit the cache, each batch starts together with
+prompts of unequal lengths in one step, goes on one token per live sequence, sequences that end
+leave the batch and give their slot back, and batches follow one another until all are served.
+"""
+from dataclasses import dataclass, field
+from typing import Callable, Iterable, List, Optional, Sequence
+
+from ..errors import RequestError
+from ..sampling import Sampler, SamplingParams
+from .step import StepEntry
+
+
+def plan_batches(prompt_lens: Sequence[int], max_new_tokens: int, max_batch: int,
+                 page_budget: int, page: int, max_position: int) -> List[List[int]]:
+    """Cuts request indices into consecutive batches: at most ``max_batch`` requests each, and
+    the pages every request may grow to (prompt plus ``max_new_tokens``, capped by
+    ``max_position``) fit ``page_budget`` together."""
+    if max_batch <= 0:
+        raise RequestError("max_batch must be positive")
+    batches, cur, used = [], [], 0
+    for i, n in enumerate(prompt_lens):
+        if n <= 0:
+            raise RequestError("request %d has an empty prompt" % i)
+        if n > max_position:
+            raise RequestError("request %d: a prompt of %d tokens exceeds max_position_embeddings %d"
+                               % (i, n, max_position))
+        need = (min(n + max_new_tokens, max_position) + page - 1) // page
+        if need > page_budget:
+            raise RequestError("request %d needs %d cache pages but the cache has %d"
+                               % (i, need, page_budget))
+        if cur and (len(cur) >= max_batch or used + need > page_budget):
+            batches.append(cur)
+            cur, used = [], 0
+        cur.append(i)
+        used += need
+    if cur:
+        batches.append(cur)
+    return batches
+
+
+@dataclass
+class SequenceState:
+    index: int                       # position of the request among all requests
+    prompt_len: int
+    output: List[int] = field(default_factory=list)
+    finished: bool = False
+    reason: str = ""
+
+    def accept(self, token: int, stop: set, max_new_tokens: int, max_position: int) -> bool:
+        """Takes the token sampled for this sequence; returns True if the sequence goes on.
+        A stop token ends it and is not emitted; so does the token budget or the position limit."""
+        if token in stop:
+            self.finished, self.reason = True, "stop"
+            return False
+        self.output.append(token)
+        if len(self.output) >= max_new_tokens:
+            self.finished, self.reason = True, "length"
+            return False
+        if self.prompt_len + len(self.output) >= max_position:
+            self.finished, self.reason = True, "max_position"
+            return False
+        return True
+
+
+class Generator:
+    """``engine`` needs ``step(entries)`` and ``end(requests)``; ``sampler`` needs
+    ``sample(logits, params, streams, counters)``."""
+
+    def __init__(self, engine, sampler, stop_tokens: Iterable[int], max_position: int,
+                 page_budget: int, page: int, max_batch: int = 64):
+        self.engine = engine
+        self.sampler = sampler
+        self.stop_tokens = set(stop_tokens)
+        self.max_position = max_position
+        self.page_budget = page_budget
+        self.page = page
+        self.max_batch = max_batch
+        self._serial = 0
+
+    def generate(self, prompts: Sequence[Sequence[int]], params: SamplingParams,
+                 max_new_tokens: int = 256, stop_tokens: Optional[Iterable[int]] = None,
+                 on_token: Optional[Callable[[int, int], None]] = None) -> List[List[int]]:
+        """Tokens generated for each prompt, in the order of the prompts.  ``on_token(index,
+        token)`` is called for every emitted token as soon as it is known."""
+        results: List[List[int]] = [[] for _ in prompts]
+        for index, token in self.stream(prompts, params, max_new_tokens, stop_tokens):
+            results[index].append(token)
+            if on_token is not None:
+                on_token(index, token)
+        return results
+
+    def stream(self, prompts: Sequence[Sequence[int]], params: SamplingParams,
+               max_new_tokens: int = 256, stop_tokens: Optional[Iterable[int]] = None):
+        """Yields ``(prompt index, token)`` for every emitted token, step by step."""
+        if max_new_tokens <= 0:
+            return
+        stop = self.stop_tokens if stop_tokens is None else set(stop_tokens)
+        lens = [len(p) for p in prompts]
+        batches = plan_batches(lens, max_new_tokens, self.max_batch, self.page_budget, self.page,
+                               self.max_position)
+        for batch in batches:
+            yield from self._run_batch(batch, prompts, params, max_new_tokens, stop)
+
+    def _run_batch(self, batch, prompts, params, max_new_tokens, stop):
+        self._serial += 1
+        states = [SequenceState(i, len(prompts[i])) for i in batch]
+        name = {st.index: ("gen", self._serial, st.index) for st in states}
+        live = list(states)
+        try:
+            entries = [StepEntry(name[st.index], list(prompts[st.index]), [st.prompt_len - 1])
+                       for st in live]
+            while True:
+                logits = self.engine.step(entries)
+                tokens = self.sampler.sample(logits, params, [st.index for st in live],
+                                             [len(st.output) for st in live])
+                ended, going, emitted = [], [], []
+                for st, tok in zip(live, tokens):
+                    n_before = len(st.output)
+                    (going if st.accept(tok, stop, max_new_tokens, self.max_position) else ended).append(st)
+                    if len(st.output) > n_before:
+                        emitted.append((st.index, tok))
+                if ended:
+                    self.engine.end([name[st.index] for st in ended])
+                live = going
+                for item in emitted:
+                    yield item
+                if not live:
+                    break
+                entries = [StepEntry(name[st.index], [st.output[-1]], [0]) for st in live]
+        finally:
+            held = [name[st.index] for st in live if self._holds(name[st.index])]
+            if held:
+                self.engine.end(held)
+
+    def _holds(self, request) -> bool:
+        holds = getattr(self.engine, "holds", None)
+        return True if holds is None else holds(request)

@@ -1,0 +1,128 @@
+"""A decoder assembled from a ModelSpec: embedding, scheduled blocks, final norm, output matrix.
+
+This class is the same for every architecture; what differs between architectures is the
+ModelSpec their configuration produces (src/libllm/llama.cc:273-312 is the reference's fixed
+counterpart for Llama).
+"""
+from typing import Dict, List, Optional
+
+import torch
+
+from ..config.spec import ModelSpec, validate_schedule
+from ..errors import ConfigError
+from ..parts import (Stream, StepContext, WeightDecl, build_block, build_feed_forward, build_mixer,
+                     build_norm)
+
+
+def _build_layers(spec: ModelSpec):
+    blocks = []
+    for ls in spec.layers:
+        mixer = build_mixer(ls.mixer)
+        ff = build_feed_forward(ls.feed_forward)
+        norms = [build_norm(n) for n in ls.norms]
+        blocks.append(build_block(ls.block, mixer, ff, norms))
+    return blocks
+
+
+def _layer_decls(block, ls):
+    out = {}
+    groups = [("mixer", block.mixer), ("feed_forward", block.feed_forward)]
+    groups += [("norm%d" % i, n) for i, n in enumerate(block.norms)]
+    for role, part in groups:
+        decls = part.weights()
+        if decls and role not in ls.prefixes:
+            raise ConfigError("layer record has no tensor-name prefix for %r" % role)
+        for rel, decl in decls.items():
+            out[ls.prefixes[role] + rel] = (part, rel, decl)
+    return out
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec):
+        validate_schedule(spec)
+        self.spec = spec
+        self.blocks = _build_layers(spec)
+        self.final_norm = build_norm(spec.final_norm)
+        self.embed_table: Optional[torch.Tensor] = None
+        self.head_weight: Optional[torch.Tensor] = None
+        self._decls = None
+
+    # ---- weights
+    def _collect(self):
+        if self._decls is None:
+            s = self.spec
+            d = {}
+            d[s.embedding.tensor] = (None, "embedding", WeightDecl((s.embedding.vocab, s.embedding.width)))
+            if not s.head.tied:
+                d[s.head.tensor] = (None, "head", WeightDecl((s.head.vocab, s.head.width)))
+            for block, ls in zip(self.blocks, s.layers):
+                for name, item in _layer_decls(block, ls).items():
+                    if name in d:
+                        raise ConfigError("tensor %r is declared by two parts" % name)
+                    d[name] = item
+            for rel, decl in self.final_norm.weights().items():
+                d[s.final_norm_prefix + rel] = (self.final_norm, rel, decl)
+            self._decls = d
+        return self._decls
+
+    def declared(self) -> Dict[str, WeightDecl]:
+        return {name: item[2] for name, item in self._collect().items()}
+
+    def bind(self, tensors: Dict[str, torch.Tensor], ops, dtype) -> None:
+        s = self.spec
+        per_part: Dict[int, Dict[str, torch.Tensor]] = {}
+        parts = {}
+        for name, (part, rel, _decl) in self._collect().items():
+            if part is None:
+                continue
+            per_part.setdefault(id(part), {})[rel] = tensors[name]
+            parts[id(part)] = part
+        for pid, part in parts.items():
+            part.bind(per_part[pid], ops, dtype)
+        for block in self.blocks:                       # parts without tensors still get ops
+            for part in [block.mixer, block.feed_forward] + list(block.norms):
+                if id(part) not in parts:
+                    part.bind({}, ops, dtype)
+        self.embed_table = tensors[s.embedding.tensor]
+        self.head_weight = self.embed_table if s.head.tied else tensors[s.head.tensor]
+
+    # ---- what the cache has to hold
+    def cache_needs(self):
+        needs = [None] * self.spec.n_cache_entries()
+        for e in self.spec.schedule:
+            if e.writes:
+                needs[e.cache] = self.blocks[e.layer].mixer.cache_need()
+        return needs
+
+    def state_needs(self):
+        needs = [None] * self.spec.n_cache_entries()
+        for e in self.spec.schedule:
+            if e.writes:
+                needs[e.cache] = self.blocks[e.layer].mixer.state_need()
+        return needs
+
+    def graph_safe(self) -> bool:
+        """True if no part reads host-side step data, so a step can be captured and replayed."""
+        for block in self.blocks:
+            for part in [block.mixer, block.feed_forward] + list(block.norms):
+                if not getattr(part, "graph_safe", False):
+                    return False
+        return getattr(self.final_norm, "graph_safe", False)
+
+    # ---- one step over packed rows
+    def forward(self, ctx: StepContext, want_rows: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+        """Runs every token of the step through the schedule; returns float32 logits
+        ``[len(want_rows), vocab]`` (None if no row is wanted)."""
+        s = self.spec
+        res = ctx.ops.embed(self.embed_table, ctx.tokens, s.embedding.scale)
+        stream = Stream(res)
+        for entry in s.schedule:
+            self.blocks[entry.layer].forward(ctx, stream, entry)
+        if want_rows is None or want_rows.numel() == 0:
+            return None
+        h = self.final_norm.add_norm(ctx, stream, rows=want_rows)
+        return ctx.ops.linear(h, self.head_weight, None, torch.float32)
+
+
+def declared_weights(spec: ModelSpec) -> Dict[str, WeightDecl]:
+    return DecoderModel(spec).declared()

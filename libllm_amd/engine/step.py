@@ -1,0 +1,221 @@
+"""The step function: runs the tokens it is given, as one batch, from the cache.
+
+A step carries, for each of its requests, the next tokens of that request (a whole prompt, a part
+of it, or one decoded token) and the places among them whose logits are wanted.  All rows of all
+requests are packed one after another; no padding enters the model.  The reference has two entry
+points for one sequence, prefill and decode (src/libllm/llama.cc:349-368); this is their
+generalisation to unequal batches.
+"""
+from dataclasses import dataclass, field
+from typing import Dict, Hashable, List, Optional, Sequence
+
+import numpy as np
+import torch
+
+from ..cache import PAGE, SequenceCache
+from ..errors import CacheError, RequestError
+from ..parts import StepContext
+from .model import DecoderModel
+
+
+@dataclass
+class StepEntry:
+    request: Hashable
+    tokens: Sequence[int]
+    want: Sequence[int] = ()          # indices into ``tokens`` whose logits are returned
+
+
+class Engine:
+    """Owns a bound model, its cache and the step function."""
+
+    GRAPH_BATCHES = (1, 2, 4, 8, 16, 32, 64)
+
+    def __init__(self, model: DecoderModel, ops, dtype: torch.dtype, max_tokens: int,
+                 max_slots: Optional[int] = None, use_graphs: bool = True):
+        self.model = model
+        self.ops = ops
+        self.dtype = dtype
+        self.device = ops.device
+        self.vocab = model.spec.vocab
+        self.cache = SequenceCache(model.cache_needs(), model.state_needs(), max_tokens,
+                                   model.spec.max_position, dtype, self.device, max_slots)
+        self.use_graphs = bool(use_graphs) and ops.supports_graphs and model.graph_safe()
+        self._graphs: Dict[int, "_DecodeGraph"] = {}
+        self.steps_run = 0
+
+    # ---- requests
+    def live_requests(self):
+        return self.cache.slots.live()
+
+    def end(self, requests) -> None:
+        for r in requests:
+            self.cache.release(r)
+
+    def holds(self, request) -> bool:
+        return self.cache.holds(request)
+
+    def length(self, request) -> int:
+        return self.cache.length(self.cache.slot_of(request))
+
+    # ---- the step
+    def step(self, entries: List[StepEntry]) -> Optional[torch.Tensor]:
+        """Returns float32 logits ``[wanted, vocab]`` in the order of the entries and of their
+        ``want`` lists, or None if nothing is wanted."""
+        if not entries:
+            raise RequestError("a step needs at least one entry")
+        seen = set()
+        for e in entries:
+            if e.request in seen:
+                raise RequestError("request %r appears twice in one step" % (e.request,))
+            seen.add(e.request)
+            if len(e.tokens) == 0:
+                raise RequestError("request %r brings no tokens" % (e.request,))
+            lo, hi = min(e.tokens), max(e.tokens)
+            if lo < 0 or hi >= self.vocab:
+                raise RequestError("request %r has a token id outside [0, %d)" % (e.request, self.vocab))
+            for w in e.want:
+                if not 0 <= w < len(e.tokens):
+                    raise RequestError("request %r wants row %d of %d" % (e.request, w, len(e.tokens)))
+        cache = self.cache
+        fresh = [e.request for e in entries if not cache.holds(e.request)]
+        if len(fresh) > cache.slots.n_free:
+            raise CacheError("no free slot: %d requests start, %d slots free"
+                             % (len(fresh), cache.slots.n_free))
+        plan = [(cache.slot_of(e.request) if cache.holds(e.request) else None,
+                 cache.length(cache.slot_of(e.request)) if cache.holds(e.request) else 0,
+                 len(e.tokens)) for e in entries]
+        for slot, length, n_new in plan:
+            if length + n_new > cache.max_position:
+                raise CacheError("a sequence of %d tokens exceeds max_position_embeddings %d"
+                                 % (length + n_new, cache.max_position))
+        if not cache.can_reserve(plan):
+            raise CacheError("the cache is full: this step needs more pages than are free "
+                             "(max_tokens %d, %d tokens held)"
+                             % (cache.n_pages * PAGE, cache.tokens_held()))
+        slots = []
+        for e in entries:
+            slot = cache.slot_of(e.request) if cache.holds(e.request) else cache.admit(e.request)
+            cache.reserve(slot, len(e.tokens))
+            slots.append(slot)
+        cache.flush()
+
+        lens = [len(e.tokens) for e in entries]
+        pos0 = [cache.length(s) for s in slots]
+        want_all_single = all(n == 1 for n in lens) and all(list(e.want) == [0] for e in entries)
+        if self.use_graphs and want_all_single and len(entries) <= self.GRAPH_BATCHES[-1]:
+            logits = self._graph_step(entries, slots, pos0)
+        else:
+            ctx, want_rows = self._context(entries, slots, lens, pos0)
+            logits = self.model.forward(ctx, want_rows)
+        for s, n in zip(slots, lens):
+            cache.commit(s, n)
+        cache.flush()
+        self.steps_run += 1
+        return logits
+
+    # ---- building the packed batch
+    def _context(self, entries, slots, lens, pos0):
+        b = len(entries)
+        m = sum(lens)
+        starts = np.zeros(b + 1, dtype=np.int64)
+        starts[1:] = np.cumsum(lens)
+        tokens = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
+        tok_seq = np.repeat(np.arange(b, dtype=np.int64), lens)
+        tok_pos = np.arange(m, dtype=np.int64) - starts[tok_seq] + np.asarray(pos0, dtype=np.int64)[tok_seq]
+        want = [int(starts[i]) + int(w) for i, e in enumerate(entries) for w in e.want]
+        packed = np.concatenate([tokens, tok_pos, tok_seq, starts, np.asarray(slots, dtype=np.int64),
+                                 np.asarray(pos0, dtype=np.int64),
+                                 np.asarray(want, dtype=np.int64)]).astype(np.int32)
+        dev = self.ops.upload_int32(packed)
+        ctx = StepContext(self.ops, self.dtype, m, b)
+        o = 0
+        ctx.tokens = dev[o:o + m]; o += m
+        ctx.tok_pos = dev[o:o + m]; o += m
+        ctx.tok_seq = dev[o:o + m]; o += m
+        ctx.seq_start = dev[o:o + b + 1]; o += b + 1
+        ctx.seq_slot = dev[o:o + b]; o += b
+        ctx.seq_pos0 = dev[o:o + b]; o += b
+        want_rows = dev[o:o + len(want)]
+        ctx.seq_lens = list(lens)
+        ctx.seq_pos0_host = list(pos0)
+        ctx.seq_slot_host = list(slots)
+        ctx.max_new = max(lens)
+        ctx.max_ctx = max(p + n for p, n in zip(pos0, lens))
+        ctx.decode = all(n == 1 for n in lens)
+        self._attach_cache(ctx)
+        return ctx, want_rows
+
+    def _attach_cache(self, ctx):
+        for entry in range(self.model.spec.n_cache_entries()):
+            view = self.cache.kv_view(entry)
+            if view is not None:
+                ctx._kv[entry] = view
+            if entry in self.cache.state:
+                ctx._state[entry] = self.cache.state[entry]
+
+    # ---- decoding one token per sequence through a captured graph
+    def _graph_step(self, entries, slots, pos0):
+        b = len(entries)
+        bucket = next(g for g in self.GRAPH_BATCHES if g >= b)
+        graph = self._graphs.get(bucket)
+        if graph is None:
+            graph = _DecodeGraph(self, bucket)
+            self._graphs[bucket] = graph
+        return graph.run([e.tokens[0] for e in entries], slots, pos0)
+
+
+class _DecodeGraph:
+    """One captured decode step for a batch of exactly ``bucket`` rows.  Rows beyond the live
+    sequences point at the cache's sink slot and page, so they change nothing that is read."""
+
+    def __init__(self, engine: Engine, bucket: int):
+        self.engine = engine
+        self.bucket = bucket
+        ops = engine.ops
+        b = bucket
+        self.host = np.zeros(7 * b + 1, dtype=np.int32)
+        self.static = ops.upload_int32(self.host)
+        ctx = StepContext(ops, engine.dtype, b, b)
+        o = 0
+        ctx.tokens = self.static[o:o + b]; o += b
+        ctx.tok_pos = self.static[o:o + b]; o += b
+        ctx.tok_seq = self.static[o:o + b]; o += b
+        ctx.seq_start = self.static[o:o + b + 1]; o += b + 1
+        ctx.seq_slot = self.static[o:o + b]; o += b
+        ctx.seq_pos0 = self.static[o:o + b]; o += b
+        self.want_rows = self.static[o:o + b]
+        ctx.max_new = 1
+        ctx.max_ctx = engine.cache.pages_per_seq * PAGE
+        ctx.decode = True
+        ctx.captured = True
+        engine._attach_cache(ctx)
+        self.ctx = ctx
+        self._fill([0] * b, [engine.cache.sink_slot] * b, [0] * b)
+        self.logits = None
+        self.graph = ops.capture(self._body)
+
+    def _body(self):
+        self.logits = self.engine.model.forward(self.ctx, self.want_rows)
+
+    def _fill(self, tokens, slots, pos0):
+        b = self.bucket
+        n = len(tokens)
+        sink = self.engine.cache.sink_slot
+        h = self.host
+        h[0:b] = 0
+        h[0:n] = tokens
+        h[b:2 * b] = 0
+        h[b:b + n] = pos0
+        h[2 * b:3 * b] = np.arange(b)
+        h[3 * b:4 * b + 1] = np.arange(b + 1)
+        h[4 * b + 1:5 * b + 1] = sink
+        h[4 * b + 1:4 * b + 1 + n] = slots
+        h[5 * b + 1:6 * b + 1] = 0
+        h[5 * b + 1:5 * b + 1 + n] = pos0
+        h[6 * b + 1:7 * b + 1] = np.arange(b)
+        self.static.copy_(torch.from_numpy(h))
+
+    def run(self, tokens, slots, pos0):
+        self._fill(tokens, slots, pos0)
+        self.graph.replay()
+        return self.logits[:len(tokens)]

@@ -1,0 +1,140 @@
+"""Building and loading the HIP kernels: one shared library, compiled with hipcc for gfx950.
+
+The library lives beside the sources (``libllm_amd/_lib``); if that folder cannot be written, a
+per-user folder under the system's temporary directory is used.  A stored hash of the sources
+decides whether what is built is current.  Nothing here falls back to another implementation: if
+the library cannot be loaded or built, KernelError says why.
+"""
+import ctypes
+import hashlib
+import os
+import shutil
+import subprocess
+import sys
+import tempfile
+import time
+from concurrent.futures import ThreadPoolExecutor
+from typing import List, Optional
+
+from ..errors import KernelError
+
+ARCH = "gfx950"
+_HERE = os.path.dirname(os.path.abspath(__file__))
+CSRC = os.path.join(os.path.dirname(_HERE), "csrc")
+LIB_NAME = "libllm_amd_hip.so"
+# packed FP32 instructions stay switched off for every kernel of this library
+FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+
+_lib: Optional[ctypes.CDLL] = None
+
+
+def sources() -> List[str]:
+    return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
+
+
+def source_hash() -> str:
+    h = hashlib.sha256()
+    for path in sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC)
+                       if f.endswith((".hip", ".h"))):
+        h.update(os.path.basename(path).encode())
+        with open(path, "rb") as f:
+            h.update(f.read())
+    h.update(" ".join(FLAGS).encode())
+    return h.hexdigest()[:20]
+
+
+def _say(msg: str) -> None:
+    print("[libllm_amd] " + msg, file=sys.stderr, flush=True)
+
+
+def _hipcc() -> Optional[str]:
+    for cand in (os.environ.get("HIPCC"), shutil.which("hipcc"),
+                 os.path.join(os.environ.get("ROCM_PATH", "/opt/rocm"), "bin", "hipcc")):
+        if cand and os.path.isfile(cand):
+            return cand
+    return None
+
+
+def _lib_dirs() -> List[str]:
+    in_tree = os.path.join(os.path.dirname(_HERE), "_lib")
+    uid = os.getuid() if hasattr(os, "getuid") else 0
+    return [in_tree, os.path.join(tempfile.gettempdir(), "libllm_amd-%d" % uid)]
+
+
+def _writable(d: str) -> bool:
+    try:
+        os.makedirs(d, exist_ok=True)
+        probe = os.path.join(d, ".probe-%d" % os.getpid())
+        with open(probe, "w"):
+            pass
+        os.remove(probe)
+        return True
+    except OSError:
+        return False
+
+
+def _current(d: str, want: str) -> bool:
+    so, stamp = os.path.join(d, LIB_NAME), os.path.join(d, LIB_NAME + ".hash")
+    if not (os.path.isfile(so) and os.path.isfile(stamp)):
+        return False
+    with open(stamp, "r") as f:
+        return f.read().strip() == want
+
+
+def build(force: bool = True, verbose: bool = True) -> str:
+    """Compiles every kernel source and links the library; returns its path."""
+    want = source_hash()
+    if not force:
+        for d in _lib_dirs():
+            if _current(d, want):
+                return os.path.join(d, LIB_NAME)
+    hipcc = _hipcc()
+    if hipcc is None:
+        raise KernelError("the HIP kernels are not built and hipcc was not found (looked at $HIPCC, "
+                          "PATH and $ROCM_PATH/bin)")
+    target = next((d for d in _lib_dirs() if _writable(d)), None)
+    if target is None:
+        raise KernelError("no writable folder for the kernel library (tried %s)" % ", ".join(_lib_dirs()))
+    objdir = os.path.join(target, "obj")
+    os.makedirs(objdir, exist_ok=True)
+    srcs = sources()
+    t0 = time.time()
+    if verbose:
+        _say("compiling %d HIP sources for %s into %s" % (len(srcs), ARCH, target))
+
+    def compile_one(src):
+        obj = os.path.join(objdir, os.path.basename(src)[:-4] + ".o")
+        cmd = [hipcc] + FLAGS + ["-I", CSRC, "-c", src, "-o", obj]
+        proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if proc.returncode != 0:
+            raise KernelError("hipcc failed on %s:\n%s" % (os.path.basename(src), proc.stdout[-4000:]))
+        if verbose:
+            _say("  compiled %s (%.0f s since start)" % (os.path.basename(src), time.time() - t0))
+        return obj
+
+    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+        objs = list(pool.map(compile_one, srcs))
+    tmp_so = os.path.join(target, LIB_NAME + ".tmp-%d" % os.getpid())
+    cmd = [hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", tmp_so] + objs
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise KernelError("linking the kernel library failed:\n%s" % proc.stdout[-4000:])
+    os.replace(tmp_so, os.path.join(target, LIB_NAME))
+    with open(os.path.join(target, LIB_NAME + ".hash"), "w") as f:
+        f.write(want)
+    if verbose:
+        _say("built %s in %.0f s" % (LIB_NAME, time.time() - t0))
+    return os.path.join(target, LIB_NAME)
+
+
+def load() -> ctypes.CDLL:
+    """The kernel library; built first if no current build exists."""
+    global _lib
+    if _lib is None:
+        path = build(force=False)
+        try:
+            _lib = ctypes.CDLL(path)
+        except OSError as e:
+            raise KernelError("cannot load %s: %s" % (path, e))
+    return _lib

@@ -1,0 +1,245 @@
+"""Host side of the kernels: checks every operand, then launches on the current HIP stream.
+
+This is the only implementation of the operations on the product path.  It needs a GPU and the
+built kernel library; without either it raises KernelError.  Matrix products in bfloat16 with many
+rows go to the vendor library through ``torch.matmul`` (the reference uses its vendor's library
+for them as well, src/flint/cuda/gemm_cublas.cc:160-197); every other operation is a kernel of
+``csrc``.
+"""
+import ctypes
+from typing import List, Optional
+
+import numpy as np
+import torch
+
+from ..errors import KernelError
+from . import build
+
+_F32, _BF16 = 0, 1
+_vp, _i, _f = ctypes.c_void_p, ctypes.c_int, ctypes.c_float
+_u64 = ctypes.c_ulonglong
+
+
+def _code(dtype: torch.dtype) -> int:
+    if dtype == torch.float32:
+        return _F32
+    if dtype == torch.bfloat16:
+        return _BF16
+    raise KernelError("unsupported storage dtype %s (float32 and bfloat16 only)" % dtype)
+
+
+_SIGNATURES = {
+    "llm_embed": [_vp, _i, _vp, _vp, _i, _i, _i, _f, _vp],
+    "llm_add_rmsnorm": [_vp, _vp, _i, _vp, _f, _vp, _i, _vp, _i, _i, _vp],
+    "llm_silu_mul": [_vp, _vp, _i, _i, _i, _vp],
+    "llm_add_bias": [_vp, _i, _vp, _i, _i, _vp],
+    "llm_rope_kv_write": [_vp, _i, _i, _vp, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp,
+                          _vp, _i, _i, _i, _vp],
+    "llm_gemm_f32": [_vp, _vp, _vp, _i, _i, _i, _vp],
+    "llm_attention_ref": [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
+                          _f, _i, _vp],
+    "llm_argmax": [_vp, _vp, _i, _i, _vp],
+    "llm_sample": [_vp, _vp, _i, _i, _f, _i, _f, _u64, _vp, _vp, _vp],
+}
+
+
+class HipOps:
+    supports_graphs = True
+
+    def __init__(self, device: Optional[str] = None):
+        if not torch.cuda.is_available():
+            raise KernelError("no GPU is visible: this library runs on an AMD GPU only")
+        self.device = torch.device(device or "cuda:0")
+        if self.device.type != "cuda":
+            raise KernelError("device %s is not a GPU" % (self.device,))
+        self.lib = build.load()
+        for name, argtypes in _SIGNATURES.items():
+            try:
+                fn = getattr(self.lib, name)
+            except AttributeError:
+                raise KernelError("the kernel library lacks %s; rebuild it" % name)
+            fn.argtypes = argtypes
+            fn.restype = _i
+        torch.backends.cuda.matmul.allow_tf32 = False
+        self.fast_attention = True
+        self.fast_gemm = True
+
+    # ---- helpers
+    def _stream(self):
+        return torch.cuda.current_stream(self.device).cuda_stream
+
+    @staticmethod
+    def _check(status: int, what: str):
+        if status != 0:
+            raise KernelError("%s: %s" % (what, {1: "the kernel refuses these operands",
+                                                 2: "the launch failed"}.get(status, "error %d" % status)))
+
+    def _dev(self, t: torch.Tensor, what: str, dtype=None, shape=None):
+        if t.device != self.device:
+            raise KernelError("%s lies on %s, not on %s" % (what, t.device, self.device))
+        if not t.is_contiguous():
+            raise KernelError("%s is not contiguous" % what)
+        if dtype is not None and t.dtype != dtype:
+            raise KernelError("%s has dtype %s, expected %s" % (what, t.dtype, dtype))
+        if shape is not None and tuple(t.shape) != tuple(shape):
+            raise KernelError("%s has shape %s, expected %s" % (what, tuple(t.shape), tuple(shape)))
+        return t.data_ptr()
+
+    def upload_int32(self, arr: np.ndarray) -> torch.Tensor:
+        return torch.from_numpy(np.ascontiguousarray(arr, dtype=np.int32)).to(self.device)
+
+    def capture(self, body):
+        """Runs ``body`` once to warm up, then captures it into a HIP graph."""
+        side = torch.cuda.Stream(self.device)
+        side.wait_stream(torch.cuda.current_stream(self.device))
+        with torch.cuda.stream(side):
+            body()
+        torch.cuda.current_stream(self.device).wait_stream(side)
+        torch.cuda.synchronize(self.device)
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            body()
+        return graph
+
+    # ---- operations
+    def embed(self, table, ids, scale=1.0):
+        v, h = table.shape
+        m = ids.shape[0]
+        out = torch.empty((m, h), dtype=torch.float32, device=self.device)
+        self._check(self.lib.llm_embed(self._dev(table, "embedding table"), _code(table.dtype),
+                                       self._dev(ids, "token ids", torch.int32), out.data_ptr(),
+                                       m, h, v, float(scale), self._stream()), "embed")
+        return out
+
+    def add_rmsnorm(self, res, delta, weight, eps, out_dtype, rows=None):
+        m, h = res.shape
+        self._dev(res, "residual stream", torch.float32)
+        self._dev(weight, "norm weight", torch.float32, (h,))
+        dptr, dcode = None, _code(out_dtype)
+        if delta is not None:
+            dptr, dcode = self._dev(delta, "delta", shape=(m, h)), _code(delta.dtype)
+        n_out = m
+        rptr = None
+        if rows is not None:
+            rptr = self._dev(rows, "row indices", torch.int32)
+            n_out = rows.shape[0]
+        out = torch.empty((n_out, h), dtype=out_dtype, device=self.device)
+        self._check(self.lib.llm_add_rmsnorm(res.data_ptr(), dptr, dcode, weight.data_ptr(),
+                                             float(eps), out.data_ptr(), _code(out_dtype), rptr,
+                                             n_out, h, self._stream()), "add_rmsnorm")
+        return out
+
+    def linear(self, x, w, bias, out_dtype):
+        m, k = x.shape
+        n, k2 = w.shape
+        if k != k2:
+            raise KernelError("linear: x is [%d, %d] but the weight is [%d, %d]" % (m, k, n, k2))
+        self._dev(x, "linear input")
+        self._dev(w, "linear weight")
+        if w.dtype == torch.float32:
+            xf = x if x.dtype == torch.float32 else x.float()
+            out = torch.empty((m, n), dtype=torch.float32, device=self.device)
+            self._check(self.lib.llm_gemm_f32(xf.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k,
+                                              self._stream()), "gemm_f32")
+        elif w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
+            out = self._linear_bf16(x, w, out_dtype)
+        else:
+            raise KernelError("linear: input %s with weight %s is not supported" % (x.dtype, w.dtype))
+        if bias is not None:
+            self._dev(bias, "bias", torch.float32, (n,))
+            self._check(self.lib.llm_add_bias(out.data_ptr(), _code(out.dtype), bias.data_ptr(), m, n,
+                                              self._stream()), "add_bias")
+        return out if out.dtype == out_dtype else out.to(out_dtype)
+
+    def _linear_bf16(self, x, w, out_dtype):
+        out = torch.matmul(x, w.t())
+        return out
+
+    def silu_mul(self, gu):
+        m, two_i = gu.shape
+        if two_i % 2:
+            raise KernelError("silu_mul: the input width %d is odd" % two_i)
+        out = torch.empty((m, two_i // 2), dtype=gu.dtype, device=self.device)
+        self._check(self.lib.llm_silu_mul(self._dev(gu, "gate_up"), out.data_ptr(), _code(gu.dtype),
+                                          m, two_i // 2, self._stream()), "silu_mul")
+        return out
+
+    def rope_kv_write(self, qkv, bias, n_heads, n_kv, hd, cos, sin, rot_dim, ctx, kv, write):
+        m, width = qkv.shape
+        need = (n_heads + (2 * n_kv if write else 0)) * hd
+        if width != need:
+            raise KernelError("rope_kv_write: rows are %d wide, expected %d" % (width, need))
+        self._dev(qkv, "qkv")
+        if m != ctx.n_tokens:
+            raise KernelError("rope_kv_write: %d rows for a step of %d tokens" % (m, ctx.n_tokens))
+        cptr = sptr = None
+        if rot_dim:
+            if cos is None or cos.shape[1] != rot_dim // 2 or cos.shape != sin.shape:
+                raise KernelError("rope_kv_write: rotary tables do not match rot_dim %d" % rot_dim)
+            if not ctx.captured and ctx.max_ctx > cos.shape[0]:
+                raise KernelError("rope_kv_write: position %d exceeds the rotary table of %d rows"
+                                  % (ctx.max_ctx - 1, cos.shape[0]))
+            cptr, sptr = self._dev(cos, "cos", torch.float32), self._dev(sin, "sin", torch.float32)
+        bptr = None
+        if bias is not None:
+            bptr = self._dev(bias, "qkv bias", torch.float32)
+            if bias.shape[0] < need:
+                raise KernelError("rope_kv_write: the bias is shorter than a row")
+        kptr = vptr = tptr = None
+        stride = 0
+        if write:
+            self._check_kv(kv, n_kv, hd, qkv.dtype)
+            kptr, vptr, tptr = kv.k_pages.data_ptr(), kv.v_pages.data_ptr(), kv.block_table.data_ptr()
+            stride = kv.block_table.shape[1]
+        self._check(self.lib.llm_rope_kv_write(
+            qkv.data_ptr(), _code(qkv.dtype), width, bptr, n_heads, n_kv, hd, cptr, sptr, rot_dim,
+            ctx.tok_pos.data_ptr(), ctx.tok_seq.data_ptr(), ctx.seq_slot.data_ptr(), tptr, stride,
+            kptr, vptr, 64, 1 if write else 0, m, self._stream()), "rope_kv_write")
+
+    def _check_kv(self, kv, n_kv, hd, dtype):
+        if kv is None:
+            raise KernelError("this layer has no cache entry")
+        shape = tuple(kv.k_pages.shape)
+        if len(shape) != 4 or shape[1:] != (n_kv, 64, hd) or tuple(kv.v_pages.shape) != shape:
+            raise KernelError("cache pages have shape %s, expected [pages, %d, 64, %d]" % (shape, n_kv, hd))
+        if kv.k_pages.dtype != dtype or kv.v_pages.dtype != dtype:
+            raise KernelError("cache dtype %s differs from the activations' %s" % (kv.k_pages.dtype, dtype))
+        self._dev(kv.k_pages, "key pages")
+        self._dev(kv.v_pages, "value pages")
+        self._dev(kv.block_table, "page table", torch.int32)
+
+    def attention(self, qkv, n_heads, n_kv, hd, ctx, kv, scale, window):
+        m, width = qkv.shape
+        if width < n_heads * hd:
+            raise KernelError("attention: rows are %d wide, queries need %d" % (width, n_heads * hd))
+        if n_heads % n_kv:
+            raise KernelError("attention: %d heads are not a multiple of %d kv heads" % (n_heads, n_kv))
+        if hd > 256:
+            raise KernelError("attention: head_dim %d above 256 is not supported" % hd)
+        self._check_kv(kv, n_kv, hd, qkv.dtype)
+        out = torch.empty((m, n_heads * hd), dtype=qkv.dtype, device=self.device)
+        self._check(self.lib.llm_attention_ref(
+            qkv.data_ptr(), _code(qkv.dtype), width, kv.k_pages.data_ptr(), kv.v_pages.data_ptr(),
+            kv.block_table.data_ptr(), kv.block_table.shape[1], 64, ctx.tok_pos.data_ptr(),
+            ctx.tok_seq.data_ptr(), ctx.seq_slot.data_ptr(), out.data_ptr(), m, n_heads, n_kv, hd,
+            float(scale), int(window), self._stream()), "attention")
+        return out
+
+    def argmax(self, logits):
+        r, v = logits.shape
+        self._dev(logits, "logits", torch.float32)
+        out = torch.empty((r,), dtype=torch.int32, device=self.device)
+        self._check(self.lib.llm_argmax(logits.data_ptr(), out.data_ptr(), r, v, self._stream()), "argmax")
+        return out
+
+    def sample(self, logits, temperature, top_k, top_p, seed, streams: List[int], counters: List[int]):
+        r, v = logits.shape
+        self._dev(logits, "logits", torch.float32)
+        if len(streams) != r or len(counters) != r:
+            raise KernelError("sample: one stream and counter per row are needed")
+        keys = torch.tensor([streams, counters], dtype=torch.int64).to(self.device)
+        out = torch.empty((r,), dtype=torch.int32, device=self.device)
+        self._check(self.lib.llm_sample(logits.data_ptr(), out.data_ptr(), r, v, float(temperature),
+                                        int(top_k), float(top_p), int(seed) & (2**64 - 1),
+                                        keys[0].data_ptr(), keys[1].data_ptr(), self._stream()), "sample")
+        return out

@@ -1,0 +1,103 @@
+"""Grouped-query causal attention over the paged cache.
+
+The reference's order (src/libllm/llama.cc:178-225): one stacked q|k|v product, split, rotate q
+and k at absolute positions, append k and v to the past, softmax(q k^T / sqrt(hd)) v with query
+head h reading kv head h // (n_heads / n_kv_heads) (src/flint/operators.cc:43-56,100-127), merge
+heads, output product.  Here the rotation and the cache write are one kernel, and attention reads
+keys and values from the cache for whole prompts and single tokens alike.
+"""
+from dataclasses import dataclass, field
+from typing import Optional
+
+import torch
+
+from ..errors import ConfigError
+from .base import PartSpec, CacheNeed, Mixer, StepContext, WeightDecl
+from .linear import Linear
+from .registry import build_position, register_mixer
+
+
+@dataclass
+class AttentionSpec(PartSpec):
+    width: int = 0
+    n_heads: int = 0
+    n_kv_heads: int = 0
+    head_dim: int = 0
+    position: PartSpec = None
+    qkv_bias: bool = False
+    window: int = 0                   # 0: every earlier key; n: only the last n keys
+    scale: Optional[float] = None     # None: head_dim ** -0.5
+    q_name: str = "q_proj"
+    k_name: str = "k_proj"
+    v_name: str = "v_proj"
+    o_name: str = "o_proj"
+
+
+@register_mixer("attention")
+class Attention(Mixer):
+    graph_safe = True      # reads nothing from the host during a step
+
+    def __init__(self, spec: AttentionSpec):
+        if min(spec.width, spec.n_heads, spec.n_kv_heads, spec.head_dim) <= 0:
+            raise ConfigError("attention sizes must be positive")
+        if spec.n_heads % spec.n_kv_heads:
+            raise ConfigError("num_attention_heads (%d) is not a multiple of num_key_value_heads (%d)"
+                              % (spec.n_heads, spec.n_kv_heads))
+        if spec.window < 0:
+            raise ConfigError("attention window must not be negative")
+        self.spec = spec
+        self.q_dim = spec.n_heads * spec.head_dim
+        self.kv_dim = spec.n_kv_heads * spec.head_dim
+        self.scale = float(spec.scale) if spec.scale is not None else float(spec.head_dim) ** -0.5
+        self.position = build_position(spec.position)
+        if self.position.rot_dim > spec.head_dim:
+            raise ConfigError("rotary dimension %d exceeds head_dim %d"
+                              % (self.position.rot_dim, spec.head_dim))
+        self.qkv = Linear(spec.width, self.q_dim + 2 * self.kv_dim)
+        self.q_only = Linear(spec.width, self.q_dim)
+        self.out = Linear(self.q_dim, spec.width)
+        self.cos = self.sin = None
+        self.bias = None
+
+    def cache_need(self):
+        s = self.spec
+        return CacheNeed("window" if s.window else "full", s.n_kv_heads, s.head_dim, s.window)
+
+    def weights(self):
+        s = self.spec
+        decl = {
+            s.q_name + ".weight": WeightDecl((self.q_dim, s.width)),
+            s.k_name + ".weight": WeightDecl((self.kv_dim, s.width)),
+            s.v_name + ".weight": WeightDecl((self.kv_dim, s.width)),
+            s.o_name + ".weight": WeightDecl((s.width, self.q_dim)),
+        }
+        if s.qkv_bias:
+            decl[s.q_name + ".bias"] = WeightDecl((self.q_dim,), role="vector", init="normal")
+            decl[s.k_name + ".bias"] = WeightDecl((self.kv_dim,), role="vector", init="normal")
+            decl[s.v_name + ".bias"] = WeightDecl((self.kv_dim,), role="vector", init="normal")
+        return decl
+
+    def bind(self, tensors, ops, dtype):
+        s = self.spec
+        parts = [tensors[n + ".weight"] for n in (s.q_name, s.k_name, s.v_name)]
+        if len({p.dtype for p in parts}) > 1:
+            parts = [p.float() for p in parts]
+        bias = None
+        if s.qkv_bias:
+            bias = torch.cat([tensors[n + ".bias"] for n in (s.q_name, s.k_name, s.v_name)]).contiguous()
+        w = torch.cat(parts, dim=0)                      # q rows, then k, then v
+        self.qkv.bind(w)
+        self.q_only.bind(w[:self.q_dim])
+        self.bias = bias                                 # added inside the rotation kernel
+        self.out.bind(tensors[s.o_name + ".weight"])
+        self.cos, self.sin = self.position.tables(w.device)
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, entry) -> torch.Tensor:
+        s = self.spec
+        kv = ctx.kv(entry.cache)
+        qkv = self.qkv(ctx, x) if entry.writes else self.q_only(ctx, x)
+        ctx.ops.rope_kv_write(qkv, self.bias, s.n_heads, s.n_kv_heads, s.head_dim, self.cos, self.sin,
+                              self.position.rot_dim, ctx, kv, entry.writes)
+        o = ctx.ops.attention(qkv, s.n_heads, s.n_kv_heads, s.head_dim, ctx, kv,
+                              self.scale, s.window)
+        return self.out(ctx, o)

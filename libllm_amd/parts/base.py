@@ -1,0 +1,172 @@
+"""Interfaces that every part of a layer implements, and what a step hands to them.
+
+A part is built from its record (sizes and constants), declares the tensors it needs by names
+relative to a prefix, is bound to the loaded tensors, and then runs on packed rows: all tokens of
+all sequences of a step lie one after another in a ``[tokens, width]`` matrix.  A part never
+learns which model or architecture it belongs to.
+"""
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Tuple
+
+import torch
+
+
+@dataclass
+class PartSpec:
+    """Base of all part records.  ``kind`` is the key under which the part is registered; each
+    kind of part defines its own record type, with its sizes and constants, beside its class."""
+    kind: str
+
+
+@dataclass
+class WeightDecl:
+    """A tensor a part expects in the weight file.
+
+    role "matrix": kept in the model's dtype (bfloat16, or float32 when the file stores 32-bit
+    or the whole model runs in 32-bit).  role "vector": small per-channel values (norm scales,
+    biases) held in float32 on the device.  role "table": integer table held as int32.
+    ``init`` says how the random-weights mode fills it: "normal", "ones" or "zeros".
+    """
+    shape: Tuple[int, ...]
+    role: str = "matrix"
+    init: str = "normal"
+
+
+@dataclass
+class CacheNeed:
+    """Keys and values a mixer keeps per token.  ``kind`` "full" keeps every position;
+    "window" needs only the last ``window`` positions.  Layers with equal needs share a group
+    of the cache, and each group has storage of its own."""
+    kind: str
+    n_kv_heads: int
+    head_dim: int
+    window: int = 0
+
+    def key(self):
+        return (self.kind, self.n_kv_heads, self.head_dim, self.window)
+
+
+@dataclass
+class StateNeed:
+    """Fixed-size state a mixer keeps per sequence (for instance a recurrent state)."""
+    shape: Tuple[int, ...]
+    dtype: torch.dtype = torch.float32
+
+
+class KVView:
+    """The keys and values of one cache entry: page pools ``[pages, kv_heads, page, head_dim]``
+    and the table that maps (slot, position // page) to a page."""
+
+    def __init__(self, k_pages, v_pages, block_table, page_size, need):
+        self.k_pages = k_pages
+        self.v_pages = v_pages
+        self.block_table = block_table
+        self.page_size = page_size
+        self.need = need
+
+
+class Stream:
+    """The residual stream of a step: the 32-bit running sum and the output of the last part,
+    which the next norm adds before it normalises (so the sum is formed once, in 32-bit)."""
+
+    def __init__(self, res: torch.Tensor):
+        self.res = res            # [tokens, width] float32
+        self.delta = None         # [tokens, width] in the activation dtype, or None
+
+
+class StepContext:
+    """Everything a part may look at during one step.
+
+    Device tensors (int32): ``tokens`` [M], ``tok_pos`` [M] absolute position of each token,
+    ``tok_seq`` [M] index of its sequence in this step, ``seq_start`` [B+1] offsets of the
+    sequences in the packed rows, ``seq_slot`` [B], ``seq_pos0`` [B] tokens already cached
+    before the step.  Host values: ``seq_lens`` and ``seq_pos0_host`` (lists), ``max_new``
+    (largest number of new tokens of a sequence) and ``max_ctx`` (largest cached length after
+    the step); under a captured graph the last two are upper bounds.
+    """
+
+    def __init__(self, ops, dtype, n_tokens, n_seqs):
+        self.ops = ops
+        self.dtype = dtype
+        self.n_tokens = n_tokens
+        self.n_seqs = n_seqs
+        self.tokens = None
+        self.tok_pos = None
+        self.tok_seq = None
+        self.seq_start = None
+        self.seq_slot = None
+        self.seq_pos0 = None
+        self.seq_lens: List[int] = []
+        self.seq_pos0_host: List[int] = []
+        self.seq_slot_host: List[int] = []
+        self.max_new = 0
+        self.max_ctx = 0
+        self.decode = False        # every sequence brings exactly one token
+        self.captured = False      # running under graph capture: host lists are not valid
+        self._kv: Dict[int, KVView] = {}
+        self._state: Dict[int, torch.Tensor] = {}
+
+    def kv(self, cache_entry: int) -> Optional[KVView]:
+        return self._kv.get(cache_entry)
+
+    def state(self, cache_entry: int) -> Optional[torch.Tensor]:
+        """Per-sequence state of a cache entry: ``[slots, *shape]``; row ``seq_slot[b]`` belongs
+        to sequence b and is zero when the sequence starts."""
+        return self._state.get(cache_entry)
+
+
+class Part:
+    """Common protocol: declare tensors, receive them."""
+
+    def weights(self) -> Dict[str, WeightDecl]:
+        return {}
+
+    def bind(self, tensors: Dict[str, torch.Tensor], ops, dtype) -> None:
+        pass
+
+
+class Mixer(Part):
+    """Mixes information between the tokens of a sequence (attention, a recurrence, ...).
+
+    ``forward(ctx, x, entry)`` takes the normalised rows ``[M, width]`` in the activation dtype
+    and returns rows of the same shape.  ``entry`` is the schedule entry of this run; the mixer
+    reads its keys/values through ``ctx.kv(entry.cache)`` and its state through
+    ``ctx.state(entry.cache)``, and writes them only if ``entry.writes``.
+    """
+
+    def cache_need(self) -> Optional[CacheNeed]:
+        return None
+
+    def state_need(self) -> Optional[StateNeed]:
+        return None
+
+    def forward(self, ctx: StepContext, x: torch.Tensor, entry) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    """Row-wise transformation: ``forward(ctx, x [M, width]) -> [M, width]``."""
+
+    def forward(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Norm(Part):
+    """``add_norm(ctx, stream, rows)``: adds ``stream.delta`` (if any) into ``stream.res`` in
+    32-bit, then returns the normalised rows in the activation dtype.  With ``rows`` (int32
+    indices) only those rows are normalised and returned, in that order."""
+
+    def add_norm(self, ctx: StepContext, stream: Stream, rows=None) -> torch.Tensor:
+        raise NotImplementedError
+
+
+class Block:
+    """Arrangement of a mixer, a feed-forward and norms around the residual stream."""
+
+    def __init__(self, mixer: Mixer, feed_forward: FeedForward, norms: List[Norm]):
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.norms = norms
+
+    def forward(self, ctx: StepContext, stream: Stream, entry) -> None:
+        raise NotImplementedError

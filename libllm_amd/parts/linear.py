@@ -1,0 +1,20 @@
+"""y = x W^T (+ b) with W stored [out, in] (src/libllm/layers.cc:56-92)."""
+from typing import Optional
+
+import torch
+
+
+class Linear:
+    def __init__(self, in_features: int, out_features: int):
+        self.in_features = in_features
+        self.out_features = out_features
+        self.weight: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+
+    def bind(self, weight: torch.Tensor, bias: Optional[torch.Tensor] = None):
+        assert tuple(weight.shape) == (self.out_features, self.in_features)
+        self.weight = weight.contiguous()
+        self.bias = bias
+
+    def __call__(self, ctx, x: torch.Tensor, out_dtype=None) -> torch.Tensor:
+        return ctx.ops.linear(x, self.weight, self.bias, out_dtype or ctx.dtype)

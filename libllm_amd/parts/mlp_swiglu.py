@@ -1,0 +1,57 @@
+"""SwiGLU feed-forward: down(silu(gate(x)) * up(x)); gate and up are one matrix product over the
+stacked weight, gate rows first (src/libllm/llama.cc:81-98, tools/llama_exporter.py:73-78,
+src/flint/cuda/swiglu.cu:44-49)."""
+from dataclasses import dataclass
+
+import torch
+
+from ..errors import ConfigError
+from .base import PartSpec, FeedForward, StepContext, WeightDecl
+from .linear import Linear
+from .registry import register_feed_forward
+
+
+@dataclass
+class SwiGLUSpec(PartSpec):
+    width: int = 0
+    intermediate: int = 0
+    activation: str = "silu"
+    gate_name: str = "gate_proj"
+    up_name: str = "up_proj"
+    down_name: str = "down_proj"
+
+
+@register_feed_forward("swiglu")
+class SwiGLU(FeedForward):
+    graph_safe = True      # reads nothing from the host during a step
+
+    def __init__(self, spec: SwiGLUSpec):
+        if spec.activation != "silu":
+            raise ConfigError("feed-forward activation %r is not supported (silu only)"
+                              % (spec.activation,))
+        if spec.width <= 0 or spec.intermediate <= 0:
+            raise ConfigError("feed-forward sizes must be positive")
+        self.spec = spec
+        self.gate_up = Linear(spec.width, 2 * spec.intermediate)
+        self.down = Linear(spec.intermediate, spec.width)
+
+    def weights(self):
+        s = self.spec
+        return {
+            s.gate_name + ".weight": WeightDecl((s.intermediate, s.width)),
+            s.up_name + ".weight": WeightDecl((s.intermediate, s.width)),
+            s.down_name + ".weight": WeightDecl((s.width, s.intermediate)),
+        }
+
+    def bind(self, tensors, ops, dtype):
+        s = self.spec
+        gate, up = tensors[s.gate_name + ".weight"], tensors[s.up_name + ".weight"]
+        if gate.dtype != up.dtype:
+            gate, up = gate.float(), up.float()
+        self.gate_up.bind(torch.cat([gate, up], dim=0))
+        self.down.bind(tensors[s.down_name + ".weight"])
+
+    def forward(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
+        gu = self.gate_up(ctx, x)
+        h = ctx.ops.silu_mul(gu)
+        return self.down(ctx, h)
