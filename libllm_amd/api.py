@@ -88,9 +88,8 @@ class Completion:
         decoder = codecs.getincrementaldecoder("utf-8")(errors="replace")
         gen = self._model._generator
         for _, token in gen.stream([self._ids], self._params, self._max):
-            text = decoder.decode(self._model._tokenizer().piece(token))
-            if text:
-                yield Chunk(text, token)
+            # one chunk per token; its text is empty while a multi-byte character is incomplete
+            yield Chunk(decoder.decode(self._model._tokenizer().piece(token)), token)
         tail = decoder.decode(b"", final=True)
         if tail:
             yield Chunk(tail, None)

@@ -5,7 +5,8 @@
   ends; a slot that is taken again starts at length 0 with zeroed state.
 * A *group* collects the cache entries whose mixers keep the same kind of keys and values (all
   positions, or a window of them, with given head count and size).  Each group has page pools of
-  its own: ``k`` and ``v`` of shape ``[entries, pages + 1, kv_heads, page, head_dim]`` and a table
+  its own: ``k`` of shape ``[entries, pages + 1, kv_heads, page, head_dim]``, ``v`` of shape
+  ``[entries, pages + 1, kv_heads, head_dim, page]`` and a table
   ``[slots + 1, pages_per_sequence]`` from (slot, position // page) to a page.  The last page and
   the last slot are a sink for padding rows and belong to nobody.
 * Per-sequence *state* of fixed size: for each cache entry whose mixer asks for it, a tensor
@@ -40,9 +41,12 @@ class CacheGroup:
         self.n_pages = n_pages
         self.sink_page = n_pages
         self.pages_per_seq = pages_per_seq
-        shape = (len(entries), n_pages + 1, need.n_kv_heads, PAGE, need.head_dim)
-        self.k = torch.zeros(shape, dtype=dtype, device=device)
-        self.v = torch.zeros(shape, dtype=dtype, device=device)
+        # keys lie [position, dim] in a page, values transposed [dim, position]: both are then
+        # read along their contiguous axis by the matrix-core attention kernels
+        self.k = torch.zeros((len(entries), n_pages + 1, need.n_kv_heads, PAGE, need.head_dim),
+                             dtype=dtype, device=device)
+        self.v = torch.zeros((len(entries), n_pages + 1, need.n_kv_heads, need.head_dim, PAGE),
+                             dtype=dtype, device=device)
         self.table_host = np.full((n_slots + 1, pages_per_seq), self.sink_page, dtype=np.int32)
         self.table = torch.from_numpy(self.table_host.copy()).to(device)
         self.held: Dict[int, Dict[int, int]] = {}      # slot -> {page index in sequence: page}

@@ -54,11 +54,11 @@ __global__ __launch_bounds__(64) void attention_ref_kernel(
     for (int j = 0; j < PAGE; ++j) {
       const float pj = __shfl(p, j, 64);
       if (pj == 0.f) continue;                             // uniform across the wave
-      const T* vr = v_pages + base + (size_t)j * hd;
+      const T* vr = v_pages + base + j;                    // values lie [dim, position]
 #pragma unroll
       for (int i = 0; i < ND; ++i) {
         const int d = lane + i * 64;
-        if (d < hd) acc[i] = fmaf(pj, Conv<T>::load(vr + d), acc[i]);
+        if (d < hd) acc[i] = fmaf(pj, Conv<T>::load(vr + (size_t)d * PAGE), acc[i]);
       }
     }
   }

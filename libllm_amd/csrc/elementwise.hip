@@ -133,7 +133,8 @@ extern "C" int llm_add_bias(void* x, int dtype, const float* b, int M, int N, hi
 //   q, k: o[j] = x[j] c - x[j+r/2] s,  o[j+r/2] = x[j+r/2] c + x[j] s  for j < r/2, r = rot_dim
 //         (rotate-half pairing, src/libllm/llama.cc:151-176); dims >= r pass through.
 //   q is rotated in place; k (rotated) and v go to the sequence's page of the cache:
-//   page = table[slot, pos / PAGE], element [page, kv_head, pos % PAGE, d].
+//   page = table[slot, pos / PAGE]; keys at [page, kv_head, pos % PAGE, d], values transposed at
+//   [page, kv_head, d, pos % PAGE].
 template <typename T, int PAGE>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride, const float* __restrict__ bias,
                                      int n_heads, int n_kv, int hd, const float* __restrict__ cos_t,
@@ -149,11 +150,12 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride, const 
   const int pass = hd - rot_dim;                 // dims that do not rotate
   const int per_head = half + pass;              // work items per rotating head
   const int n_rot_heads = n_heads + (write_kv ? n_kv : 0);
-  size_t page_base = 0;
+  size_t page_base = 0, v_base = 0;
   if (write_kv) {
     const int slot = seq_slot[tok_seq[m]];
     const int page = table[(size_t)slot * table_stride + pos / PAGE];
     page_base = ((size_t)page * n_kv) * PAGE * hd + (size_t)(pos % PAGE) * hd;
+    v_base = ((size_t)page * n_kv) * PAGE * hd + (size_t)(pos % PAGE);
   }
   const float* c = cos_t + (size_t)pos * half;
   const float* s = sin_t + (size_t)pos * half;
@@ -185,7 +187,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride, const 
       const int h = it / hd, d = it % hd;
       float v = Conv<T>::load(vrow + it);
       if (b) v += b[it];
-      Conv<T>::store(v_pages + page_base + (size_t)h * PAGE * hd + d, v);
+      Conv<T>::store(v_pages + v_base + ((size_t)h * hd + d) * PAGE, v);
     }
   }
 }

@@ -1,0 +1,35 @@
+// Matrix-core (MFMA) fragments for gfx950, bfloat16 inputs with float32 accumulation.
+//
+// v_mfma_f32_16x16x32_bf16 computes C[16x16] += A[16x32] * B[32x16] per wave.  Lane l holds
+//   A[i = l % 16][k = 8 * (l / 16) .. + 7]     (8 consecutive k of one row)
+//   B[k = 8 * (l / 16) .. + 7][j = l % 16]     (8 consecutive k of one column)
+//   C[i = 4 * (l / 16) + e][j = l % 16], e = 0..3
+// Which real index a k slot stands for is free as long as A and B agree.
+#pragma once
+#include "common.h"
+
+typedef __attribute__((__vector_size__(8 * sizeof(__bf16)))) __bf16 bf16x8;
+typedef __attribute__((__vector_size__(4 * sizeof(float)))) float f32x4;
+
+union Frag {
+  uint4 u;
+  bf16x8 v;
+  bf16_t h[8];
+};
+
+__device__ __forceinline__ Frag frag_zero() {
+  Frag f;
+  f.u = make_uint4(0u, 0u, 0u, 0u);
+  return f;
+}
+
+// 16 bytes from global memory (the address must be 16-byte aligned)
+__device__ __forceinline__ Frag frag_load(const bf16_t* p) {
+  Frag f;
+  f.u = *reinterpret_cast<const uint4*>(p);
+  return f;
+}
+
+__device__ __forceinline__ f32x4 mfma_bf16(const Frag& a, const Frag& b, f32x4 c) {
+  return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, c, 0, 0, 0);
+}

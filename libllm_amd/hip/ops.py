@@ -38,6 +38,12 @@ _SIGNATURES = {
     "llm_gemm_f32": [_vp, _vp, _vp, _i, _i, _i, _vp],
     "llm_attention_ref": [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
                           _f, _i, _vp],
+    "llm_gemm_skinny_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "llm_attention_mfma_supported": [_i],
+    "llm_attention_prefill_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i,
+                                   _i, _i, _f, _i, _vp],
+    "llm_attention_decode_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i,
+                                  _i, _i, _f, _i, _i, _vp],
     "llm_argmax": [_vp, _vp, _i, _i, _vp],
     "llm_sample": [_vp, _vp, _i, _i, _f, _i, _f, _u64, _vp, _vp, _vp],
 }
@@ -151,9 +157,24 @@ class HipOps:
                                               self._stream()), "add_bias")
         return out if out.dtype == out_dtype else out.to(out_dtype)
 
+    SKINNY_ROWS = 64        # most rows the streaming matrix product takes at once
+
     def _linear_bf16(self, x, w, out_dtype):
-        out = torch.matmul(x, w.t())
-        return out
+        m, k = x.shape
+        n = w.shape[0]
+        skinny_ok = self.fast_gemm and k % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
+        if skinny_ok and (m <= self.SKINNY_ROWS or out_dtype == torch.float32):
+            # float32 results for many rows (logits of whole prompts) go through the same kernel
+            # 64 rows at a time: a row's logits are then the same bits whatever the batch holds
+            odt = torch.float32 if out_dtype == torch.float32 else torch.bfloat16
+            out = torch.empty((m, n), dtype=odt, device=self.device)
+            for m0 in range(0, m, self.SKINNY_ROWS):
+                mm = min(self.SKINNY_ROWS, m - m0)
+                self._check(self.lib.llm_gemm_skinny_bf16(
+                    x.data_ptr() + m0 * k * 2, w.data_ptr(), out.data_ptr() + m0 * n * out.element_size(),
+                    _code(odt), mm, n, k, 0, self._stream()), "gemm_skinny_bf16")
+            return out
+        return torch.matmul(x, w.t())
 
     def silu_mul(self, gu):
         m, two_i = gu.shape
@@ -200,8 +221,11 @@ class HipOps:
         if kv is None:
             raise KernelError("this layer has no cache entry")
         shape = tuple(kv.k_pages.shape)
-        if len(shape) != 4 or shape[1:] != (n_kv, 64, hd) or tuple(kv.v_pages.shape) != shape:
-            raise KernelError("cache pages have shape %s, expected [pages, %d, 64, %d]" % (shape, n_kv, hd))
+        vshape = tuple(kv.v_pages.shape)
+        if (len(shape) != 4 or shape[1:] != (n_kv, 64, hd) or len(vshape) != 4
+                or vshape != (shape[0], n_kv, hd, 64)):
+            raise KernelError("cache pages have shapes %s / %s, expected [pages, %d, 64, %d] and "
+                              "[pages, %d, %d, 64]" % (shape, vshape, n_kv, hd, n_kv, hd))
         if kv.k_pages.dtype != dtype or kv.v_pages.dtype != dtype:
             raise KernelError("cache dtype %s differs from the activations' %s" % (kv.k_pages.dtype, dtype))
         self._dev(kv.k_pages, "key pages")
@@ -218,6 +242,32 @@ class HipOps:
             raise KernelError("attention: head_dim %d above 256 is not supported" % hd)
         self._check_kv(kv, n_kv, hd, qkv.dtype)
         out = torch.empty((m, n_heads * hd), dtype=qkv.dtype, device=self.device)
+        table = kv.block_table
+        if (self.fast_attention and qkv.dtype == torch.bfloat16 and width % 8 == 0
+                and self.lib.llm_attention_mfma_supported(hd)):
+            if ctx.decode:
+                if m != ctx.n_seqs:
+                    raise KernelError("attention: a decode step has one row per sequence")
+                pages = (ctx.max_ctx + 63) // 64
+                if window:
+                    pages = min(pages, window // 64 + 2)
+                n_split = max(1, min(pages, 64, -(-1024 // (m * n_kv))))
+                part_o = torch.empty((m, n_heads, n_split, hd), dtype=torch.float32, device=self.device)
+                part_ml = torch.empty((m, n_heads, n_split, 2), dtype=torch.float32, device=self.device)
+                self._check(self.lib.llm_attention_decode_bf16(
+                    qkv.data_ptr(), width, kv.k_pages.data_ptr(), kv.v_pages.data_ptr(),
+                    table.data_ptr(), table.shape[1], 64, ctx.seq_slot.data_ptr(),
+                    ctx.seq_pos0.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), m,
+                    n_heads, n_kv, hd, float(scale), int(window), n_split, self._stream()),
+                    "attention_decode_bf16")
+            else:
+                self._check(self.lib.llm_attention_prefill_bf16(
+                    qkv.data_ptr(), width, kv.k_pages.data_ptr(), kv.v_pages.data_ptr(),
+                    table.data_ptr(), table.shape[1], 64, ctx.seq_start.data_ptr(),
+                    ctx.seq_slot.data_ptr(), ctx.seq_pos0.data_ptr(), out.data_ptr(), ctx.n_seqs,
+                    ctx.max_new, n_heads, n_kv, hd, float(scale), int(window), self._stream()),
+                    "attention_prefill_bf16")
+            return out
         self._check(self.lib.llm_attention_ref(
             qkv.data_ptr(), _code(qkv.dtype), width, kv.k_pages.data_ptr(), kv.v_pages.data_ptr(),
             kv.block_table.data_ptr(), kv.block_table.shape[1], 64, ctx.tok_pos.data_ptr(),

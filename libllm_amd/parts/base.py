@@ -54,8 +54,9 @@ class StateNeed:
 
 
 class KVView:
-    """The keys and values of one cache entry: page pools ``[pages, kv_heads, page, head_dim]``
-    and the table that maps (slot, position // page) to a page."""
+    """The keys and values of one cache entry: key pages ``[pages, kv_heads, page, head_dim]``,
+    value pages ``[pages, kv_heads, head_dim, page]`` (transposed), and the table that maps
+    (slot, position // page) to a page."""
 
     def __init__(self, k_pages, v_pages, block_table, page_size, need):
         self.k_pages = k_pages

@@ -61,7 +61,7 @@ class CpuOps:
             pos = ctx.tok_pos.long()
             pages = kv.block_table.long()[slots, pos // kv.page_size]
             kv.k_pages[pages, :, pos % kv.page_size, :] = k.to(kv.k_pages.dtype)
-            kv.v_pages[pages, :, pos % kv.page_size, :] = v.to(kv.v_pages.dtype)
+            kv.v_pages[pages, :, :, pos % kv.page_size] = v.to(kv.v_pages.dtype)
 
     def attention(self, qkv, n_heads, n_kv, hd, ctx, kv, scale, window):
         m = qkv.shape[0]
@@ -75,7 +75,7 @@ class CpuOps:
             keys = torch.arange(first, pos + 1)
             pages = kv.block_table[slot].long()[keys // page]
             k = kv.k_pages[pages, :, keys % page, :].float()       # [L, n_kv, hd]
-            v = kv.v_pages[pages, :, keys % page, :].float()
+            v = kv.v_pages[pages, :, :, keys % page].float()
             q = qkv[t, :n_heads * hd].float().reshape(n_heads, hd)
             k = k.repeat_interleave(group, dim=1)
             v = v.repeat_interleave(group, dim=1)

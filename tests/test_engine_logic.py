@@ -1,0 +1,170 @@
+"""The engine's own logic (packing, cache, schedule, generation) on the CPU, with a torch stand-in
+for the kernels: the same traces as on the GPU, against the plain implementation."""
+import io
+
+import numpy as np
+import pytest
+import torch
+
+import toy
+import traces
+from cpu_ops import CpuOps
+from libllm_amd import CacheError, Model, RequestError
+from libllm_amd.config import ScheduleEntry, config_from_dict
+from libllm_amd.engine import DecoderModel, Engine, StepEntry
+from libllm_amd.engine.trace import replay
+from libllm_amd.runtime import load_engine
+from libllm_amd.weights import load_tensors, random_tensors
+from plain import files, llama, sampling
+from tiny import TINY_A, TINY_B, TINY_C, make_model
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    base = tmp_path_factory.mktemp("models")
+    out = {}
+    for name, cfg in (("A", TINY_A), ("B", TINY_B), ("C", TINY_C)):
+        path = make_model(base, cfg, seed=40 + len(out), name=name)
+        cfg_json, weights = files.read_model_dir(path)
+        out[name] = (path, llama.PlainConfig(cfg_json), weights)
+    return out
+
+
+def err(out, ref):
+    return float(np.abs(np.asarray(out, dtype=np.float64) - ref).max() / np.abs(ref).mean())
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_traces_agree_with_plain(models, tmp_path, name):
+    path, cfg, weights = models[name]
+    rng = np.random.default_rng(1)
+    requests = {"r%d" % i: rng.integers(0, cfg.vocab, size=n).tolist() for i, n in enumerate([70, 5, 1, 66, 33])}
+    ids = list(requests)
+    groups = [{r: requests[r] for r in ids[:3]}, {r: requests[r] for r in ids[3:]}]
+    for mode, steps in (("whole", traces.whole(requests)), ("tail", traces.tail_one_by_one(requests, 6)),
+                        ("batches", traces.batches(groups))):
+        engine = load_engine(path, dtype="float32", max_tokens=traces.max_tokens_needed(steps), ops=CpuOps())
+        out_dir = tmp_path / mode
+        replay(engine, traces.lines(steps), str(out_dir), log=io.StringIO())
+        engine.cache.check()
+        assert engine.cache.slots.n_free == engine.cache.slots.n_slots
+        got = traces.collect(steps, str(out_dir), cfg.vocab)
+        for rid, toks in requests.items():
+            ref = llama.logits_all(cfg, weights, toks)
+            assert err(np.stack([got[rid][p] for p in range(len(toks))]), ref) < 1e-4
+
+
+def test_step_refuses_bad_requests(models):
+    path, cfg, _ = models["A"]
+    engine = load_engine(path, dtype="float32", max_tokens=128, ops=CpuOps())
+    for bad in ([], [StepEntry("a", [], [])], [StepEntry("a", [1], [1])], [StepEntry("a", [cfg.vocab], [])],
+                [StepEntry("a", [-1], [])], [StepEntry("a", [1], []), StepEntry("a", [2], [])]):
+        with pytest.raises(RequestError):
+            engine.step(bad)
+    assert not engine.live_requests()
+    with pytest.raises(CacheError):
+        engine.step([StepEntry("a", [1] * 129, [])])           # beyond max_position_embeddings 128
+    with pytest.raises(CacheError):
+        engine.end(["nobody"])
+    assert engine.step([StepEntry("a", [1, 2], [])]) is None and engine.length("a") == 2
+    engine.end(["a"])
+    engine.cache.check()
+
+
+def test_generation_matches_plain(models):
+    path, cfg, weights = models["B"]
+    rng = np.random.default_rng(2)
+    prompts = [rng.integers(10, cfg.vocab, size=n).tolist() for n in (1, 17, 40, 70)]
+    model = Model(path, dtype="float32", max_tokens=512, ops=CpuOps(), max_batch=3)
+    assert model.name == "llama"
+    got = model.generate(prompts, max_new_tokens=5, temperature=0.0)
+    assert got == [sampling.generate(cfg, weights, p, 5) for p in prompts]
+    got = model.generate(prompts, max_new_tokens=5, temperature=0.8, top_k=50, top_p=0.8, seed=3)
+    want = [sampling.generate(cfg, weights, p, 5, 0.8, 50, 0.8, seed=3, stream=i) for i, p in enumerate(prompts)]
+    assert got == want
+    assert model.generate(prompts[:1], max_new_tokens=5, temperature=0.8, seed=3) == want[:1]   # whatever the batch
+    first = got[1][0]
+    assert model.generate(prompts, 5, temperature=0.8, seed=3, stop_tokens=[first])[1] == []
+    model.engine.cache.check()
+    chunks = list(model.complete(prompts[1], temperature=0.0, max_new_tokens=3))
+    assert [c.token_id for c in chunks if c.token_id is not None] == sampling.generate(cfg, weights, prompts[1], 3)
+
+
+def build(spec, seed, ops, max_tokens=512):
+    model = DecoderModel(spec)
+    tensors = random_tensors(model.declared(), seed, std=0.1, norm_std=0.2, dtype=torch.float32)
+    model.bind(tensors, ops, torch.float32)
+    return Engine(model, ops, torch.float32, max_tokens), {k: v.double().numpy() for k, v in tensors.items()}
+
+
+def test_schedule_may_repeat_a_layer_or_share_a_cache_entry():
+    cfg_t = config_from_dict(TINY_A)
+    cfg = llama.PlainConfig(TINY_A)
+    ids = np.random.default_rng(3).integers(0, cfg.vocab, size=20).tolist()
+    # layer 0 twice: the same weights run twice, each run with keys of its own
+    spec = cfg_t.to_spec()
+    spec.schedule = [ScheduleEntry(0, 0), ScheduleEntry(0, 1), ScheduleEntry(1, 2)]
+    engine, w = build(spec, 5, CpuOps())
+    x = llama.embedding(w["model.embed_tokens.weight"], ids)
+    for layer in (0, 0, 1):
+        x = llama.decode_layer(cfg, w, layer, x, np.arange(len(ids)))
+    ref = llama.lm_head(cfg, w, llama.rms_norm(x, w["model.norm.weight"], cfg.eps))
+    whole = engine.step([StepEntry("a", ids, list(range(20)))]).double().numpy()
+    assert err(whole, ref) < 1e-4
+    parts = [engine.step([StepEntry("b", ids[:13], list(range(13)))])] + \
+            [engine.step([StepEntry("b", [t], [0])]) for t in ids[13:]]
+    assert err(torch.cat(parts).double().numpy(), ref) < 1e-4
+    # layer 1 reads the keys and values that layer 0 wrote: it differs from its own-cache result
+    spec = cfg_t.to_spec()
+    spec.schedule = [ScheduleEntry(0, 0), ScheduleEntry(1, 0, writes=False)]
+    shared, _ = build(spec, 5, CpuOps())
+    assert shared.model.spec.n_cache_entries() == 1 and len(shared.cache.groups[0].entries) == 1
+    a = shared.step([StepEntry("a", ids, list(range(20)))])
+    b = torch.cat([shared.step([StepEntry("b", ids[:7], list(range(7)))])] +
+                  [shared.step([StepEntry("b", [t], [0])]) for t in ids[7:]])
+    assert err(b.double().numpy(), a.double().numpy()) < 1e-4       # consistent however it is cut
+    own, _ = build(cfg_t.to_spec(), 5, CpuOps())
+    assert err(own.step([StepEntry("a", ids, list(range(20)))]).double().numpy(), a.double().numpy()) > 1e-2
+
+
+def test_layers_may_differ_and_groups_get_storage_of_their_own():
+    spec = config_from_dict(TINY_A).to_spec()
+    spec.layers[1].mixer.n_kv_heads = 4                              # another grouping in layer 1
+    spec.layers[1].mixer.window = 70                                 # and a window
+    spec.layers[1].feed_forward.intermediate = 96
+    engine, _ = build(spec, 6, CpuOps(), max_tokens=256)
+    kinds = [(g.need.kind, g.need.n_kv_heads, g.need.window, g.entries) for g in engine.cache.groups]
+    assert kinds == [("full", 2, 0, [0]), ("window", 4, 70, [1])]
+    ids = np.random.default_rng(4).integers(0, 256, size=128).tolist()
+    whole = engine.step([StepEntry("a", ids, list(range(128)))])
+    engine.end(["a"])
+    cut = torch.cat([engine.step([StepEntry("b", ids[:90], list(range(90)))])] +
+                    [engine.step([StepEntry("b", [t], [0])]) for t in ids[90:]])
+    assert err(cut.double().numpy(), whole.double().numpy()) < 1e-4
+    win = engine.cache.groups[1]
+    assert sorted(win.held[engine.cache.slot_of("b")]) == [0, 1] or sorted(win.held[engine.cache.slot_of("b")]) == [1]
+    engine.end(["b"])
+    engine.cache.check()
+
+
+def test_toy_mixer_with_state_of_its_own():
+    cfg_t = config_from_dict(TINY_A)
+    cfg = llama.PlainConfig(TINY_A)
+    engine, w = build(toy.toy_spec(cfg_t), 7, CpuOps())
+    assert not engine.use_graphs and list(engine.cache.state) == [1] and engine.cache.state[1].shape[1:] == (64,)
+    assert engine.cache.groups[0].entries == [0]                     # the toy keeps no keys or values
+    rng = np.random.default_rng(5)
+    reqs = {"a": rng.integers(0, 256, size=30).tolist(), "b": rng.integers(0, 256, size=11).tolist()}
+    steps = traces.batches([reqs, {"c": reqs["b"]}], {"a": 12, "b": 4, "c": 10})
+    got = {}
+    for s in steps:
+        out = engine.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        row = 0
+        for e in s["entries"]:
+            for _ in e["want"]:
+                got.setdefault(e["id"], []).append(out[row].double().numpy())
+                row += 1
+        engine.end(s["end"])
+    for rid, toks in (("a", reqs["a"]), ("b", reqs["b"]), ("c", reqs["b"])):   # c reuses a slot: clean state
+        ref = toy.toy_oracle(cfg, w, w["model.layers.1.toy.mix.weight"], toks)
+        assert err(np.stack(got[rid]), ref) < 1e-4

@@ -1,0 +1,94 @@
+"""Generation through the entry points on the GPU: greedy and sampled tokens against the plain
+implementation, the Python entry point and the command line."""
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+from plain import files, llama, sampling
+from tiny import TINY_A, TINY_B, make_model
+
+pytestmark = pytest.mark.gpu
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope="module")
+def model_b(tmp_path_factory):
+    path = make_model(tmp_path_factory.mktemp("gen"), TINY_B, seed=31)
+    cfg_json, weights = files.read_model_dir(path)
+    return path, llama.PlainConfig(cfg_json), weights
+
+
+def clear_steps(cfg, weights, prompt, tokens, margin):
+    """How many leading tokens of a greedy continuation are decided by a clear margin."""
+    ids = list(prompt)
+    for n, tok in enumerate(tokens):
+        top = np.sort(llama.logits_all(cfg, weights, ids)[-1])
+        if top[-1] - top[-2] < margin:
+            return n
+        ids.append(tok)
+    return len(tokens)
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_greedy_generation_through_the_entry_point(model_b, dtype):
+    from libllm_amd import Device, Model
+    path, cfg, weights = model_b
+    rng = np.random.default_rng(2)
+    prompts = [rng.integers(10, cfg.vocab, size=n).tolist() for n in (1, 17, 40, 70, 64, 3)]
+    model = Model(path, Device.AUTO, dtype=dtype, max_tokens=1024, max_batch=4)   # two batches
+    got = model.generate(prompts, max_new_tokens=12, temperature=0.0)
+    want = [sampling.generate(cfg, weights, p, 12) for p in prompts]
+    if dtype == "float32":
+        assert got == want
+    else:
+        # bfloat16 may turn a near tie; up to the first unclear step the tokens are the plain ones
+        for p, g, w in zip(prompts, got, want):
+            n = clear_steps(cfg, weights, p, w, margin=0.25)
+            assert g[:n] == w[:n]
+        assert sum(g == w for g, w in zip(got, want)) >= 3
+    model.engine.cache.check()
+    assert model.engine.cache.slots.n_free == model.engine.cache.slots.n_slots
+
+
+def test_sampled_generation_and_stop_tokens(model_b):
+    from libllm_amd import Model
+    path, cfg, weights = model_b
+    rng = np.random.default_rng(3)
+    prompts = [rng.integers(10, cfg.vocab, size=n).tolist() for n in (1, 17, 40, 70)]   # BASELINE's tiny B workload
+    model = Model(path, dtype="float32", max_tokens=1024)
+    got = model.generate(prompts, max_new_tokens=12, temperature=0.8, top_k=50, top_p=0.8, seed=4)
+    want = [sampling.generate(cfg, weights, p, 12, 0.8, 50, 0.8, seed=4, stream=i) for i, p in enumerate(prompts)]
+    for i, (g, w) in enumerate(zip(got, want)):
+        if g != w:                                     # only a draw on a boundary of the running sum may differ
+            n = next(k for k in range(len(w)) if k >= len(g) or g[k] != w[k])
+            logits = llama.logits_all(cfg, weights, prompts[i] + w[:n])[-1]
+            assert sampling.margin(logits, 0.8, 50, 0.8, sampling.uniform(4, i, n)) < 1e-4
+    assert sum(g == w for g, w in zip(got, want)) >= 3
+    again = model.generate(prompts, max_new_tokens=12, temperature=0.8, top_k=50, top_p=0.8, seed=4)
+    assert again == got                                 # a seed fixes the tokens
+    stop = got[2][3]
+    cut = model.generate(prompts, max_new_tokens=12, temperature=0.8, top_k=50, top_p=0.8, seed=4, stop_tokens=[stop])
+    assert cut[2] == got[2][:got[2].index(stop)]        # the stop token is not emitted; others go on
+    chunks = list(model.complete(prompts[1], top_k=1, max_new_tokens=5))
+    assert [c.token_id for c in chunks if c.token_id is not None] == sampling.generate(cfg, weights, prompts[1], 5)
+
+
+def test_command_line(model_b):
+    path, cfg, weights = model_b
+    prompt = [11, 12, 13, 14]
+    want = sampling.generate(cfg, weights, prompt, 6)
+    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "llm"), "chat", "-m", path, "-device", "auto",
+                           "-dtype", "float32", "-ids", "-temperature", "0", "-max_new_tokens", "6"],
+                          input=" ".join(map(str, prompt)) + "\n:new\n\n", capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stderr
+    assert " ".join(map(str, want)) in proc.stdout
+    assert "tokens, time=" in proc.stdout and "ms per token" in proc.stdout
+
+
+def test_smoke_entry():
+    sys.path.insert(0, ROOT)
+    import __graft_entry__
+    __graft_entry__.smoke()

@@ -1,0 +1,378 @@
+"""Each HIP kernel alone against a plain torch reference in float64, at sizes other than the
+tiny models': odd widths, tails, head sizes in steps of 16, many kv groups, long key ranges."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import PAGE, attention_oracle, fill_kv, make_ctx, make_kv, read_kv
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from libllm_amd.hip import HipOps
+    return HipOps()
+
+
+def rnd(shape, dtype, seed, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return (torch.randn(shape, generator=g) * scale).to(dtype)
+
+
+BF16_2ULP = 2.0 ** -7     # two units in the last place of the largest value, for a result rounded once or twice
+
+
+def max_err(out, ref):
+    """max|out - ref| / max|ref|: a bfloat16 result rounded once is within 2^-9 of the largest value."""
+    out = torch.as_tensor(out).double().cpu()
+    ref = torch.as_tensor(ref).double().cpu()
+    return float((out - ref).abs().max() / ref.abs().max().clamp_min(1e-30))
+
+
+def close(out, ref, dtype, f32=1e-5, bf16=BF16_2ULP):
+    return max_err(out, ref) < (f32 if dtype == torch.float32 else bf16)
+
+
+# ------------------------------------------------------------------------------- embedding
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed(ops, dtype):
+    table = rnd((517, 96), dtype, 1).cuda()
+    ids = torch.tensor([0, 516, 3, 3, 77, 100], dtype=torch.int32).cuda()
+    out = ops.embed(table, ids, 1.0)
+    assert out.dtype == torch.float32
+    assert torch.equal(out.cpu(), table.float().cpu()[ids.cpu().long()])
+    out = ops.embed(table, ids, 2.5)
+    assert torch.equal(out.cpu(), table.float().cpu()[ids.cpu().long()] * 2.5)
+
+
+def test_embed_reference_vector(ops):
+    # src/flint/cpu/test.cc:101-144
+    wte = torch.tensor([[0.1, 0.2], [0.3, 0.4], [0.2, 0.3], [0.4, 0.5], [0.7, 0.8]]).cuda()
+    ids = torch.tensor([0, 1, 2, 1, 3, 4], dtype=torch.int32).cuda()
+    want = torch.tensor([[0.1, 0.2], [0.3, 0.4], [0.2, 0.3], [0.3, 0.4], [0.4, 0.5], [0.7, 0.8]])
+    assert torch.allclose(ops.embed(wte, ids, 1.0).cpu(), want)
+
+
+# ------------------------------------------------------------------------------- norm
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width", [10, 11, 192, 2050, 9000])     # 10/11: src/flint/cuda/test.cc:243-248
+def test_add_rmsnorm(ops, dtype, width):
+    m, eps = 7, 1e-5
+    res = rnd((m, width), torch.float32, 2, 3.0).cuda()
+    delta = rnd((m, width), dtype, 3).cuda()
+    w = (1.0 + rnd((width,), torch.float32, 4, 0.3)).cuda()
+    res0 = res.clone()
+    out = ops.add_rmsnorm(res, delta, w, eps, dtype)
+    x = res0.double() + delta.double()
+    assert torch.allclose(res.double(), x, rtol=1e-6, atol=1e-6)          # the sum is kept in 32-bit
+    ref = x * w.double() / torch.sqrt((x * x).mean(-1, keepdim=True) + eps)
+    assert close(out, ref, dtype)
+    # no delta, gathered rows
+    rows = torch.tensor([5, 0, 5], dtype=torch.int32).cuda()
+    before = res.clone()
+    out = ops.add_rmsnorm(res, None, w, eps, dtype, rows)
+    assert torch.equal(res, before)
+    assert close(out, ref[rows.long()], dtype)
+
+
+def test_rmsnorm_zero_and_eps(ops):
+    res = torch.zeros((2, 64), device="cuda")
+    w = torch.ones(64, device="cuda")
+    out = ops.add_rmsnorm(res, None, w, 1e-6, torch.float32)
+    assert torch.equal(out.cpu(), torch.zeros(2, 64))                      # eps inside the root: no NaN
+    res = torch.full((1, 64), 1e-3, device="cuda")
+    out = ops.add_rmsnorm(res, None, w, 1e-2, torch.float32)                # eps dominates
+    assert torch.allclose(out.cpu(), torch.full((1, 64), 1e-3 / math.sqrt(1e-6 + 1e-2)), rtol=1e-5)
+
+
+# ------------------------------------------------------------------------------- matrix products
+@pytest.mark.parametrize("mnk", [(1, 1, 1), (1, 513, 64), (7, 33, 129), (64, 64, 64), (65, 130, 257),
+                                 (2, 1000, 192), (300, 70, 16), (1, 1, 2050)])
+def test_gemm_f32(ops, mnk):
+    m, n, k = mnk
+    x = rnd((m, k), torch.float32, 5).cuda()
+    w = rnd((n, k), torch.float32, 6).cuda()
+    out = ops.linear(x, w, None, torch.float32)
+    ref = x.double() @ w.double().t()
+    assert max_err(out, ref) < 2e-6
+
+
+def test_linear_bias_and_mixed_dtypes(ops):
+    x = rnd((5, 40), torch.bfloat16, 7).cuda()
+    w32 = rnd((24, 40), torch.float32, 8).cuda()        # a matrix stored in 32-bit stays so
+    b = rnd((24,), torch.float32, 9).cuda()
+    out = ops.linear(x, w32, b, torch.bfloat16)
+    ref = x.double() @ w32.double().t() + b.double()
+    assert out.dtype == torch.bfloat16 and close(out, ref, torch.bfloat16)
+
+
+@pytest.mark.parametrize("m", [1, 3, 16, 17, 33, 64])
+@pytest.mark.parametrize("nk", [(16, 8), (24, 136), (1000, 2048), (2050, 264), (40, 4104)])
+@pytest.mark.parametrize("out_dtype", DTYPES)
+def test_gemm_skinny(ops, m, nk, out_dtype):
+    n, k = nk
+    x = rnd((m, k), torch.bfloat16, 10).cuda()
+    w = rnd((n, k), torch.bfloat16, 11).cuda()
+    out = ops.linear(x, w, None, out_dtype)
+    assert out.dtype == out_dtype and tuple(out.shape) == (m, n)
+    ref = x.double() @ w.double().t()
+    assert max_err(out, ref) < (2e-6 if out_dtype == torch.float32 else BF16_2ULP)
+
+
+def test_gemm_skinny_rows_per_block_and_batch_invariance(ops):
+    k, n = 520, 300
+    x = rnd((64, k), torch.bfloat16, 12).cuda()
+    w = rnd((n, k), torch.bfloat16, 13).cuda()
+    full = ops.linear(x, w, None, torch.float32)
+    for m in (1, 5, 16, 40):                             # a row's result does not depend on the batch
+        part = ops.linear(x[:m].contiguous(), w, None, torch.float32)
+        assert torch.equal(part, full[:m])
+    big = rnd((200, k), torch.bfloat16, 14).cuda()       # many rows with float32 output: chunks of 64
+    out = ops.linear(big, w, None, torch.float32)
+    assert max_err(out, big.double() @ w.double().t()) < 2e-6
+    for rows in (16, 32, 64):
+        c = torch.empty((64, n), dtype=torch.float32, device="cuda")
+        st = ops.lib.llm_gemm_skinny_bf16(x.data_ptr(), w.data_ptr(), c.data_ptr(), 0, 64, n, k, rows,
+                                          torch.cuda.current_stream().cuda_stream)
+        assert st == 0 and max_err(c, full) < 2e-6
+
+
+def test_gemm_skinny_refuses(ops):
+    x = rnd((2, 12), torch.bfloat16, 1).cuda()           # K not a multiple of 8: the library product runs
+    w = rnd((16, 12), torch.bfloat16, 2).cuda()
+    out = ops.linear(x, w, None, torch.bfloat16)
+    assert close(out, x.double() @ w.double().t(), torch.bfloat16)
+    c = torch.empty((2, 16), dtype=torch.bfloat16, device="cuda")
+    st = ops.lib.llm_gemm_skinny_bf16(x.data_ptr(), w.data_ptr(), c.data_ptr(), 1, 2, 16, 12, 0, 0)
+    assert st == 1                                        # refused, not wrong
+
+
+def test_large_bf16_product(ops):
+    x = rnd((300, 256), torch.bfloat16, 3).cuda()
+    w = rnd((520, 256), torch.bfloat16, 4).cuda()
+    out = ops.linear(x, w, None, torch.bfloat16)
+    assert close(out, x.double() @ w.double().t(), torch.bfloat16)
+
+
+# ------------------------------------------------------------------------------- SiLU-mul
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("width", [150, 152, 1024])              # src/flint/cuda/test.cc:208-211
+def test_silu_mul(ops, dtype, width):
+    gu = rnd((9, width), dtype, 15, 2.0).cuda()
+    out = ops.silu_mul(gu)
+    i = width // 2
+    g, u = gu[:, :i].double(), gu[:, i:].double()
+    ref = g / (1 + torch.exp(-g)) * u
+    assert close(out, ref, dtype, f32=2e-6)
+    swapped = u / (1 + torch.exp(-u)) * g                          # gating the wrong half must differ
+    assert not close(out, swapped, dtype, f32=1e-2, bf16=1e-2)
+
+
+def test_silu_mul_limits(ops):
+    gu = torch.tensor([[0.0, 30.0, -30.0, 5.0, 3.0, 2.0, 7.0, 11.0]], device="cuda")
+    out = ops.silu_mul(gu).cpu()
+    assert out[0, 0] == 0.0                                        # gate 0 -> 0
+    assert abs(out[0, 1] - 30.0 * 2.0) < 1e-4                      # large gate -> gate * up
+    assert abs(out[0, 2]) < 1e-10
+
+
+# ------------------------------------------------------------------------------- rotation + cache write
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(4, 2, 16, 16), (6, 1, 32, 32), (6, 3, 48, 24), (5, 5, 80, 80), (32, 8, 64, 0)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_rope_kv_write(ops, dtype, shape, bias):
+    n_heads, n_kv, hd, rot = shape
+    seqs = [(2, 0, 5), (0, 61, 9), (1, 130, 1)]                   # crosses page borders
+    ctx = make_ctx(ops, dtype, seqs)
+    kv = make_kv("cuda", dtype, 3, 4, n_kv, hd, seed=1)
+    m = ctx.n_tokens
+    width = (n_heads + 2 * n_kv) * hd
+    qkv = rnd((m, width), dtype, 16).cuda()
+    b = rnd((width,), torch.float32, 17).cuda() if bias else None
+    half = rot // 2
+    inv = 1.0 / (10000.0 ** (torch.arange(0, rot, 2, dtype=torch.float64) / max(rot, 1)))
+    ang = torch.arange(300, dtype=torch.float64)[:, None] * inv[None, :]
+    cos, sin = (torch.cos(ang).float().cuda(), torch.sin(ang).float().cuda()) if rot else (None, None)
+    x = qkv.double().cpu() + (b.double().cpu() if bias else 0)
+    ops.rope_kv_write(qkv, b, n_heads, n_kv, hd, cos, sin, rot, ctx, kv, True)
+    pos = ctx.tok_pos.cpu().long()
+    heads = x[:, :(n_heads + n_kv) * hd].reshape(m, n_heads + n_kv, hd).clone()
+    if rot:
+        c, s = torch.cos(ang)[pos][:, None, :], torch.sin(ang)[pos][:, None, :]
+        x1, x2 = heads[..., :half].clone(), heads[..., half:rot].clone()
+        heads[..., :half] = x1 * c - x2 * s
+        heads[..., half:rot] = x2 * c + x1 * s
+    tol = dict(f32=2e-6)
+    assert close(qkv[:, :n_heads * hd], heads[:, :n_heads].reshape(m, -1), dtype, **tol)
+    o = 0
+    for slot, p0, n in seqs:
+        k_got, v_got = read_kv(kv, slot, p0 + n)
+        assert close(k_got[p0:], heads[o:o + n, n_heads:], dtype, **tol)
+        v_ref = x[o:o + n, (n_heads + n_kv) * hd:].reshape(n, n_kv, hd)
+        assert close(v_got[p0:], v_ref, dtype, **tol)
+        assert torch.count_nonzero(k_got[:p0]) == 0               # nothing else is touched
+        o += n
+
+
+def test_rope_pairing_and_sign(ops):
+    # a unit vector in dimension 0 at position p becomes cos at 0 and +sin at hd/2:
+    # o[j] = x[j] c - x[j+hd/2] s, o[j+hd/2] = x[j+hd/2] c + x[j] s   (src/libllm/llama.cc:151-176)
+    hd = 16
+    ctx = make_ctx(ops, torch.float32, [(0, 3, 1)])
+    kv = make_kv("cuda", torch.float32, 1, 1, 1, hd)
+    qkv = torch.zeros((1, 3 * hd), device="cuda")
+    qkv[0, 0] = 1.0
+    theta = 0.7
+    cos = torch.full((8, hd // 2), math.cos(theta), device="cuda")
+    sin = torch.full((8, hd // 2), math.sin(theta), device="cuda")
+    ops.rope_kv_write(qkv, None, 1, 1, hd, cos, sin, hd, ctx, kv, True)
+    q = qkv[0, :hd].cpu()
+    assert abs(q[0] - math.cos(theta)) < 1e-6 and abs(q[hd // 2] - math.sin(theta)) < 1e-6
+    assert torch.count_nonzero(q) == 2
+
+
+# ------------------------------------------------------------------------------- attention
+def run_attention(ops, dtype, n_heads, n_kv, hd, seqs, window=0, seed=0, boost=None, fast=True):
+    """seqs: (slot, past, new).  Returns (out, oracle) over all new tokens."""
+    ctx = make_ctx(ops, dtype, seqs)
+    pages = max((p + n + PAGE - 1) // PAGE for _, p, n in seqs)
+    kv = make_kv("cuda", dtype, max(s for s, _, _ in seqs) + 1, pages, n_kv, hd, seed=seed)
+    scale = hd ** -0.5
+    q = rnd((ctx.n_tokens, n_heads * hd + 24), dtype, seed + 1)   # wider rows: a stride is honoured
+    ref, o = [], 0
+    for slot, past, new in seqs:
+        keys = rnd((past + new, n_kv, hd), dtype, seed + 10 + slot)
+        vals = rnd((past + new, n_kv, hd), dtype, seed + 20 + slot)
+        if boost is not None:                                       # one far key stands out
+            key_pos, gain = boost
+            keys[key_pos] = keys[key_pos] * gain
+        fill_kv(kv, slot, keys, vals)
+        for t in range(new):
+            qt = q[o + t, :n_heads * hd].double().reshape(n_heads, hd)
+            ref.append(attention_oracle(qt, keys.double(), vals.double(), past + t, scale, window).reshape(-1))
+        o += new
+    ops.fast_attention = fast
+    try:
+        out = ops.attention(q.cuda(), n_heads, n_kv, hd, ctx, kv, scale, window)
+    finally:
+        ops.fast_attention = True
+    return out.double().cpu(), torch.stack(ref)
+
+
+# (heads, kv heads, queries, keys, head size): the cases of src/flint/cuda/test.cc:349-362
+REFERENCE_CASES = [(8, 8, 8, 8, 128), (8, 8, 128, 128, 128), (8, 2, 6, 10, 128), (8, 2, 1, 10, 128),
+                   (8, 2, 1, 2048, 128), (8, 2, 4, 1024, 128), (8, 8, 16, 16, 16), (8, 2, 6, 10, 16)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("case", REFERENCE_CASES)
+def test_attention_reference_cases(ops, dtype, case):
+    n_heads, n_kv, lq, lk, hd = case
+    out, ref = run_attention(ops, dtype, n_heads, n_kv, hd, [(0, lk - lq, lq)])
+    assert max_err(out, ref) < (1e-5 if dtype == torch.float32 else BF16_2ULP)
+
+
+@pytest.mark.parametrize("fast", [True, False])
+@pytest.mark.parametrize("hd", [16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 256, 144])
+def test_attention_head_sizes_bf16(ops, hd, fast):
+    # unequal batch: a fresh prompt, a continued one crossing pages, a single token with a long past
+    seqs = [(1, 0, 70), (0, 100, 37), (2, 300, 1)]
+    out, ref = run_attention(ops, torch.bfloat16, 6, 3, hd, seqs, seed=hd, fast=fast)
+    assert max_err(out, ref) < BF16_2ULP
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("groups", [(5, 5), (6, 1), (20, 1), (12, 4), (3, 3)])
+def test_attention_groups_decode_and_prefill(ops, dtype, groups):
+    n_heads, n_kv = groups
+    for seqs in ([(0, 129, 1), (1, 0, 1), (2, 64, 1), (3, 63, 1)],          # decode: one token each
+                 [(0, 129, 3), (1, 0, 65)]):
+        out, ref = run_attention(ops, dtype, n_heads, n_kv, 64, seqs, seed=3)
+        assert max_err(out, ref) < (1e-5 if dtype == torch.float32 else BF16_2ULP)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 5, 64, 65, 200])
+def test_attention_window(ops, dtype, window):
+    for seqs in ([(0, 0, 150)], [(0, 333, 1), (1, 64, 1)], [(0, 190, 20)]):
+        out, ref = run_attention(ops, dtype, 4, 2, 32, seqs, window=window, seed=window)
+        assert max_err(out, ref) < (1e-5 if dtype == torch.float32 else BF16_2ULP)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("far", [0, 3, 63, 64, 700])
+def test_attention_far_key_stands_out(ops, dtype, far):
+    """With random scores a lost key among hundreds changes little; here one key's score is made
+    to dominate, so that dropping or misplacing it cannot pass."""
+    for seqs in ([(0, 900, 1)], [(0, 0, 901)]):
+        out, ref = run_attention(ops, dtype, 4, 2, 64, seqs, seed=9, boost=(far, 12.0))
+        assert max_err(out, ref) < (1e-5 if dtype == torch.float32 else BF16_2ULP)
+
+
+def test_attention_single_token_is_value(ops):
+    # one query, no past: the output is the value itself
+    out, ref = run_attention(ops, torch.float32, 4, 4, 32, [(0, 0, 1)])
+    assert max_err(out, ref) < 1e-6
+
+
+# ------------------------------------------------------------------------------- sampling
+def test_argmax_reference_vectors(ops):
+    # src/flint/cuda/test.cc:376-392
+    p = torch.tensor([[0.4, 0.3, 0.2, 0.1], [0.1, 0.2, 0.6, 0.1], [0.05, 0.05, 0.1, 0.8]]).cuda()
+    assert ops.argmax(p).tolist() == [0, 2, 3]
+    # src/flint/cuda/test.cc:405-415: the maximum lies beyond the first block of the row
+    v = torch.zeros((2, 2050))
+    v[0, 2049], v[1, 1100] = 0.4, 0.7
+    assert ops.argmax(v.cuda()).tolist() == [2049, 1100]
+    t = torch.zeros((1, 5000))
+    t[0, 17] = t[0, 4000] = t[0, 999] = 3.0                                 # ties: lowest index
+    assert ops.argmax(t.cuda()).tolist() == [17]
+
+
+def test_sampling_matches_plain(ops):
+    from plain import sampling
+    g = torch.Generator().manual_seed(21)
+    for vocab, top_k, top_p, temp in [(1000, 50, 0.8, 0.8), (517, 0, 1.0, 1.3), (128256, 50, 0.9, 1.0),
+                                      (300, 300, 0.5, 0.7), (2050, 1024, 0.95, 2.0), (64, 7, 1.0, 0.5)]:
+        logits = (torch.randn((24, vocab), generator=g) * 3.0)
+        streams = list(range(100, 124))
+        counters = list(range(24))
+        k = 0 if top_k >= vocab else top_k
+        if k == 0 and top_p < 1.0:
+            k = vocab
+        got = ops.sample(logits.cuda(), temp, k, top_p, 77, streams, counters).tolist()
+        bad = 0
+        for r in range(24):
+            u = sampling.uniform(77, streams[r], counters[r])
+            want = sampling.sample(logits[r].double().numpy(), temp, k, top_p, u)
+            if got[r] != want:
+                # only a draw within rounding of a boundary of the running sum may differ
+                assert sampling.margin(logits[r].double().numpy(), temp, k, top_p, u) < 1e-5, (vocab, r)
+                bad += 1
+        assert bad <= 2
+
+
+def test_sampling_seed_and_top1(ops):
+    g = torch.Generator().manual_seed(5)
+    logits = torch.randn((6, 999), generator=g).cuda()
+    a = ops.sample(logits, 1.0, 40, 0.9, 1234, [0] * 6, list(range(6))).tolist()
+    b = ops.sample(logits, 1.0, 40, 0.9, 1234, [0] * 6, list(range(6))).tolist()
+    assert a == b                                                           # src/flint/cuda/test.cc:394-403
+    c = ops.sample(logits, 1.0, 40, 0.9, 1235, [0] * 6, list(range(6))).tolist()
+    assert a != c
+    top1 = ops.sample(logits, 1.0, 1, 1.0, 1, [0] * 6, list(range(6))).tolist()
+    assert top1 == ops.argmax(logits).tolist()                              # top_k 1 is arg-max
+
+
+def test_sampling_distribution(ops):
+    # many draws of one row follow its probabilities
+    logits = torch.tensor([[0.0, 1.0, 2.0, 3.0, -50.0]]).repeat(4000, 1).cuda()
+    got = ops.sample(logits, 1.0, 0, 1.0, 3, [0] * 4000, list(range(4000))).cpu().numpy()
+    freq = np.bincount(got, minlength=5) / 4000.0
+    p = torch.softmax(logits[0].double().cpu(), 0).numpy()
+    assert np.abs(freq - p).max() < 0.03

@@ -1,0 +1,222 @@
+"""The engine against the plain implementation, through the trace replay that drives the
+framework's own step function and cache: each request alone and whole; with its last 32 tokens one
+by one; in batches of unequal lengths whose shorter requests end earlier, one batch after another
+so that slots and pages are used again; long decoding; the first tokens of a sequence.  In 32-bit
+and in bfloat16, for tiny configurations that differ in every size and option."""
+import io
+import json
+import os
+import subprocess
+import sys
+
+import numpy as np
+import pytest
+
+import traces
+from helpers import assert_logits_close
+from plain import files, llama
+from tiny import TINY_A, TINY_B, TINY_C, make_model
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CONFIGS = {"A": TINY_A, "B": TINY_B, "C": TINY_C}
+DTYPES = ["float32", "bfloat16"]
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    base = tmp_path_factory.mktemp("models")
+    out = {}
+    for name, cfg in CONFIGS.items():
+        path = make_model(base, cfg, seed=17 + len(name), name=name)
+        cfg_json, weights = files.read_model_dir(path)
+        out[name] = (path, llama.PlainConfig(cfg_json), weights)
+    return out
+
+
+def make_requests(cfg, lengths, seed):
+    rng = np.random.default_rng(seed)
+    return {"r%d" % i: rng.integers(0, cfg.vocab, size=min(n, cfg.max_pos)).tolist()
+            for i, n in enumerate(lengths)}
+
+
+_oracle_cache = {}
+
+
+def oracle(name, cfg, weights, toks):
+    key = (name, tuple(toks))
+    if key not in _oracle_cache:
+        _oracle_cache[key] = llama.logits_all(cfg, weights, toks)
+    return _oracle_cache[key]
+
+
+def run_replay(path, dtype, steps, out_dir, max_tokens=None, use_graphs=True):
+    from libllm_amd.engine.trace import replay
+    from libllm_amd.runtime import load_engine
+    need = traces.max_tokens_needed(steps)
+    engine = load_engine(path, dtype=dtype, max_tokens=max_tokens or need, use_graphs=use_graphs)
+    log = io.StringIO()
+    replay(engine, traces.lines(steps), str(out_dir), log=log)
+    assert log.getvalue().split() == [w for s in steps for w in ("done", str(s["step"]))]
+    engine.cache.check()
+    assert engine.cache.slots.n_free == engine.cache.slots.n_slots          # everything given back
+    assert all(g.pool.n_free == g.pool.n_pages for g in engine.cache.groups)
+    return engine
+
+
+WORST = {}
+
+
+def check(name, cfg, weights, requests, got, dtype):
+    worst = WORST.get(dtype, 0.0)
+    for rid, toks in requests.items():
+        ref = oracle(name, cfg, weights, toks)
+        assert sorted(got[rid]) == list(range(len(toks))), "positions of %s" % rid
+        out = np.stack([got[rid][p] for p in range(len(toks))])
+        err, row = assert_logits_close(out, ref, dtype, "%s %s %s" % (name, dtype, rid))
+        worst = max(worst, row)
+        # arg-max agrees wherever the oracle's margin exceeds the error (src/libllm/llama_test.cc:182-187)
+        top2 = np.sort(ref, axis=-1)[:, -2:]
+        clear = (top2[:, 1] - top2[:, 0]) > 2 * np.abs(out - ref).max(axis=-1)
+        assert (out.argmax(-1)[clear] == ref.argmax(-1)[clear]).all()
+    WORST[dtype] = worst
+    print("worst row error so far (%s): %.3g" % (dtype, worst))
+    return worst
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_whole_tail_and_batches_agree_with_plain(models, tmp_path, name, dtype):
+    path, cfg, weights = models[name]
+    lengths = [70, 33, 100, 5, 64, 129, 1, 65]
+    requests = make_requests(cfg, lengths, seed=3)
+    ids = list(requests)
+    groups = [{r: requests[r] for r in ids[0:3]}, {r: requests[r] for r in ids[3:6]},
+              {r: requests[r] for r in ids[6:8]}]
+    decode = {"r0": 20, "r1": 32, "r2": 3, "r3": 4, "r4": 1, "r5": 40, "r6": 0, "r7": 64}
+    results = {}
+    for mode, steps in (("whole", traces.whole(requests)), ("tail", traces.tail_one_by_one(requests)),
+                        ("batches", traces.batches(groups, decode))):
+        out_dir = tmp_path / mode
+        run_replay(path, dtype, steps, out_dir)            # the cache is exactly as large as needed
+        got = traces.collect(steps, str(out_dir), cfg.vocab)
+        check(name, cfg, weights, requests, got, dtype)
+        results[mode] = got
+    # the three ways of cutting agree with each other, beyond rounding
+    for rid, toks in requests.items():
+        a = np.stack([results["whole"][rid][p] for p in range(len(toks))])
+        for mode in ("tail", "batches"):
+            b = np.stack([results[mode][rid][p] for p in range(len(toks))])
+            assert_logits_close(b, a, dtype, "%s against whole, %s" % (mode, rid))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_slots_and_pages_are_reused(models, tmp_path, dtype):
+    """Six batches through a cache that holds one batch: every page and slot is used again,
+    with stale keys of earlier requests still in it."""
+    name = "B"
+    path, cfg, weights = models[name]
+    requests = make_requests(cfg, [90, 40, 120, 66, 10, 128, 77, 30, 64, 100, 3, 50], seed=8)
+    ids = list(requests)
+    groups = [{r: requests[r] for r in ids[i:i + 2]} for i in range(0, len(ids), 2)]
+    steps = traces.batches(groups)
+    run_replay(path, dtype, steps, tmp_path, max_tokens=traces.max_tokens_needed(steps))
+    check(name, cfg, weights, requests, traces.collect(steps, str(tmp_path), cfg.vocab), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("use_graphs", [True, False])
+def test_long_decoding(models, tmp_path, dtype, use_graphs):
+    """A short prompt, then 200 tokens one by one across three page borders, three requests
+    of different lengths together."""
+    name = "A" if use_graphs else "C"
+    path, cfg, weights = models[name]
+    base = 120 if name == "A" else 260
+    requests = make_requests(cfg, [base, base - 57, base - 101], seed=5)
+    decode = {r: len(t) - 3 for r, t in requests.items()}
+    steps = traces.batches([requests], decode)
+    run_replay(path, dtype, steps, tmp_path, use_graphs=use_graphs)
+    check(name, cfg, weights, requests, traces.collect(steps, str(tmp_path), cfg.vocab), dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_first_tokens(models, tmp_path, dtype):
+    name = "B"
+    path, cfg, weights = models[name]
+    requests = make_requests(cfg, [1, 2, 3, 4], seed=6)
+    for mode, steps in (("whole", traces.whole(requests)), ("tail", traces.tail_one_by_one(requests)),
+                        ("batch", traces.batches([requests], {r: len(t) - 1 for r, t in requests.items()}))):
+        out_dir = tmp_path / mode
+        run_replay(path, dtype, steps, out_dir)
+        check(name, cfg, weights, requests, traces.collect(steps, str(out_dir), cfg.vocab), dtype)
+
+
+def _decode_rows(engine, requests, n_last):
+    from libllm_amd.engine import StepEntry
+    engine.step([StepEntry(r, t[:-n_last], []) for r, t in requests.items()])
+    rows = []
+    for i in range(n_last, 0, -1):
+        out = engine.step([StepEntry(r, [t[-i]], [0]) for r, t in requests.items()])
+        rows.append(out.cpu().numpy().copy())
+    return np.stack(rows)                                    # [steps, requests, vocab]
+
+
+def test_padding_changes_nothing(models):
+    """Three sequences decode through the graph captured for four rows, the fourth row being
+    padding.  In 32-bit the same bits come out without graphs (no padding row at all); in
+    bfloat16 the same bits come out when the fourth row is a real sequence."""
+    from libllm_amd.runtime import load_engine
+    path, cfg, weights = models["A"]
+    three = make_requests(cfg, [9, 70, 31], seed=12)
+    four = dict(three, extra=make_requests(cfg, [50], seed=13)["r0"])
+    padded = load_engine(path, dtype="float32", max_tokens=1024, use_graphs=True)
+    plain_path = load_engine(path, dtype="float32", max_tokens=1024, use_graphs=False)
+    a, b = _decode_rows(padded, three, 4), _decode_rows(plain_path, three, 4)
+    assert len(padded._graphs) == 1 and not plain_path._graphs
+    assert np.array_equal(a, b)
+    e3 = load_engine(path, dtype="bfloat16", max_tokens=1024, use_graphs=True)
+    e4 = load_engine(path, dtype="bfloat16", max_tokens=1024, use_graphs=True)
+    a, b = _decode_rows(e3, three, 4), _decode_rows(e4, four, 4)
+    assert list(e3._graphs) == [4] and list(e4._graphs) == [4]
+    assert np.array_equal(a, b[:, :3])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_trace_run_program(models, tmp_path, dtype):
+    """bin/trace_run as a user starts it: a child process fed through its standard input, one
+    step after each ``done`` line."""
+    name = "C"
+    path, cfg, weights = models[name]
+    requests = make_requests(cfg, [40, 7, 66], seed=21)
+    steps = traces.batches([requests], {"r0": 5, "r1": 6, "r2": 2})
+    out_dir = tmp_path / "out"
+    proc = subprocess.Popen([sys.executable, os.path.join(ROOT, "bin", "trace_run"), "--model", path,
+                             "--dtype", dtype, "--out", str(out_dir), "--max-tokens",
+                             str(traces.max_tokens_needed(steps))],
+                            stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
+    for s in steps:
+        proc.stdin.write(json.dumps(s) + "\n")
+        proc.stdin.flush()
+        assert proc.stdout.readline().strip() == "done %d" % s["step"]
+    proc.stdin.close()
+    assert proc.wait(timeout=60) == 0
+    check(name, cfg, weights, requests, traces.collect(steps, str(out_dir), cfg.vocab), dtype)
+
+
+def test_cache_full_is_an_error(models):
+    from libllm_amd import CacheError
+    from libllm_amd.engine import StepEntry
+    from libllm_amd.runtime import load_engine
+    path, cfg, _ = models["A"]
+    engine = load_engine(path, dtype="float32", max_tokens=128)
+    engine.step([StepEntry("a", [1] * 64, [])])
+    engine.step([StepEntry("b", [1] * 64, [])])
+    with pytest.raises(CacheError):
+        engine.step([StepEntry("a", [1], [0])])               # a third page does not exist
+    engine.end(["b"])
+    assert engine.step([StepEntry("a", [1], [0])]).shape == (1, cfg.vocab)
+    with pytest.raises(CacheError):
+        engine.step([StepEntry("c", [1] * 100, [])])          # beyond what is free; nothing is admitted
+    assert not engine.holds("c")
+    engine.cache.check()

@@ -1,0 +1,211 @@
+"""Each part of a layer alone on the GPU against the plain function it stands for, at sizes of its
+own, and the parts that tests define themselves."""
+import numpy as np
+import pytest
+import torch
+
+import toy
+import traces
+from helpers import assert_logits_close, make_ctx, make_kv, rel_err
+from libllm_amd.config import ScheduleEntry, config_from_dict
+from libllm_amd.engine import DecoderModel, Engine, StepEntry
+from libllm_amd.parts import Stream, build_block, build_feed_forward, build_mixer, build_norm
+from libllm_amd.parts.attention import AttentionSpec
+from libllm_amd.parts.mlp_swiglu import SwiGLUSpec
+from libllm_amd.parts.norm_rms import RMSNormSpec
+from libllm_amd.parts.rope import RotaryPosition, RotarySpec
+from libllm_amd.weights import random_tensors
+from plain import llama
+from tiny import TINY_A, TINY_B
+
+pytestmark = pytest.mark.gpu
+DTYPES = [torch.float32, torch.bfloat16]
+
+# a layer of its own shape: 5 heads in 5 groups... no: 10 heads over 5 kv heads, head size 48, width 112
+LAYER = {"hidden_size": 112, "num_attention_heads": 10, "num_key_value_heads": 5, "head_dim": 48,
+         "intermediate_size": 264, "num_hidden_layers": 1, "vocab_size": 300, "rms_norm_eps": 3e-6,
+         "rope_theta": 77777.0, "max_position_embeddings": 512, "tie_word_embeddings": False,
+         "rope_scaling": {"rope_type": "llama3", "factor": 4.0, "low_freq_factor": 1.0,
+                          "high_freq_factor": 4.0, "original_max_position_embeddings": 128},
+         "model_type": "llama"}
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from libllm_amd.hip import HipOps
+    return HipOps()
+
+
+def tol(dtype):
+    return 1e-4 if dtype == torch.float32 else 0.06
+
+
+def weights_for(part, prefix, seed, dtype):
+    decl = {prefix + k: v for k, v in part.weights().items()}
+    t = random_tensors(decl, seed, std=0.1, norm_std=0.3, dtype=torch.bfloat16)   # exactly representable
+    dev = {}
+    for k, v in t.items():
+        vector = decl[k].role == "vector"
+        dev[k[len(prefix):]] = v.to("cuda", torch.float32 if (vector or dtype == torch.float32) else dtype)
+    return dev, {k: v.double().numpy() for k, v in t.items()}
+
+
+def rows(m, width, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn((m, width), generator=g).to(torch.bfloat16).to(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_norm_part(ops, dtype):
+    norm = build_norm(RMSNormSpec(kind="rms", width=112, eps=3e-6))
+    dev, host = weights_for(norm, "n.", 1, dtype)
+    norm.bind(dev, ops, dtype)
+    ctx = make_ctx(ops, dtype, [(0, 0, 9)])
+    res = rows(9, 112, torch.float32, 2).cuda()
+    delta = rows(9, 112, dtype, 3).cuda()
+    stream = Stream(res.clone())
+    stream.delta = delta
+    out = norm.add_norm(ctx, stream)
+    x = res.double().cpu().numpy() + delta.double().cpu().numpy()
+    assert stream.delta is None and np.allclose(stream.res.cpu().numpy(), x, atol=1e-6)
+    assert rel_err(out.double().cpu().numpy(), llama.rms_norm(x, host["n.weight"], 3e-6)) < tol(dtype)
+
+
+def test_rotary_part_tables(ops):
+    for cfg in (TINY_B, LAYER, TINY_A):
+        spec = RotarySpec(kind="rotary", rot_dim=cfg["head_dim"], theta=cfg["rope_theta"],
+                          max_position=cfg["max_position_embeddings"], scaling=cfg["rope_scaling"])
+        part = RotaryPosition(spec)
+        inv = llama.rope_inv_freq(cfg["head_dim"], cfg["rope_theta"], cfg["rope_scaling"])
+        assert np.allclose(part.inv_freq().numpy(), inv, rtol=1e-12)
+        cos, sin = part.tables("cuda")
+        c, s = llama.rope_table(np.arange(cfg["max_position_embeddings"]), inv)
+        half = cfg["head_dim"] // 2
+        assert cos.dtype == torch.float32 and tuple(cos.shape) == (cfg["max_position_embeddings"], half)
+        assert np.abs(cos.cpu().numpy() - c[:, :half]).max() < 1e-7 and np.abs(sin.cpu().numpy() - s[:, :half]).max() < 1e-7
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_part(ops, dtype):
+    cfg = llama.PlainConfig(LAYER)
+    spec = config_from_dict(LAYER).to_spec().layers[0].mixer
+    assert isinstance(spec, AttentionSpec)
+    mixer = build_mixer(spec)
+    dev, host = weights_for(mixer, "model.layers.0.self_attn.", 4, dtype)
+    mixer.bind(dev, ops, dtype)
+    x = rows(150, 112, dtype, 5)
+    ref = llama.attention_block(cfg, host, 0, x.double().numpy(), np.arange(150))
+    # the whole sequence at once, then the same in two steps with a single token at the end
+    for cuts in ([150], [100, 49, 1]):
+        kv = make_kv("cuda", dtype, 2, 3, 5, 48, seed=len(cuts))
+        got, start = [], 0
+        for n in cuts:
+            ctx = make_ctx(ops, dtype, [(1, start, n)])
+            ctx._kv[0] = kv
+            got.append(mixer.forward(ctx, x[start:start + n].cuda().contiguous(), ScheduleEntry(0, 0)))
+            start += n
+        assert rel_err(torch.cat(got).double().cpu().numpy(), ref) < tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_feed_forward_part(ops, dtype):
+    cfg = llama.PlainConfig(LAYER)
+    ff = build_feed_forward(SwiGLUSpec(kind="swiglu", width=112, intermediate=264))
+    dev, host = weights_for(ff, "model.layers.0.mlp.", 6, dtype)
+    ff.bind(dev, ops, dtype)
+    for m in (1, 70):                                              # few rows and many take different kernels
+        x = rows(m, 112, dtype, 7)
+        out = ff.forward(make_ctx(ops, dtype, [(0, 0, m)]), x.cuda())
+        assert rel_err(out.double().cpu().numpy(), llama.mlp(cfg, host, 0, x.double().numpy())) < tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_block_arrangement(ops, dtype):
+    cfg = llama.PlainConfig(LAYER)
+    ls = config_from_dict(LAYER).to_spec().layers[0]
+    block = build_block(ls.block, build_mixer(ls.mixer), build_feed_forward(ls.feed_forward),
+                        [build_norm(n) for n in ls.norms])
+    host = {}
+    for role, part in (("mixer", block.mixer), ("feed_forward", block.feed_forward),
+                       ("norm0", block.norms[0]), ("norm1", block.norms[1])):
+        dev, h = weights_for(part, ls.prefixes[role], 8 + len(host), dtype)
+        part.bind(dev, ops, dtype)
+        host.update(h)
+    x = rows(75, 112, torch.float32, 9)
+    kv = make_kv("cuda", dtype, 1, 2, 5, 48)
+    ctx = make_ctx(ops, dtype, [(0, 0, 75)])
+    ctx._kv[0] = kv
+    stream = Stream(x.cuda().clone())
+    block.forward(ctx, stream, ScheduleEntry(0, 0))
+    out = stream.res.double().cpu().numpy() + stream.delta.double().cpu().numpy()   # the next norm adds it
+    assert rel_err(out, llama.decode_layer(cfg, host, 0, x.double().numpy(), np.arange(75))) < tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embedding_and_head_without_layers(ops, dtype):
+    spec = config_from_dict(dict(LAYER, tie_word_embeddings=True)).to_spec()
+    spec.layers, spec.schedule = [], []
+    model = DecoderModel(spec)
+    t = random_tensors(model.declared(), 3, std=0.1, norm_std=0.3)
+    model.bind({k: v.to("cuda", torch.float32 if (dtype == torch.float32 or v.dim() == 1) else dtype)
+                for k, v in t.items()}, ops, dtype)
+    engine = Engine(model, ops, dtype, max_tokens=64)
+    ids = [3, 299, 0, 17]
+    out = engine.step([StepEntry("a", ids, [0, 1, 2, 3])])
+    e = t["model.embed_tokens.weight"].double().numpy()
+    ref = llama.rms_norm(e[ids], t["model.norm.weight"].double().numpy(), 3e-6) @ e.T   # tied: the table again
+    assert rel_err(out.double().cpu().numpy(), ref) < tol(dtype)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_mixer_registers_builds_and_steps(ops, dtype):
+    """A mixer with state of its own, defined in tests/toy.py, inside a Llama model on the GPU."""
+    cfg_t = config_from_dict(TINY_A)
+    cfg = llama.PlainConfig(TINY_A)
+    model = DecoderModel(toy.toy_spec(cfg_t))
+    t = random_tensors(model.declared(), 7, std=0.1, norm_std=0.2)
+    model.bind({k: v.to("cuda", torch.float32 if (dtype == torch.float32 or v.dim() == 1) else dtype)
+                for k, v in t.items()}, ops, dtype)
+    engine = Engine(model, ops, dtype, max_tokens=512)
+    assert not engine.use_graphs and list(engine.cache.state) == [1]
+    w = {k: v.double().numpy() for k, v in t.items()}
+    rng = np.random.default_rng(5)
+    reqs = {"a": rng.integers(0, 256, size=30).tolist(), "b": rng.integers(0, 256, size=11).tolist()}
+    steps = traces.batches([reqs, {"c": reqs["b"]}], {"a": 12, "b": 4, "c": 10})
+    got = {}
+    for s in steps:
+        out = engine.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        row = 0
+        for e in s["entries"]:
+            for _ in e["want"]:
+                got.setdefault(e["id"], []).append(out[row].double().cpu().numpy())
+                row += 1
+        engine.end(s["end"])
+    for rid, toks in (("a", reqs["a"]), ("b", reqs["b"]), ("c", reqs["b"])):
+        ref = toy.toy_oracle(cfg, w, w["model.layers.1.toy.mix.weight"], toks)
+        assert_logits_close(np.stack(got[rid]), ref, dtype, rid)
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_schedule_and_mixed_layers_on_the_gpu(ops, dtype):
+    """A layer run twice, a run that reads another run's keys, and a layer with a window and
+    another grouping: whole prompts and single tokens agree."""
+    spec = config_from_dict(TINY_A).to_spec()
+    spec.layers[1].mixer.n_kv_heads = 4
+    spec.layers[1].mixer.window = 70
+    spec.schedule = [ScheduleEntry(0, 0), ScheduleEntry(1, 1), ScheduleEntry(0, 2), ScheduleEntry(1, 1, writes=False)]
+    model = DecoderModel(spec)
+    t = random_tensors(model.declared(), 9, std=0.1, norm_std=0.2)
+    model.bind({k: v.to("cuda", torch.float32 if (dtype == torch.float32 or v.dim() == 1) else dtype)
+                for k, v in t.items()}, ops, dtype)
+    engine = Engine(model, ops, dtype, max_tokens=256)
+    assert [(g.need.kind, g.entries) for g in engine.cache.groups] == [("full", [0, 2]), ("window", [1])]
+    ids = np.random.default_rng(4).integers(0, 256, size=128).tolist()
+    whole = engine.step([StepEntry("a", ids, list(range(128)))]).double().cpu().numpy()
+    engine.end(["a"])
+    cut = torch.cat([engine.step([StepEntry("b", ids[:90], list(range(90)))]).clone()] +
+                    [engine.step([StepEntry("b", [x], [0])]).clone() for x in ids[90:]]).double().cpu().numpy()
+    assert_logits_close(cut, whole, dtype, "cut against whole")
+    engine.end(["b"])
+    engine.cache.check()
