@@ -1,0 +1,206 @@
+#!/usr/bin/env python3
+"""Serving benchmark on one MI355X: decoded tokens a second of a Llama-3.2-1B-shaped model with
+random weights at batch 8 and a context of 4,096 tokens, plus the prefill of 2,048 tokens and
+decoding at batch 1 and 64.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
+
+A step is one decode step of the engine that generation uses: the step function over the cache
+(as a captured graph), arg-max sampling on the device and the sampled tokens fed back.  The
+sequences are first filled by real prompt steps so that the timed steps end at the context length.
+One JSON line is printed; everything else goes to standard error.
+
+The reference's own tool reports prompt and decoding speed of one sequence
+(src/libllm/benchmark_main.cc:52-86); it publishes no numbers, so ``vs_baseline`` is null.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+HBM_BYTES_PER_S = 8.0e12
+DENSE_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+# Llama-3.2-1B sizes
+FULL = {
+    "model_type": "llama", "num_hidden_layers": 16, "hidden_size": 2048, "num_attention_heads": 32,
+    "num_key_value_heads": 8, "head_dim": 64, "intermediate_size": 8192, "vocab_size": 128256,
+    "rope_theta": 500000.0,
+    "rope_scaling": {"rope_type": "llama3", "factor": 32.0, "low_freq_factor": 1.0,
+                     "high_freq_factor": 4.0, "original_max_position_embeddings": 8192},
+    "rms_norm_eps": 1e-5, "tie_word_embeddings": True, "max_position_embeddings": 131072,
+    "hidden_act": "silu", "bos_token_id": 128000, "eos_token_id": 128001,
+}
+
+
+def log(msg):
+    print("[bench] " + msg, file=sys.stderr, flush=True)
+
+
+def weight_bytes(cfg, itemsize):
+    """Bytes of every weight a decode step reads once (the tied table serves as output matrix)."""
+    h, i = cfg.hidden_size, cfg.intermediate_size
+    q, kv = cfg.num_attention_heads * cfg.head_dim, cfg.num_key_value_heads * cfg.head_dim
+    per_layer = (q + 2 * kv) * h + h * q + 3 * h * i
+    head = cfg.vocab_size * h
+    norms = (2 * cfg.num_hidden_layers + 1) * h * 4
+    return (cfg.num_hidden_layers * per_layer + head) * itemsize + norms
+
+
+def kv_bytes_per_token(cfg, itemsize):
+    return 2 * cfg.num_hidden_layers * cfg.num_key_value_heads * cfg.head_dim * itemsize
+
+
+def prefill_flops(cfg, t):
+    h, i = cfg.hidden_size, cfg.intermediate_size
+    q, kv = cfg.num_attention_heads * cfg.head_dim, cfg.num_key_value_heads * cfg.head_dim
+    linear = 2.0 * t * cfg.num_hidden_layers * ((q + 2 * kv) * h + h * q + 3 * h * i)
+    attention = cfg.num_hidden_layers * 4.0 * q * (t * (t + 1) / 2.0)
+    head = 2.0 * cfg.vocab_size * h                       # logits of the last position only
+    return linear + attention + head
+
+
+def fill(engine, torch, names, length, vocab, seed, chunk_tokens=16384):
+    """Brings every named sequence to ``length`` cached tokens through prompt steps."""
+    from libllm_amd.engine import StepEntry
+    g = torch.Generator().manual_seed(seed)
+    per_step = max(1, chunk_tokens // max(length, 1))
+    for i in range(0, len(names), per_step):
+        group = names[i:i + per_step]
+        entries = [StepEntry(n, torch.randint(0, vocab, (length,), generator=g).tolist(), [])
+                   for n in group]
+        engine.step(entries)
+    torch.cuda.synchronize()
+
+
+def decode_steps(engine, sampler, params, torch, names, tokens, n):
+    from libllm_amd.engine import StepEntry
+    for k in range(n):
+        logits = engine.step([StepEntry(r, [t], [0]) for r, t in zip(names, tokens)])
+        tokens = sampler.sample(logits, params, list(range(len(names))), [k] * len(names))
+    return tokens
+
+
+def time_decode(engine, sampler, params, torch, batch, context, steps, warmup, vocab, tag):
+    names = [(tag, i) for i in range(batch)]
+    start = context - steps - warmup
+    if start < 1:
+        raise SystemExit("context %d is too short for %d steps" % (context, steps + warmup))
+    fill(engine, torch, names, start, vocab, seed=batch)
+    tokens = [(11 * i + 5) % vocab for i in range(batch)]
+    tokens = decode_steps(engine, sampler, params, torch, names, tokens, warmup)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    decode_steps(engine, sampler, params, torch, names, tokens, steps)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    engine.end(names)
+    return dt
+
+
+def time_prefill(engine, torch, tokens, vocab, reps):
+    from libllm_amd.engine import StepEntry
+    g = torch.Generator().manual_seed(99)
+    prompt = torch.randint(0, vocab, (tokens,), generator=g).tolist()
+    best = None
+    for r in range(reps + 1):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        engine.step([StepEntry("prefill", prompt, [tokens - 1])])
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        engine.end(["prefill"])
+        if r > 0:                                           # the first run warms up
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--layers", type=int, default=FULL["num_hidden_layers"])
+    ap.add_argument("--batch", type=int, default=8)
+    ap.add_argument("--context", type=int, default=4096)
+    ap.add_argument("--prefill", type=int, default=2048)
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU only: this library does not run on several (--gpus %d)" % args.gpus)
+        return 2
+
+    import torch
+
+    from libllm_amd.config import config_from_dict
+    from libllm_amd.runtime import random_engine
+    from libllm_amd.sampling import Sampler, SamplingParams
+
+    d = dict(FULL)
+    d["num_hidden_layers"] = args.layers
+    cfg = config_from_dict(d)
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    itemsize = 2 if short == "bf16" else 4
+    biggest = max(args.batch, 1 if args.no_points else 64)
+    max_tokens = biggest * (args.context + 64) + 4096
+    log("building %d layers of %d with random weights, cache for %d tokens" %
+        (args.layers, FULL["num_hidden_layers"], max_tokens))
+    engine = random_engine(cfg, seed=0, dtype=args.dtype, max_tokens=max_tokens)
+    sampler = Sampler(engine.ops, cfg.vocab_size)
+    params = SamplingParams(temperature=0.0)
+    vocab = cfg.vocab_size
+
+    pre_s = time_prefill(engine, torch, args.prefill, vocab, reps=3)
+    pf = prefill_flops(cfg, args.prefill)
+    log("prefill of %d tokens: %.2f ms" % (args.prefill, pre_s * 1e3))
+
+    dt = time_decode(engine, sampler, params, torch, args.batch, args.context, args.steps, args.warmup,
+                     vocab, "main")
+    ms = dt / args.steps * 1e3
+    value = args.batch * args.steps / dt
+    log("decode at batch %d: %.3f ms a step, %.0f tokens/s" % (args.batch, ms, value))
+    mean_ctx = args.context - args.steps / 2.0
+    step_bytes = weight_bytes(cfg, itemsize) + args.batch * mean_ctx * kv_bytes_per_token(cfg, itemsize)
+    achieved = step_bytes / (dt / args.steps) / 1e9
+
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            dtb = time_decode(engine, sampler, params, torch, b, args.context, args.steps, args.warmup,
+                              vocab, "b%d" % b)
+            points["decode_b%d" % b] = round(b * args.steps / dtb, 1)
+            log("decode at batch %d: %.3f ms a step, %.0f tokens/s" % (b, dtb / args.steps * 1e3, b * args.steps / dtb))
+
+    out = {
+        "metric": "decode tok/s at batch %d, context %d (Llama-3.2-1B shape)" % (args.batch, args.context),
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": short,
+        "data": "synthetic: uniform random token ids, random weights N(0, 0.02)",
+        "config": {
+            "model": "Llama-3.2-1B shape", "layers": args.layers, "layers_full": FULL["num_hidden_layers"],
+            "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads,
+            "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
+            "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "tied_head": True,
+            "rope": "theta 5e5, llama3 factor 32", "global_batch": args.batch, "seq_len": args.context,
+            "prefill_tokens": args.prefill, "sampling": "greedy", "parallelism": "single GPU",
+        },
+        "prefill": {"value": round(args.prefill / pre_s, 1), "tokens": args.prefill,
+                    "ms": round(pre_s * 1e3, 3), "frac": round(pf / pre_s / DENSE_FLOPS[short], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_BYTES_PER_S / 1e9,
+                     "unit": "GB/s", "frac": round(achieved / (HBM_BYTES_PER_S / 1e9), 4)},
+        "points": points,
+    }
+    print(json.dumps(out), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

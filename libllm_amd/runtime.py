@@ -7,7 +7,8 @@ from .config import config_from_dir
 from .engine.model import DecoderModel
 from .engine.step import Engine
 from .errors import ConfigError
-from .weights import load_tensors
+from .weights import load_tensors, random_tensors
+from .weights.loader import place
 
 _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16,
            "float32": torch.float32, "fp32": torch.float32}
@@ -39,6 +40,27 @@ def load_engine(model_dir: str, dtype="bfloat16", max_tokens: int = 8192, ops=No
     model = DecoderModel(spec)
     ops = ops if ops is not None else default_ops()
     tensors = load_tensors(model_dir, model.declared(), spec.optional_tensors, tdtype, ops.device)
+    model.bind(tensors, ops, tdtype)
+    engine = Engine(model, ops, tdtype, max_tokens, max_slots=max_slots, use_graphs=use_graphs)
+    engine.config = config
+    return engine
+
+
+def random_engine(config, seed: int = 0, dtype="bfloat16", max_tokens: int = 8192, ops=None,
+                  max_slots: Optional[int] = None, use_graphs: bool = True, std: float = 0.02) -> Engine:
+    """The random-weights mode without a file: every tensor the model declares is drawn on the
+    device from ``seed`` (matrices normal with ``std``, norm scales 1) and bound as a loaded file
+    would be.  ``config`` is a typed configuration."""
+    tdtype = parse_dtype(dtype)
+    spec = config.to_spec()
+    model = DecoderModel(spec)
+    ops = ops if ops is not None else default_ops()
+    declared = model.declared()
+    tensors = {}
+    for name in sorted(declared):
+        t = random_tensors({name: declared[name]}, seed, std=std, dtype=torch.bfloat16,
+                           device=ops.device)[name]
+        tensors[name] = place(t, declared[name], tdtype, ops.device)
     model.bind(tensors, ops, tdtype)
     engine = Engine(model, ops, tdtype, max_tokens, max_slots=max_slots, use_graphs=use_graphs)
     engine.config = config

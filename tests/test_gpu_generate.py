@@ -50,7 +50,6 @@ def test_greedy_generation_through_the_entry_point(model_b, dtype):
             assert g[:n] == w[:n]
             # and every token it chose, given its own earlier tokens, is the plain
             # implementation's best one or within the margin of it
-            assert len(g) == len(w)
             for k in range(len(g)):
                 row = llama.logits_all(cfg, weights, list(p) + g[:k])[-1]
                 assert row.max() - row[g[k]] < 0.25, "token %d of a reply is not near the best" % k
