@@ -25,38 +25,85 @@ __device__ __forceinline__ float counter_uniform(uint64_t seed, uint64_t stream,
 }
 
 // ---------------------------------------------------------------------------------- arg-max
+// The largest logit of a row, the lowest index winning a tie (the reference's top_k == 1 case,
+// src/flint/cuda/test.cc:385-392).  Two stages so that a few rows still fill the GPU: blocks
+// (row, part) reduce a slice of the vocabulary to one (value, index) pair, then one block per row
+// reduces the pairs.
+__device__ __forceinline__ bool better(float v, int i, float bv, int bi) {
+  return v > bv || (v == bv && i < bi);
+}
+
 template <int NT>
-__global__ __launch_bounds__(NT) void argmax_kernel(const float* __restrict__ logits, int V,
-                                                     int* __restrict__ out) {
-  __shared__ float sv[NT / 64];
-  __shared__ int si[NT / 64];
-  const float* x = logits + (size_t)blockIdx.x * V;
-  float bv = -INFINITY;
-  int bi = 0x7fffffff;
-  for (int i = threadIdx.x; i < V; i += NT) {
-    const float v = x[i];
-    if (v > bv || (bi == 0x7fffffff && v == bv)) { bv = v; bi = i; }
-  }
+__device__ __forceinline__ void block_argmax(float& bv, int& bi, float* sv, int* si) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) {
     const float ov = __shfl_xor(bv, off, 64);
     const int oi = __shfl_xor(bi, off, 64);
-    if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+    if (better(ov, oi, bv, bi)) { bv = ov; bi = oi; }
   }
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   if (lane == 0) { sv[wave] = bv; si[wave] = bi; }
   __syncthreads();
   if (threadIdx.x == 0) {
     for (int w = 1; w < NT / 64; ++w)
-      if (sv[w] > bv || (sv[w] == bv && si[w] < bi)) { bv = sv[w]; bi = si[w]; }
-    out[blockIdx.x] = (bi == 0x7fffffff) ? 0 : bi;
+      if (better(sv[w], si[w], bv, bi)) { bv = sv[w]; bi = si[w]; }
   }
 }
 
-extern "C" int llm_argmax(const float* logits, int* out, int R, int V, hipStream_t stream) {
+template <int NT>
+__global__ __launch_bounds__(NT) void argmax_part_kernel(const float* __restrict__ logits, int V,
+                                                          int per_part, float* __restrict__ pv,
+                                                          int* __restrict__ pi) {
+  __shared__ float sv[NT / 64];
+  __shared__ int si[NT / 64];
+  const float* x = logits + (size_t)blockIdx.y * V;
+  const int lo = blockIdx.x * per_part;
+  const int hi = min(V, lo + per_part);
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int i = lo + threadIdx.x; i < hi; i += NT) {
+    const float v = x[i];
+    if (v > bv || (bi == 0x7fffffff && v == bv)) { bv = v; bi = i; }   // a thread's indices only grow
+  }
+  block_argmax<NT>(bv, bi, sv, si);
+  if (threadIdx.x == 0) {
+    pv[blockIdx.y * gridDim.x + blockIdx.x] = bv;
+    pi[blockIdx.y * gridDim.x + blockIdx.x] = bi;
+  }
+}
+
+template <int NT>
+__global__ __launch_bounds__(NT) void argmax_final_kernel(const float* __restrict__ pv,
+                                                           const int* __restrict__ pi, int parts,
+                                                           int* __restrict__ out) {
+  __shared__ float sv[NT / 64];
+  __shared__ int si[NT / 64];
+  float bv = -INFINITY;
+  int bi = 0x7fffffff;
+  for (int p = threadIdx.x; p < parts; p += NT) {
+    const float v = pv[blockIdx.x * parts + p];
+    const int i = pi[blockIdx.x * parts + p];
+    if (better(v, i, bv, bi)) { bv = v; bi = i; }
+  }
+  block_argmax<NT>(bv, bi, sv, si);
+  if (threadIdx.x == 0) out[blockIdx.x] = (bi == 0x7fffffff) ? 0 : bi;
+}
+
+// How many parts a row of V logits is cut into; the scratch arrays hold R * parts entries.
+extern "C" int llm_argmax_parts(int V) {
+  int parts = (V + 2047) / 2048;
+  return parts < 1 ? 1 : (parts > 256 ? 256 : parts);
+}
+
+extern "C" int llm_argmax(const float* logits, int* out, float* part_val, int* part_idx, int R, int V,
+                          hipStream_t stream) {
   if (R <= 0) return LLM_OK;
-  if (V <= 0) return LLM_ERR_ARG;
-  argmax_kernel<256><<<R, 256, 0, stream>>>(logits, V, out);
+  if (V <= 0 || R > 65535 || !part_val || !part_idx) return LLM_ERR_ARG;
+  const int parts = llm_argmax_parts(V);
+  const int per_part = (V + parts - 1) / parts;
+  argmax_part_kernel<256><<<dim3(parts, R), 256, 0, stream>>>(logits, V, per_part, part_val, part_idx);
+  if (hipGetLastError() != hipSuccess) return LLM_ERR_LAUNCH;
+  argmax_final_kernel<64><<<R, 64, 0, stream>>>(part_val, part_idx, parts, out);
   return llm_launch_status();
 }
 

@@ -38,13 +38,15 @@ _SIGNATURES = {
     "llm_gemm_f32": [_vp, _vp, _vp, _i, _i, _i, _vp],
     "llm_attention_ref": [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
                           _f, _i, _vp],
-    "llm_gemm_skinny_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "llm_gemm_skinny_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _vp],
+    "llm_gemm_skinny_swiglu_bf16": [_vp, _vp, _vp, _i, _i, _i, _vp],
     "llm_attention_mfma_supported": [_i],
     "llm_attention_prefill_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i,
                                    _i, _i, _f, _i, _vp],
     "llm_attention_decode_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i,
                                   _i, _i, _f, _i, _i, _vp],
-    "llm_argmax": [_vp, _vp, _i, _i, _vp],
+    "llm_argmax": [_vp, _vp, _vp, _vp, _i, _i, _vp],
+    "llm_argmax_parts": [_i],
     "llm_sample": [_vp, _vp, _i, _i, _f, _i, _f, _u64, _vp, _vp, _vp],
 }
 
@@ -172,9 +174,29 @@ class HipOps:
                 mm = min(self.SKINNY_ROWS, m - m0)
                 self._check(self.lib.llm_gemm_skinny_bf16(
                     x.data_ptr() + m0 * k * 2, w.data_ptr(), out.data_ptr() + m0 * n * out.element_size(),
-                    _code(odt), mm, n, k, 0, self._stream()), "gemm_skinny_bf16")
+                    _code(odt), mm, n, k, self._stream()), "gemm_skinny_bf16")
             return out
         return torch.matmul(x, w.t())
+
+    def linear_swiglu(self, x, w):
+        """silu(x Wg^T) * (x Wu^T) for the stacked weight ``w = [Wg; Wu]``: one kernel for few
+        rows in bfloat16, else the product followed by the SiLU-mul kernel."""
+        m, k = x.shape
+        two_i = w.shape[0]
+        if two_i % 2:
+            raise KernelError("linear_swiglu: the stacked weight has an odd number of rows")
+        inter = two_i // 2
+        if (self.fast_gemm and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+                and m <= self.SKINNY_ROWS and k % 8 == 0 and inter % 16 == 0 and k == w.shape[1]
+                and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
+            self._dev(x, "linear input")
+            self._dev(w, "linear weight")
+            out = torch.empty((m, inter), dtype=torch.bfloat16, device=self.device)
+            self._check(self.lib.llm_gemm_skinny_swiglu_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(),
+                                                             m, inter, k, self._stream()),
+                        "gemm_skinny_swiglu_bf16")
+            return out
+        return self.silu_mul(self.linear(x, w, None, x.dtype))
 
     def silu_mul(self, gu):
         m, two_i = gu.shape
@@ -279,7 +301,11 @@ class HipOps:
         r, v = logits.shape
         self._dev(logits, "logits", torch.float32)
         out = torch.empty((r,), dtype=torch.int32, device=self.device)
-        self._check(self.lib.llm_argmax(logits.data_ptr(), out.data_ptr(), r, v, self._stream()), "argmax")
+        parts = self.lib.llm_argmax_parts(v)
+        part_val = torch.empty((r * parts,), dtype=torch.float32, device=self.device)
+        part_idx = torch.empty((r * parts,), dtype=torch.int32, device=self.device)
+        self._check(self.lib.llm_argmax(logits.data_ptr(), out.data_ptr(), part_val.data_ptr(),
+                                        part_idx.data_ptr(), r, v, self._stream()), "argmax")
         return out
 
     def sample(self, logits, temperature, top_k, top_p, seed, streams: List[int], counters: List[int]):

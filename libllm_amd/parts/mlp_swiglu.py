@@ -52,6 +52,5 @@ class SwiGLU(FeedForward):
         self.down.bind(tensors[s.down_name + ".weight"])
 
     def forward(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
-        gu = self.gate_up(ctx, x)
-        h = ctx.ops.silu_mul(gu)
+        h = ctx.ops.linear_swiglu(x, self.gate_up.weight)
         return self.down(ctx, h)

@@ -34,6 +34,9 @@ class CpuOps:
             return y.to(torch.bfloat16)
         return y.to(out_dtype)
 
+    def linear_swiglu(self, x, w):
+        return self.silu_mul(self.linear(x, w, None, x.dtype))
+
     def silu_mul(self, gu):
         i = gu.shape[1] // 2
         g, u = gu[:, :i].float(), gu[:, i:].float()

@@ -135,11 +135,30 @@ def test_gemm_skinny_rows_per_block_and_batch_invariance(ops):
     big = rnd((200, k), torch.bfloat16, 14).cuda()       # many rows with float32 output: chunks of 64
     out = ops.linear(big, w, None, torch.float32)
     assert max_err(out, big.double() @ w.double().t()) < 2e-6
-    for rows in (16, 32, 64):
-        c = torch.empty((64, n), dtype=torch.float32, device="cuda")
-        st = ops.lib.llm_gemm_skinny_bf16(x.data_ptr(), w.data_ptr(), c.data_ptr(), 0, 64, n, k, rows,
-                                          torch.cuda.current_stream().cuda_stream)
-        assert st == 0 and max_err(c, full) < 2e-6
+    half = ops.linear(x, w, None, torch.bfloat16)         # the bfloat16 output is the rounded sum
+    assert torch.equal(half, full.to(torch.bfloat16))
+
+
+@pytest.mark.parametrize("m", [1, 7, 16, 30, 64])
+@pytest.mark.parametrize("ik", [(16, 8), (48, 136), (160, 64), (512, 192), (8192, 2048), (208, 1032)])
+def test_gemm_skinny_swiglu(ops, m, ik):
+    inter, k = ik
+    x = rnd((m, k), torch.bfloat16, 20).cuda()
+    w = rnd((2 * inter, k), torch.bfloat16, 21, 3.0 / k ** 0.5).cuda()
+    out = ops.linear_swiglu(x, w)
+    assert out.dtype == torch.bfloat16 and tuple(out.shape) == (m, inter)
+    gu = (x.double() @ w.double().t()).to(torch.bfloat16).double()    # the product is stored rounded
+    g, u = gu[:, :inter], gu[:, inter:]
+    ref = g / (1 + torch.exp(-g)) * u
+    assert max_err(out, ref) < 2 * BF16_2ULP
+    ops.fast_gemm = False                                               # the unfused path agrees
+    try:
+        slow = ops.linear_swiglu(x, w)
+    finally:
+        ops.fast_gemm = True
+    assert max_err(slow, ref) < 2 * BF16_2ULP
+    swapped = u / (1 + torch.exp(-u)) * g                               # gating the wrong half must differ
+    assert max_err(out, swapped) > 0.05
 
 
 def test_gemm_skinny_refuses(ops):
@@ -148,7 +167,7 @@ def test_gemm_skinny_refuses(ops):
     out = ops.linear(x, w, None, torch.bfloat16)
     assert close(out, x.double() @ w.double().t(), torch.bfloat16)
     c = torch.empty((2, 16), dtype=torch.bfloat16, device="cuda")
-    st = ops.lib.llm_gemm_skinny_bf16(x.data_ptr(), w.data_ptr(), c.data_ptr(), 1, 2, 16, 12, 0, 0)
+    st = ops.lib.llm_gemm_skinny_bf16(x.data_ptr(), w.data_ptr(), c.data_ptr(), 1, 2, 16, 12, 0)
     assert st == 1                                        # refused, not wrong
 
 
