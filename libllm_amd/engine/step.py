@@ -29,6 +29,7 @@ class Engine:
     """Owns a bound model, its cache and the step function."""
 
     GRAPH_BATCHES = (1, 2, 4, 8, 16, 32, 64)
+    GRAPH_MIN_CTX = 1024
 
     def __init__(self, model: DecoderModel, ops, dtype: torch.dtype, max_tokens: int,
                  max_slots: Optional[int] = None, use_graphs: bool = True):
@@ -40,7 +41,7 @@ class Engine:
         self.cache = SequenceCache(model.cache_needs(), model.state_needs(), max_tokens,
                                    model.spec.max_position, dtype, self.device, max_slots)
         self.use_graphs = bool(use_graphs) and ops.supports_graphs and model.graph_safe()
-        self._graphs: Dict[int, "_DecodeGraph"] = {}
+        self._graphs: Dict[tuple, "_DecodeGraph"] = {}     # (batch bucket, context bucket) -> graph
         self.steps_run = 0
 
     # ---- requests
@@ -157,18 +158,25 @@ class Engine:
     def _graph_step(self, entries, slots, pos0):
         b = len(entries)
         bucket = next(g for g in self.GRAPH_BATCHES if g >= b)
-        graph = self._graphs.get(bucket)
+        # the longest context a graph serves is part of its key: kernels size their grids by it
+        limit = self.cache.pages_per_seq * PAGE
+        ctx_bucket = self.GRAPH_MIN_CTX
+        while ctx_bucket < max(pos0) + 1:
+            ctx_bucket *= 2
+        ctx_bucket = min(ctx_bucket, limit)
+        graph = self._graphs.get((bucket, ctx_bucket))
         if graph is None:
-            graph = _DecodeGraph(self, bucket)
-            self._graphs[bucket] = graph
+            graph = _DecodeGraph(self, bucket, ctx_bucket)
+            self._graphs[(bucket, ctx_bucket)] = graph
         return graph.run([e.tokens[0] for e in entries], slots, pos0)
 
 
 class _DecodeGraph:
-    """One captured decode step for a batch of exactly ``bucket`` rows.  Rows beyond the live
-    sequences point at the cache's sink slot and page, so they change nothing that is read."""
+    """One captured decode step for a batch of exactly ``bucket`` rows whose sequences hold at
+    most ``max_ctx`` tokens after the step.  Rows beyond the live sequences point at the cache's
+    sink slot and page, so they change nothing that is read."""
 
-    def __init__(self, engine: Engine, bucket: int):
+    def __init__(self, engine: Engine, bucket: int, max_ctx: int):
         self.engine = engine
         self.bucket = bucket
         ops = engine.ops
@@ -185,7 +193,7 @@ class _DecodeGraph:
         ctx.seq_pos0 = self.static[o:o + b]; o += b
         self.want_rows = self.static[o:o + b]
         ctx.max_new = 1
-        ctx.max_ctx = engine.cache.pages_per_seq * PAGE
+        ctx.max_ctx = max_ctx
         ctx.decode = True
         ctx.captured = True
         engine._attach_cache(ctx)

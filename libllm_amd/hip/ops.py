@@ -43,8 +43,9 @@ _SIGNATURES = {
     "llm_attention_mfma_supported": [_i],
     "llm_attention_prefill_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i,
                                    _i, _i, _f, _i, _vp],
-    "llm_attention_decode_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _i,
-                                  _i, _i, _f, _i, _i, _vp],
+    "llm_attention_decode_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i,
+                                  _i, _i, _i, _f, _i, _i, _i, _vp],
+    "llm_attention_decode_waves": [_i],
     "llm_argmax": [_vp, _vp, _vp, _vp, _i, _i, _vp],
     "llm_argmax_parts": [_i],
     "llm_sample": [_vp, _vp, _i, _i, _f, _i, _f, _u64, _vp, _vp, _vp],
@@ -273,14 +274,16 @@ class HipOps:
                 pages = (ctx.max_ctx + 63) // 64
                 if window:
                     pages = min(pages, window // 64 + 2)
-                n_split = max(1, min(pages, 64, -(-1024 // (m * n_kv))))
-                part_o = torch.empty((m, n_heads, n_split, hd), dtype=torch.float32, device=self.device)
-                part_ml = torch.empty((m, n_heads, n_split, 2), dtype=torch.float32, device=self.device)
+                waves = self.lib.llm_attention_decode_waves(hd)
+                # a page for each wave, as long as the grid stays within a few thousand blocks
+                n_blocks = max(1, min(-(-pages // waves), max(1, 4096 // (m * n_kv))))
+                part_o = torch.empty((m, n_heads, n_blocks, hd), dtype=torch.float32, device=self.device)
+                part_ml = torch.empty((m, n_heads, n_blocks, 2), dtype=torch.float32, device=self.device)
                 self._check(self.lib.llm_attention_decode_bf16(
                     qkv.data_ptr(), width, kv.k_pages.data_ptr(), kv.v_pages.data_ptr(),
                     table.data_ptr(), table.shape[1], 64, ctx.seq_slot.data_ptr(),
-                    ctx.seq_pos0.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), m,
-                    n_heads, n_kv, hd, float(scale), int(window), n_split, self._stream()),
+                    ctx.seq_pos0.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), m, n_heads, n_kv, hd, float(scale),
+                    int(window), n_blocks, -(-pages // (n_blocks * waves)), self._stream()),
                     "attention_decode_bf16")
             else:
                 self._check(self.lib.llm_attention_prefill_bf16(
