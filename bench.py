@@ -80,11 +80,19 @@ def fill(engine, torch, names, length, vocab, seed, chunk_tokens=16384):
 
 
 def decode_steps(engine, sampler, params, torch, names, tokens, n):
+    """``n`` decode steps as the generation loop runs them: a step is queued with the tokens the
+    sampler left on the device, and the host reads each step's tokens while the next one runs."""
     from libllm_amd.engine import StepEntry
-    for k in range(n):
-        logits = engine.step([StepEntry(r, [t], [0]) for r, t in zip(names, tokens)])
-        tokens = sampler.sample(logits, params, list(range(len(names))), [k] * len(names))
-    return tokens
+    streams = list(range(len(names)))
+    logits = engine.step([StepEntry(r, [t], [0]) for r, t in zip(names, tokens)])
+    pending = sampler.sample_device(logits, params, streams, [0] * len(names))
+    placeholders = [StepEntry(r, [0], [0]) for r in names]
+    for k in range(1, n):
+        logits = engine.step(placeholders, tokens_device=pending.device)
+        ahead = sampler.sample_device(logits, params, streams, [k] * len(names))
+        pending.tokens()                                   # the host sees every token, one step late
+        pending = ahead
+    return pending.tokens()
 
 
 def time_decode(engine, sampler, params, torch, batch, context, steps, warmup, vocab, tag):

@@ -57,14 +57,71 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ res, const TD* __restrict
   for (int i = threadIdx.x; i < H; i += NT) Conv<TO>::store(o + i, x[i] * w[i] * inv);
 }
 
+// The same for rows of up to NT * 4 * NV elements (a multiple of 4): a thread keeps its share of
+// the row in registers, so the row, the delta and the weight are each read once and all loads are
+// in flight together.
+template <typename TD, typename TO, int NT, int NV>
+__global__ __launch_bounds__(NT) void add_rmsnorm_reg_kernel(float* __restrict__ res,
+                                                              const TD* __restrict__ delta,
+                                                              const float* __restrict__ w, float eps,
+                                                              TO* __restrict__ out,
+                                                              const int* __restrict__ rows, int H) {
+  __shared__ float scratch[NT / 64];
+  const int b = blockIdx.x;
+  const int r = rows ? rows[b] : b;
+  float* x = res + (size_t)r * H;
+  const TD* d = delta ? delta + (size_t)r * H : nullptr;
+  float4 v[NV], wv[NV];
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int i = (threadIdx.x + j * NT) * 4;
+    const bool in = i < H;
+    v[j] = in ? *reinterpret_cast<const float4*>(x + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+    wv[j] = in ? *reinterpret_cast<const float4*>(w + i) : make_float4(0.f, 0.f, 0.f, 0.f);
+    if (d && in) {
+      v[j].x += Conv<TD>::load(d + i);
+      v[j].y += Conv<TD>::load(d + i + 1);
+      v[j].z += Conv<TD>::load(d + i + 2);
+      v[j].w += Conv<TD>::load(d + i + 3);
+      *reinterpret_cast<float4*>(x + i) = v[j];
+    }
+  }
+  float ss = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) ss += v[j].x * v[j].x + v[j].y * v[j].y + v[j].z * v[j].z + v[j].w * v[j].w;
+  ss = block_sum<NT>(ss, scratch);
+  const float inv = 1.0f / sqrtf(ss / (float)H + eps);
+  TO* o = out + (size_t)b * H;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int i = (threadIdx.x + j * NT) * 4;
+    if (i < H) {
+      Conv<TO>::store(o + i, v[j].x * wv[j].x * inv);
+      Conv<TO>::store(o + i + 1, v[j].y * wv[j].y * inv);
+      Conv<TO>::store(o + i + 2, v[j].z * wv[j].z * inv);
+      Conv<TO>::store(o + i + 3, v[j].w * wv[j].w * inv);
+    }
+  }
+}
+
 extern "C" int llm_add_rmsnorm(float* res, const void* delta, int delta_dtype, const float* w,
                                float eps, void* out, int out_dtype, const int* rows, int n_out,
                                int H, hipStream_t stream) {
   if (n_out <= 0) return LLM_OK;
   if (H <= 0) return LLM_ERR_ARG;
   constexpr int NT = 256;
-#define LAUNCH(TD, TO) \
-  add_rmsnorm_kernel<TD, TO, NT><<<n_out, NT, 0, stream>>>(res, (const TD*)delta, w, eps, (TO*)out, rows, H)
+  const bool reg = (H % 4 == 0) && H <= NT * 4 * 4 && ((((uintptr_t)res) | ((uintptr_t)w)) & 15) == 0;
+  const bool reg2 = reg && H <= NT * 4 * 2;
+#define LAUNCH(TD, TO) do {                                                                         \
+  if (reg2)                                                                                         \
+    add_rmsnorm_reg_kernel<TD, TO, NT, 2><<<n_out, NT, 0, stream>>>(res, (const TD*)delta, w, eps,  \
+                                                                    (TO*)out, rows, H);             \
+  else if (reg)                                                                                     \
+    add_rmsnorm_reg_kernel<TD, TO, NT, 4><<<n_out, NT, 0, stream>>>(res, (const TD*)delta, w, eps,  \
+                                                                    (TO*)out, rows, H);             \
+  else                                                                                              \
+    add_rmsnorm_kernel<TD, TO, NT><<<n_out, NT, 0, stream>>>(res, (const TD*)delta, w, eps, (TO*)out, rows, H); \
+  } while (0)
   if (delta == nullptr) delta_dtype = out_dtype;
   if (delta_dtype == LLM_DTYPE_F32 && out_dtype == LLM_DTYPE_F32) LAUNCH(float, float);
   else if (delta_dtype == LLM_DTYPE_BF16 && out_dtype == LLM_DTYPE_BF16) LAUNCH(bf16_t, bf16_t);

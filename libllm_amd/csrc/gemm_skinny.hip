@@ -11,23 +11,39 @@
 // which step does not depend on M or on the tile shape: an output is the same bits whatever else
 // is in the batch.
 //
-// Epilogues: plain store, or SwiGLU over a stacked [gate; up] weight (out[m, i] =
+// Epilogues: plain store; SwiGLU over a stacked [gate; up] weight (out[m, i] =
 // silu(gate_i) * up_i, src/flint/cuda/swiglu.cu:44-49), where a wave owns a gate tile and the up
-// tile of the same columns; gate and up are rounded to the activation dtype first, as the
-// unfused path stores them.
+// tile of the same columns, gate and up rounded to the activation dtype first, as the unfused path
+// stores them; or accumulation into a float32 matrix (the residual stream).
+//
+// Fused RMS norm (up to 16 rows): X is then the float32 residual stream.  Staging multiplies each
+// element by the norm's weight and rounds to bfloat16, and sums the squares of the row on the way
+// (every block stages whole rows); the factor 1/sqrt(mean(x^2) + eps) of a row is applied to its
+// outputs in the epilogue (src/flint/cuda/rms_norm.cu:45-76 computes the same product).  `rows`
+// optionally names the rows of the stream to use.
 #include "mfma.h"
 
 #define SK_WK 8            // waves that split K
 #define SK_EPI_NONE 0
 #define SK_EPI_SWIGLU 1
+#define SK_EPI_ACCUM 2
 
 // MT: 16-row tiles of X; RT: 16-row tiles of W per wave; WN: row groups per block; G: granules of
 // 2 steps that a wave takes per chunk (a chunk is 512*G elements of K).
-template <int MT, int RT, int WN, int G, int EPI, typename OutT>
+struct SkinnyNorm {
+  const float* x;          // float32 rows [*, K]
+  const float* weight;     // [K]
+  const int* rows;         // row of x for each of the M rows, or null for 0..M-1
+  float eps;
+};
+
+template <int MT, int RT, int WN, int G, int EPI, bool XNORM, typename OutT>
 __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ X,
+                                                                      SkinnyNorm norm,
                                                                       const bf16_t* __restrict__ W,
                                                                       OutT* __restrict__ C, int M,
                                                                       int N, int K, int n_out) {
+  static_assert(!XNORM || (MT == 1 && WN == 1), "the fused norm is built for up to 16 rows");
   constexpr int NT = WN * SK_WK * 64;
   constexpr int CK = 512 * G;                    // elements of K per chunk
   constexpr int ROW_B = CK * 2;                  // bytes of a staged row; 16-byte pieces are swizzled
@@ -38,6 +54,8 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   constexpr int ROWS_PASS = NT / XV;             // rows staged per pass of the block
   constexpr int PASSES = (16 * MT + ROWS_PASS - 1) / ROWS_PASS;
   __shared__ __attribute__((aligned(16))) unsigned char lds[LDS_BYTES];
+  __shared__ float s_ss[XNORM ? SK_WK : 1][PASSES];
+  __shared__ float s_inv[16 * MT];
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int wn = wave / SK_WK, wk = wave % SK_WK;
@@ -72,19 +90,53 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   // staging of X: thread t carries piece (t % XV) of rows (t / XV) + p * ROWS_PASS
   const int x_col = tid % XV, x_row0 = tid / XV;
   uint4 xr[PASSES];
-  auto load_x = [&](int chunk) {
+  float4 xf[XNORM ? PASSES : 1][2], wf[2];
+  float ss[XNORM ? PASSES : 1];
+  const float* xsrc[XNORM ? PASSES : 1];
+  if (XNORM) {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
       const int row = x_row0 + p * ROWS_PASS;
-      const int k = chunk * CK + x_col * 8;
-      xr[p] = (row < M && k < K) ? *reinterpret_cast<const uint4*>(X + (size_t)row * K + k)
-                                 : make_uint4(0u, 0u, 0u, 0u);
+      ss[p] = 0.f;
+      const int src = (row < M) ? (norm.rows ? norm.rows[row] : row) : 0;
+      xsrc[p] = norm.x + (size_t)src * K;
+    }
+  }
+  auto load_x = [&](int chunk) {
+    const int k = chunk * CK + x_col * 8;
+    if (XNORM) {
+      const bool in = k < K;
+      wf[0] = in ? *reinterpret_cast<const float4*>(norm.weight + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+      wf[1] = in ? *reinterpret_cast<const float4*>(norm.weight + k + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int p = 0; p < PASSES; ++p) {
+        const int row = x_row0 + p * ROWS_PASS;
+        const bool ok = in && row < M;
+        xf[p][0] = ok ? *reinterpret_cast<const float4*>(xsrc[p] + k) : make_float4(0.f, 0.f, 0.f, 0.f);
+        xf[p][1] = ok ? *reinterpret_cast<const float4*>(xsrc[p] + k + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+    } else {
+#pragma unroll
+      for (int p = 0; p < PASSES; ++p) {
+        const int row = x_row0 + p * ROWS_PASS;
+        xr[p] = (row < M && k < K) ? *reinterpret_cast<const uint4*>(X + (size_t)row * K + k)
+                                   : make_uint4(0u, 0u, 0u, 0u);
+      }
     }
   };
   auto store_x = [&]() {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
       const int row = x_row0 + p * ROWS_PASS;
+      if (XNORM) {
+        const float4 a0 = xf[p][0], a1 = xf[p][1];
+        ss[p] += a0.x * a0.x + a0.y * a0.y + a0.z * a0.z + a0.w * a0.w + a1.x * a1.x + a1.y * a1.y +
+                 a1.z * a1.z + a1.w * a1.w;
+        xr[p].x = (uint32_t)f32_to_bf16(a0.x * wf[0].x) | ((uint32_t)f32_to_bf16(a0.y * wf[0].y) << 16);
+        xr[p].y = (uint32_t)f32_to_bf16(a0.z * wf[0].z) | ((uint32_t)f32_to_bf16(a0.w * wf[0].w) << 16);
+        xr[p].z = (uint32_t)f32_to_bf16(a1.x * wf[1].x) | ((uint32_t)f32_to_bf16(a1.y * wf[1].y) << 16);
+        xr[p].w = (uint32_t)f32_to_bf16(a1.z * wf[1].z) | ((uint32_t)f32_to_bf16(a1.w * wf[1].w) << 16);
+      }
       if (row < 16 * MT) *reinterpret_cast<uint4*>(lds + row * ROW_B + ((x_col ^ (row & 7)) * 16)) = xr[p];
     }
   };
@@ -139,6 +191,24 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
     __syncthreads();
   }
 
+  if (XNORM) {
+    // a wave stages one row per pass: rows (wave / (XV/64)) + p * ROWS_PASS; XV/64 waves share a row
+    constexpr int WPR = XV / 64;
+#pragma unroll
+    for (int p = 0; p < PASSES; ++p) {
+      const float t = wave_sum(ss[p]);
+      if (lane == 0) s_ss[wave][p] = t;
+    }
+    __syncthreads();
+    if (tid < 16 * MT) {
+      const int p = tid / ROWS_PASS, w0 = (tid % ROWS_PASS) * WPR;
+      float t = 0.f;
+#pragma unroll
+      for (int w = 0; w < WPR; ++w) t += s_ss[w0 + w][p];
+      s_inv[tid] = 1.0f / sqrtf(t / (float)K + norm.eps);
+    }
+  }
+
   // ---- add the partial sums of the 8 waves in order, apply the epilogue, store
   float* red = reinterpret_cast<float*>(lds);
 #pragma unroll
@@ -169,9 +239,10 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
         gsum[0] += pg.x; gsum[1] += pg.y; gsum[2] += pg.z; gsum[3] += pg.w;
         usum[0] += pu.x; usum[1] += pu.y; usum[2] += pu.z; usum[3] += pu.w;
       }
+      const float scale = XNORM ? s_inv[mt * 16 + (ln & 15)] : 1.0f;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float gt = bf16_to_f32(f32_to_bf16(gsum[e])), up = bf16_to_f32(f32_to_bf16(usum[e]));
+        const float gt = bf16_to_f32(f32_to_bf16(gsum[e] * scale)), up = bf16_to_f32(f32_to_bf16(usum[e] * scale));
         v[e] = up * gt / (1.0f + expf(-gt));
       }
       n = ((blockIdx.x * WN + w_n) * OUT_RT + ort) * 16 + 4 * (ln >> 4);
@@ -183,13 +254,19 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
             red + ((((w * WN + w_n) * RT + ort) * MT + mt) * 64 + ln) * 4);
         sum[0] += p.x; sum[1] += p.y; sum[2] += p.z; sum[3] += p.w;
       }
+      const float scale = XNORM ? s_inv[mt * 16 + (ln & 15)] : 1.0f;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] = sum[e];
+      for (int e = 0; e < 4; ++e) v[e] = sum[e] * scale;
       n = ((blockIdx.x * WN + w_n) * RT + ort) * 16 + 4 * (ln >> 4);
     }
     const int m = mt * 16 + (ln & 15);
     if (m >= M || n >= ldc) continue;
     OutT* dst = C + (size_t)m * ldc + n;
+    if (EPI == SK_EPI_ACCUM) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        if (n + e < ldc) v[e] += Conv<OutT>::load(dst + e);
+    }
     if (n + 3 < ldc && (ldc & 3) == 0) {
       if (sizeof(OutT) == 2) {
         uint2 pk;
@@ -207,53 +284,82 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   }
 }
 
-template <int MT, int RT, int WN, int G, int EPI, typename OutT>
-static int launch_skinny(const bf16_t* X, const bf16_t* W, OutT* C, int M, int N, int K, int n_out,
-                         hipStream_t stream) {
-  const int rows = (EPI == SK_EPI_SWIGLU) ? n_out : N;
+struct SkinnyArgs {
+  const bf16_t* X;
+  SkinnyNorm norm;
+  const bf16_t* W;
+  void* C;
+  int M, N, K, n_out;
+  hipStream_t stream;
+};
+
+template <int MT, int RT, int WN, int G, int EPI, bool XNORM, typename OutT>
+static int launch_skinny(const SkinnyArgs& a) {
+  const int rows = (EPI == SK_EPI_SWIGLU) ? a.n_out : a.N;
   const int tiles = (rows + 15) / 16;
   constexpr int OUT_RT = (EPI == SK_EPI_SWIGLU) ? RT / 2 : RT;
   const int blocks = (tiles + OUT_RT * WN - 1) / (OUT_RT * WN);
-  gemm_skinny_kernel<MT, RT, WN, G, EPI, OutT>
-      <<<blocks, WN * SK_WK * 64, 0, stream>>>(X, W, C, M, N, K, n_out);
+  gemm_skinny_kernel<MT, RT, WN, G, EPI, XNORM, OutT><<<blocks, WN * SK_WK * 64, 0, a.stream>>>(
+      a.X, a.norm, a.W, (OutT*)a.C, a.M, a.N, a.K, a.n_out);
   return llm_launch_status();
 }
 
 template <int EPI, typename OutT>
-static int pick_shape(const bf16_t* X, const bf16_t* W, OutT* C, int M, int N, int K, int n_out,
-                      hipStream_t stream) {
+static int pick_shape(const SkinnyArgs& a) {
   constexpr int RT = (EPI == SK_EPI_SWIGLU) ? 2 : 1;
-  switch ((M + 15) / 16) {
-    case 1: return launch_skinny<1, RT, 1, 2, EPI, OutT>(X, W, C, M, N, K, n_out, stream);
-    case 2: return launch_skinny<2, RT, 2 / RT, 1, EPI, OutT>(X, W, C, M, N, K, n_out, stream);
-    case 3: return launch_skinny<3, RT, 2 / RT, 1, EPI, OutT>(X, W, C, M, N, K, n_out, stream);
-    case 4: return launch_skinny<4, RT, 2 / RT, 1, EPI, OutT>(X, W, C, M, N, K, n_out, stream);
+  const int mt = (a.M + 15) / 16;
+  if (a.norm.x != nullptr) {
+    if (mt != 1) return LLM_ERR_ARG;
+    if constexpr (EPI != SK_EPI_ACCUM) return launch_skinny<1, RT, 1, 2, EPI, true, OutT>(a);
+    return LLM_ERR_ARG;
+  }
+  switch (mt) {
+    case 1: return launch_skinny<1, RT, 1, 2, EPI, false, OutT>(a);
+    case 2: return launch_skinny<2, RT, 2 / RT, 1, EPI, false, OutT>(a);
+    case 3: return launch_skinny<3, RT, 2 / RT, 1, EPI, false, OutT>(a);
+    case 4: return launch_skinny<4, RT, 2 / RT, 1, EPI, false, OutT>(a);
   }
   return LLM_ERR_ARG;
 }
 
-static bool skinny_args_ok(const void* X, const void* W, const void* C, int M, int K) {
-  if (M > 64 || K <= 0 || (K & 7)) return false;
-  if ((((uintptr_t)X) | ((uintptr_t)W) | ((uintptr_t)C)) & 15) return false;
-  return true;
-}
-
-extern "C" int llm_gemm_skinny_bf16(const void* X, const void* W, void* C, int out_dtype, int M, int N,
-                                    int K, hipStream_t stream) {
+// C[M, N] (epilogue 0: stored as out_dtype; 2: added into the float32 C) or C[M, N/2] (epilogue 1,
+// SwiGLU over W = [Wg; Wu], N/2 a multiple of 16) from X[M, K] and W[N, K].  X is bfloat16, or,
+// with norm_x given (M <= 16), the rows `norm_rows` of the float32 matrix norm_x, RMS-normalised
+// with norm_weight and norm_eps on the way.
+extern "C" int llm_gemm_skinny_bf16(const void* X, const float* norm_x, const float* norm_weight,
+                                    float norm_eps, const int* norm_rows, const void* W, void* C,
+                                    int epilogue, int out_dtype, int M, int N, int K,
+                                    hipStream_t stream) {
   if (M <= 0 || N <= 0) return LLM_OK;
-  if (!skinny_args_ok(X, W, C, M, K)) return LLM_ERR_ARG;
-  if (out_dtype == LLM_DTYPE_BF16)
-    return pick_shape<SK_EPI_NONE, bf16_t>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, N, K, N, stream);
-  if (out_dtype == LLM_DTYPE_F32)
-    return pick_shape<SK_EPI_NONE, float>((const bf16_t*)X, (const bf16_t*)W, (float*)C, M, N, K, N, stream);
+  if (M > 64 || K <= 0 || (K & 7)) return LLM_ERR_ARG;
+  const void* x = norm_x ? (const void*)norm_x : X;
+  if (x == nullptr || W == nullptr || C == nullptr) return LLM_ERR_ARG;
+  if ((((uintptr_t)x) | ((uintptr_t)W) | ((uintptr_t)C)) & 15) return LLM_ERR_ARG;
+  if (norm_x && (norm_weight == nullptr || (((uintptr_t)norm_weight) & 15) || M > 16 || !(norm_eps >= 0.f)))
+    return LLM_ERR_ARG;
+  SkinnyArgs a;
+  a.X = (const bf16_t*)X;
+  a.norm.x = norm_x;
+  a.norm.weight = norm_weight;
+  a.norm.rows = norm_rows;
+  a.norm.eps = norm_eps;
+  a.W = (const bf16_t*)W;
+  a.C = C;
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.n_out = N;
+  a.stream = stream;
+  if (epilogue == SK_EPI_NONE) {
+    if (out_dtype == LLM_DTYPE_BF16) return pick_shape<SK_EPI_NONE, bf16_t>(a);
+    if (out_dtype == LLM_DTYPE_F32) return pick_shape<SK_EPI_NONE, float>(a);
+  } else if (epilogue == SK_EPI_SWIGLU) {
+    if ((N & 31) || out_dtype != LLM_DTYPE_BF16) return LLM_ERR_ARG;
+    a.n_out = N / 2;
+    return pick_shape<SK_EPI_SWIGLU, bf16_t>(a);
+  } else if (epilogue == SK_EPI_ACCUM) {
+    if (out_dtype != LLM_DTYPE_F32) return LLM_ERR_ARG;
+    return pick_shape<SK_EPI_ACCUM, float>(a);
+  }
   return LLM_ERR_ARG;
-}
-
-// out[M, I] = silu(X Wg^T) * (X Wu^T) with W = [Wg; Wu] stacked, [2I, K]; I a multiple of 16.
-extern "C" int llm_gemm_skinny_swiglu_bf16(const void* X, const void* W, void* C, int M, int I, int K,
-                                           hipStream_t stream) {
-  if (M <= 0 || I <= 0) return LLM_OK;
-  if (!skinny_args_ok(X, W, C, M, K) || (I & 15)) return LLM_ERR_ARG;
-  return pick_shape<SK_EPI_SWIGLU, bf16_t>((const bf16_t*)X, (const bf16_t*)W, (bf16_t*)C, M, 2 * I, K, I,
-                                            stream);
 }

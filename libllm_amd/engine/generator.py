@@ -66,6 +66,20 @@ class SequenceState:
         return True
 
 
+class _Rows:
+    """Some rows of tokens that are still on their way to the host."""
+
+    def __init__(self, pending, index):
+        self._pending, self._index = pending, list(index)
+
+    def tokens(self):
+        all_tokens = self._pending.tokens()
+        return [all_tokens[i] for i in self._index]
+
+    def rows(self, index):
+        return self._pending.rows([self._index[i] for i in index])
+
+
 class Generator:
     """``engine`` needs ``step(entries)`` and ``end(requests)``; ``sampler`` needs
     ``sample(logits, params, streams, counters)``."""
@@ -106,17 +120,36 @@ class Generator:
             yield from self._run_batch(batch, prompts, params, max_new_tokens, stop)
 
     def _run_batch(self, batch, prompts, params, max_new_tokens, stop):
+        """One batch from its prompt step to its last token.
+
+        Where the engine takes tokens from the device and the sampler can leave them there, the
+        next step is queued before the host has seen the tokens it continues from: only a stop
+        token is news to the host, and a sequence that drew one has then run one step in vain,
+        whose result is dropped.  Everything else that ends a sequence (the token budget, the
+        position limit) is known from lengths alone, and such a sequence is not queued again."""
         self._serial += 1
         states = [SequenceState(i, len(prompts[i])) for i in batch]
         name = {st.index: ("gen", self._serial, st.index) for st in states}
         live = list(states)
+        ahead = (getattr(self.sampler, "samples_ahead", False)
+                 and getattr(self.engine, "takes_device_tokens", False))
         try:
             entries = [StepEntry(name[st.index], list(prompts[st.index]), [st.prompt_len - 1])
                        for st in live]
+            logits = self.engine.step(entries)
+            pending = self._draw(logits, params, live, 0, ahead)
             while True:
-                logits = self.engine.step(entries)
-                tokens = self.sampler.sample(logits, params, [st.index for st in live],
-                                             [len(st.output) for st in live])
+                queued = None
+                if ahead:
+                    # sequences that go on unless their token turns out to be a stop token
+                    cand = [st for st in live if len(st.output) + 1 < max_new_tokens
+                            and st.prompt_len + len(st.output) + 1 < self.max_position]
+                    if cand:
+                        rows = pending.rows([live.index(st) for st in cand])
+                        logits = self.engine.step([StepEntry(name[st.index], [0], [0]) for st in cand],
+                                                  tokens_device=rows)
+                        queued = (cand, self._draw(logits, params, cand, 1, True))
+                tokens = pending.tokens() if ahead else pending
                 ended, going, emitted = [], [], []
                 for st, tok in zip(live, tokens):
                     n_before = len(st.output)
@@ -130,11 +163,26 @@ class Generator:
                     yield item
                 if not live:
                     break
-                entries = [StepEntry(name[st.index], [st.output[-1]], [0]) for st in live]
+                if queued is not None:
+                    cand, drawn = queued
+                    pending = _Rows(drawn, [cand.index(st) for st in live])
+                else:
+                    logits = self.engine.step([StepEntry(name[st.index], [st.output[-1]], [0])
+                                               for st in live])
+                    pending = self._draw(logits, params, live, 0, ahead)
         finally:
             held = [name[st.index] for st in live if self._holds(name[st.index])]
             if held:
                 self.engine.end(held)
+
+    def _draw(self, logits, params, seqs, lead, ahead):
+        """Samples one token for each sequence; ``lead`` counts tokens that are drawn but not yet
+        in ``output``."""
+        streams = [st.index for st in seqs]
+        counters = [len(st.output) + lead for st in seqs]
+        if ahead:
+            return self.sampler.sample_device(logits, params, streams, counters)
+        return self.sampler.sample(logits, params, streams, counters)
 
     def _holds(self, request) -> bool:
         holds = getattr(self.engine, "holds", None)

@@ -120,7 +120,7 @@ class DecoderModel:
             self.blocks[entry.layer].forward(ctx, stream, entry)
         if want_rows is None or want_rows.numel() == 0:
             return None
-        h = self.final_norm.add_norm(ctx, stream, rows=want_rows)
+        h = self.final_norm.add_norm(ctx, stream, rows=want_rows, lazy=True)
         return ctx.ops.linear(h, self.head_weight, None, torch.float32)
 
 

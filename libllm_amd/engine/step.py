@@ -59,11 +59,24 @@ class Engine:
         return self.cache.length(self.cache.slot_of(request))
 
     # ---- the step
-    def step(self, entries: List[StepEntry]) -> Optional[torch.Tensor]:
+    takes_device_tokens = True
+
+    def step(self, entries: List[StepEntry], tokens_device: Optional[torch.Tensor] = None
+             ) -> Optional[torch.Tensor]:
         """Returns float32 logits ``[wanted, vocab]`` in the order of the entries and of their
-        ``want`` lists, or None if nothing is wanted."""
+        ``want`` lists, or None if nothing is wanted.
+
+        With ``tokens_device`` (int32 on the device, one per entry, for instance what the sampler
+        just wrote) every entry brings exactly one token and that tensor holds it: the ids in the
+        entries are placeholders, and the host need not know the tokens to start the step."""
         if not entries:
             raise RequestError("a step needs at least one entry")
+        if tokens_device is not None:
+            if (tokens_device.dtype != torch.int32 or tokens_device.device != self.device
+                    or tuple(tokens_device.shape) != (len(entries),)):
+                raise RequestError("tokens_device must be int32 on the device, one per entry")
+            if any(len(e.tokens) != 1 for e in entries):
+                raise RequestError("with tokens_device every entry brings exactly one token")
         seen = set()
         for e in entries:
             if e.request in seen:
@@ -72,7 +85,7 @@ class Engine:
             if len(e.tokens) == 0:
                 raise RequestError("request %r brings no tokens" % (e.request,))
             lo, hi = min(e.tokens), max(e.tokens)
-            if lo < 0 or hi >= self.vocab:
+            if tokens_device is None and (lo < 0 or hi >= self.vocab):
                 raise RequestError("request %r has a token id outside [0, %d)" % (e.request, self.vocab))
             for w in e.want:
                 if not 0 <= w < len(e.tokens):
@@ -104,9 +117,11 @@ class Engine:
         pos0 = [cache.length(s) for s in slots]
         want_all_single = all(n == 1 for n in lens) and all(list(e.want) == [0] for e in entries)
         if self.use_graphs and want_all_single and len(entries) <= self.GRAPH_BATCHES[-1]:
-            logits = self._graph_step(entries, slots, pos0)
+            logits = self._graph_step(entries, slots, pos0, tokens_device)
         else:
             ctx, want_rows = self._context(entries, slots, lens, pos0)
+            if tokens_device is not None:
+                ctx.tokens = tokens_device.contiguous()
             logits = self.model.forward(ctx, want_rows)
         for s, n in zip(slots, lens):
             cache.commit(s, n)
@@ -155,7 +170,7 @@ class Engine:
                 ctx._state[entry] = self.cache.state[entry]
 
     # ---- decoding one token per sequence through a captured graph
-    def _graph_step(self, entries, slots, pos0):
+    def _graph_step(self, entries, slots, pos0, tokens_device=None):
         b = len(entries)
         bucket = next(g for g in self.GRAPH_BATCHES if g >= b)
         # the longest context a graph serves is part of its key: kernels size their grids by it
@@ -168,7 +183,7 @@ class Engine:
         if graph is None:
             graph = _DecodeGraph(self, bucket, ctx_bucket)
             self._graphs[(bucket, ctx_bucket)] = graph
-        return graph.run([e.tokens[0] for e in entries], slots, pos0)
+        return graph.run([e.tokens[0] for e in entries], slots, pos0, tokens_device)
 
 
 class _DecodeGraph:
@@ -176,13 +191,19 @@ class _DecodeGraph:
     most ``max_ctx`` tokens after the step.  Rows beyond the live sequences point at the cache's
     sink slot and page, so they change nothing that is read."""
 
+    RING = 4
+
     def __init__(self, engine: Engine, bucket: int, max_ctx: int):
         self.engine = engine
         self.bucket = bucket
         ops = engine.ops
         b = bucket
-        self.host = np.zeros(7 * b + 1, dtype=np.int32)
-        self.static = ops.upload_int32(self.host)
+        # pinned host copies, so that an upload does not wait for the device; a ring of them, as
+        # the device may run several steps behind the host and each upload reads its copy late
+        self.ring = [torch.zeros(7 * b + 1, dtype=torch.int32, pin_memory=True) for _ in range(self.RING)]
+        self.ring_done = [None] * self.RING
+        self.turn = 0
+        self.static = self.ring[0].to(ops.device)
         ctx = StepContext(ops, engine.dtype, b, b)
         o = 0
         ctx.tokens = self.static[o:o + b]; o += b
@@ -209,7 +230,10 @@ class _DecodeGraph:
         b = self.bucket
         n = len(tokens)
         sink = self.engine.cache.sink_slot
-        h = self.host
+        self.turn = (self.turn + 1) % self.RING
+        if self.ring_done[self.turn] is not None:
+            self.ring_done[self.turn].synchronize()        # its last upload has been read
+        h = self.ring[self.turn].numpy()
         h[0:b] = 0
         h[0:n] = tokens
         h[b:2 * b] = 0
@@ -221,9 +245,14 @@ class _DecodeGraph:
         h[5 * b + 1:6 * b + 1] = 0
         h[5 * b + 1:5 * b + 1 + n] = pos0
         h[6 * b + 1:7 * b + 1] = np.arange(b)
-        self.static.copy_(torch.from_numpy(h))
+        self.static.copy_(self.ring[self.turn], non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+        self.ring_done[self.turn] = done
 
-    def run(self, tokens, slots, pos0):
+    def run(self, tokens, slots, pos0, tokens_device=None):
         self._fill(tokens, slots, pos0)
+        if tokens_device is not None:
+            self.static[:len(tokens)].copy_(tokens_device, non_blocking=True)
         self.graph.replay()
         return self.logits[:len(tokens)]

@@ -38,8 +38,7 @@ _SIGNATURES = {
     "llm_gemm_f32": [_vp, _vp, _vp, _i, _i, _i, _vp],
     "llm_attention_ref": [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
                           _f, _i, _vp],
-    "llm_gemm_skinny_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _vp],
-    "llm_gemm_skinny_swiglu_bf16": [_vp, _vp, _vp, _i, _i, _i, _vp],
+    "llm_gemm_skinny_bf16": [_vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
     "llm_attention_mfma_supported": [_i],
     "llm_attention_prefill_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i,
                                    _i, _i, _f, _i, _vp],
@@ -50,6 +49,15 @@ _SIGNATURES = {
     "llm_argmax_parts": [_i],
     "llm_sample": [_vp, _vp, _i, _i, _f, _i, _f, _u64, _vp, _vp, _vp],
 }
+
+
+class NormedRows:
+    """Rows ``rows`` (all, if None) of the float32 matrix ``res``, to be RMS-normalised with
+    ``weight`` and ``eps``: what ``HipOps.normed`` returns."""
+
+    def __init__(self, res, weight, eps, rows=None):
+        self.res, self.weight, self.eps, self.rows = res, weight, eps, rows
+        self.n_rows = res.shape[0] if rows is None else rows.shape[0]
 
 
 class HipOps:
@@ -138,20 +146,85 @@ class HipOps:
                                              n_out, h, self._stream()), "add_rmsnorm")
         return out
 
-    def linear(self, x, w, bias, out_dtype):
-        m, k = x.shape
+    SKINNY_ROWS = 64        # most rows the streaming matrix product takes at once
+    NORM_ROWS = 16          # most rows for which the norm is fused into the product
+    NORM_COLS = 4096        # and most rows of the weight
+    _EPI_NONE, _EPI_SWIGLU, _EPI_ACCUM = 0, 1, 2
+
+    def normed(self, res, weight, eps, rows=None):
+        """Rows of the float32 stream ``res`` that are to be RMS-normalised: a record that
+        ``linear`` and ``linear_swiglu`` take in place of a matrix, fusing the norm into the
+        product where they can and running the norm kernel first where they cannot."""
+        return NormedRows(res, weight, float(eps), rows)
+
+    def _materialise(self, x, dtype):
+        if isinstance(x, NormedRows):
+            return self.add_rmsnorm(x.res, None, x.weight, x.eps, dtype, x.rows)
+        return x
+
+    def _skinny_ok(self, x, w, m, k):
+        if not (self.fast_gemm and w.dtype == torch.bfloat16 and k % 8 == 0 and w.data_ptr() % 16 == 0):
+            return False
+        if isinstance(x, NormedRows):
+            # every block normalises the rows itself: worth it only while the blocks are few
+            return (m <= self.NORM_ROWS and w.shape[0] <= self.NORM_COLS
+                    and x.res.data_ptr() % 16 == 0 and x.weight.data_ptr() % 16 == 0)
+        return x.dtype == torch.bfloat16 and x.data_ptr() % 16 == 0
+
+    def _skinny(self, x, w, out, epilogue, m0=0, mm=None):
+        """Launches the skinny kernel on rows m0 .. m0+mm of x (a matrix or NormedRows)."""
+        n, k = w.shape
+        if isinstance(x, NormedRows):
+            xp, nx, nw, eps = None, x.res.data_ptr(), x.weight.data_ptr(), x.eps
+            rows = None if x.rows is None else x.rows.data_ptr()
+            mm = x.n_rows
+        else:
+            xp, nx, nw, eps, rows = x.data_ptr() + m0 * k * 2, None, None, 0.0, None
+        width = n // 2 if epilogue == self._EPI_SWIGLU else n
+        self._check(self.lib.llm_gemm_skinny_bf16(
+            xp, nx, nw, eps, rows, w.data_ptr(), out.data_ptr() + m0 * width * out.element_size(),
+            epilogue, _code(out.dtype), mm, n, k, self._stream()), "gemm_skinny_bf16")
+
+    def linear(self, x, w, bias, out_dtype, residual=None):
+        """x W^T (+ bias) as ``out_dtype``.  ``x`` is a matrix or a ``normed`` record.  With
+        ``residual`` (the float32 stream, same shape as the result) the product is added into it
+        where the kernel can do that, and None is returned; otherwise the result is returned and
+        the caller adds it."""
+        lazy = isinstance(x, NormedRows)
+        m, k = (x.n_rows, x.res.shape[1]) if lazy else x.shape
         n, k2 = w.shape
         if k != k2:
             raise KernelError("linear: x is [%d, %d] but the weight is [%d, %d]" % (m, k, n, k2))
-        self._dev(x, "linear input")
         self._dev(w, "linear weight")
+        if lazy:
+            self._dev(x.res, "residual stream", torch.float32)
+            self._dev(x.weight, "norm weight", torch.float32, (k,))
+        else:
+            self._dev(x, "linear input")
+        if self._skinny_ok(x, w, m, k) and bias is None:
+            if residual is not None and m <= self.SKINNY_ROWS:
+                self._dev(residual, "residual stream", torch.float32, (m, n))
+                self._skinny(x, w, residual, self._EPI_ACCUM, 0, m)
+                return None
+            if m <= self.SKINNY_ROWS or (out_dtype == torch.float32 and not lazy):
+                # float32 results for many rows (logits of whole prompts) go through the same kernel
+                # 64 rows at a time: a row's logits are then the same bits whatever the batch holds
+                odt = torch.float32 if out_dtype == torch.float32 else torch.bfloat16
+                out = torch.empty((m, n), dtype=odt, device=self.device)
+                for m0 in range(0, m, self.SKINNY_ROWS):
+                    self._skinny(x, w, out, self._EPI_NONE, m0, min(self.SKINNY_ROWS, m - m0))
+                return out
+        if lazy:
+            x = self._materialise(x, torch.float32 if w.dtype == torch.float32 else torch.bfloat16)
+            if self._skinny_ok(x, w, m, k) and bias is None:
+                return self.linear(x, w, None, out_dtype, residual)
         if w.dtype == torch.float32:
             xf = x if x.dtype == torch.float32 else x.float()
             out = torch.empty((m, n), dtype=torch.float32, device=self.device)
             self._check(self.lib.llm_gemm_f32(xf.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k,
                                               self._stream()), "gemm_f32")
         elif w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
-            out = self._linear_bf16(x, w, out_dtype)
+            out = torch.matmul(x, w.t())
         else:
             raise KernelError("linear: input %s with weight %s is not supported" % (x.dtype, w.dtype))
         if bias is not None:
@@ -160,43 +233,30 @@ class HipOps:
                                               self._stream()), "add_bias")
         return out if out.dtype == out_dtype else out.to(out_dtype)
 
-    SKINNY_ROWS = 64        # most rows the streaming matrix product takes at once
-
-    def _linear_bf16(self, x, w, out_dtype):
-        m, k = x.shape
-        n = w.shape[0]
-        skinny_ok = self.fast_gemm and k % 8 == 0 and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0
-        if skinny_ok and (m <= self.SKINNY_ROWS or out_dtype == torch.float32):
-            # float32 results for many rows (logits of whole prompts) go through the same kernel
-            # 64 rows at a time: a row's logits are then the same bits whatever the batch holds
-            odt = torch.float32 if out_dtype == torch.float32 else torch.bfloat16
-            out = torch.empty((m, n), dtype=odt, device=self.device)
-            for m0 in range(0, m, self.SKINNY_ROWS):
-                mm = min(self.SKINNY_ROWS, m - m0)
-                self._check(self.lib.llm_gemm_skinny_bf16(
-                    x.data_ptr() + m0 * k * 2, w.data_ptr(), out.data_ptr() + m0 * n * out.element_size(),
-                    _code(odt), mm, n, k, self._stream()), "gemm_skinny_bf16")
-            return out
-        return torch.matmul(x, w.t())
-
-    def linear_swiglu(self, x, w):
+    def linear_swiglu(self, x, w, dtype=None):
         """silu(x Wg^T) * (x Wu^T) for the stacked weight ``w = [Wg; Wu]``: one kernel for few
-        rows in bfloat16, else the product followed by the SiLU-mul kernel."""
-        m, k = x.shape
+        rows in bfloat16, else the product followed by the SiLU-mul kernel.  ``x`` is a matrix or
+        a ``normed`` record; ``dtype`` is the activation dtype (needed for a record)."""
+        lazy = isinstance(x, NormedRows)
+        m, k = (x.n_rows, x.res.shape[1]) if lazy else x.shape
+        dtype = dtype or (x.dtype if not lazy else None)
         two_i = w.shape[0]
         if two_i % 2:
             raise KernelError("linear_swiglu: the stacked weight has an odd number of rows")
         inter = two_i // 2
-        if (self.fast_gemm and x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-                and m <= self.SKINNY_ROWS and k % 8 == 0 and inter % 16 == 0 and k == w.shape[1]
-                and x.data_ptr() % 16 == 0 and w.data_ptr() % 16 == 0):
-            self._dev(x, "linear input")
+        if k != w.shape[1]:
+            raise KernelError("linear_swiglu: x is [%d, %d] but the weight is %s" % (m, k, tuple(w.shape)))
+        if (self._skinny_ok(x, w, m, k) and m <= self.SKINNY_ROWS and inter % 16 == 0
+                and dtype == torch.bfloat16):
             self._dev(w, "linear weight")
             out = torch.empty((m, inter), dtype=torch.bfloat16, device=self.device)
-            self._check(self.lib.llm_gemm_skinny_swiglu_bf16(x.data_ptr(), w.data_ptr(), out.data_ptr(),
-                                                             m, inter, k, self._stream()),
-                        "gemm_skinny_swiglu_bf16")
+            self._skinny(x, w, out, self._EPI_SWIGLU, 0, m)
             return out
+        if lazy:
+            if dtype is None:
+                raise KernelError("linear_swiglu: a normed record needs the activation dtype")
+            x = self._materialise(x, dtype)
+            return self.linear_swiglu(x, w, dtype)
         return self.silu_mul(self.linear(x, w, None, x.dtype))
 
     def silu_mul(self, gu):

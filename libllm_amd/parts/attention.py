@@ -36,6 +36,8 @@ class AttentionSpec(PartSpec):
 @register_mixer("attention")
 class Attention(Mixer):
     graph_safe = True      # reads nothing from the host during a step
+    takes_normed = True    # the input goes to a matrix product only
+    adds_to_stream = True  # the output product can add into the residual stream
 
     def __init__(self, spec: AttentionSpec):
         if min(spec.width, spec.n_heads, spec.n_kv_heads, spec.head_dim) <= 0:
@@ -92,7 +94,7 @@ class Attention(Mixer):
         self.out.bind(tensors[s.o_name + ".weight"])
         self.cos, self.sin = self.position.tables(w.device)
 
-    def forward(self, ctx: StepContext, x: torch.Tensor, entry) -> torch.Tensor:
+    def forward(self, ctx: StepContext, x, entry, residual=None):
         s = self.spec
         kv = ctx.kv(entry.cache)
         qkv = self.qkv(ctx, x) if entry.writes else self.q_only(ctx, x)
@@ -100,4 +102,4 @@ class Attention(Mixer):
                               self.position.rot_dim, ctx, kv, entry.writes)
         o = ctx.ops.attention(qkv, s.n_heads, s.n_kv_heads, s.head_dim, ctx, kv,
                               self.scale, s.window)
-        return self.out(ctx, o)
+        return self.out(ctx, o, residual=residual)

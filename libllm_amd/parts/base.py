@@ -133,7 +133,15 @@ class Mixer(Part):
     and returns rows of the same shape.  ``entry`` is the schedule entry of this run; the mixer
     reads its keys/values through ``ctx.kv(entry.cache)`` and its state through
     ``ctx.state(entry.cache)``, and writes them only if ``entry.writes``.
+
+    Two optional abilities, off unless the class sets them (they apply to feed-forwards too):
+    ``takes_normed = True``: ``x`` may be the record that ``ops.normed`` returns instead of a
+    matrix; the part hands it to ``ops.linear`` / ``ops.linear_swiglu`` only, which fuse the norm
+    into the product.  ``adds_to_stream = True``: ``forward`` takes a keyword ``residual`` (the
+    float32 stream) and may add its result into it, returning None.
     """
+    takes_normed = False
+    adds_to_stream = False
 
     def cache_need(self) -> Optional[CacheNeed]:
         return None
@@ -147,6 +155,8 @@ class Mixer(Part):
 
 class FeedForward(Part):
     """Row-wise transformation: ``forward(ctx, x [M, width]) -> [M, width]``."""
+    takes_normed = False
+    adds_to_stream = False
 
     def forward(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
         raise NotImplementedError
@@ -155,9 +165,11 @@ class FeedForward(Part):
 class Norm(Part):
     """``add_norm(ctx, stream, rows)``: adds ``stream.delta`` (if any) into ``stream.res`` in
     32-bit, then returns the normalised rows in the activation dtype.  With ``rows`` (int32
-    indices) only those rows are normalised and returned, in that order."""
+    indices) only those rows are normalised and returned, in that order.  With ``lazy`` a norm
+    that can be fused into a matrix product may return ``ctx.ops.normed(...)`` instead, when
+    nothing is left to add."""
 
-    def add_norm(self, ctx: StepContext, stream: Stream, rows=None) -> torch.Tensor:
+    def add_norm(self, ctx: StepContext, stream: Stream, rows=None, lazy=False) -> torch.Tensor:
         raise NotImplementedError
 
 

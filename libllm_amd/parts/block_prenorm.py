@@ -15,7 +15,14 @@ class PreNormBlock(Block):
         super().__init__(mixer, feed_forward, norms)
 
     def forward(self, ctx: StepContext, stream: Stream, entry) -> None:
-        h = self.norms[0].add_norm(ctx, stream)
-        stream.delta = self.mixer.forward(ctx, h, entry)
-        h = self.norms[1].add_norm(ctx, stream)
-        stream.delta = self.feed_forward.forward(ctx, h)
+        mixer, ff = self.mixer, self.feed_forward
+        h = self.norms[0].add_norm(ctx, stream, lazy=mixer.takes_normed)
+        if mixer.adds_to_stream:
+            stream.delta = mixer.forward(ctx, h, entry, residual=stream.res)
+        else:
+            stream.delta = mixer.forward(ctx, h, entry)
+        h = self.norms[1].add_norm(ctx, stream, lazy=ff.takes_normed)
+        if ff.adds_to_stream:
+            stream.delta = ff.forward(ctx, h, residual=stream.res)
+        else:
+            stream.delta = ff.forward(ctx, h)

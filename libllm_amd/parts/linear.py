@@ -16,5 +16,9 @@ class Linear:
         self.weight = weight.contiguous()
         self.bias = bias
 
-    def __call__(self, ctx, x: torch.Tensor, out_dtype=None) -> torch.Tensor:
-        return ctx.ops.linear(x, self.weight, self.bias, out_dtype or ctx.dtype)
+    def __call__(self, ctx, x, out_dtype=None, residual=None):
+        """``x``: a matrix or an ``ops.normed`` record.  With ``residual`` the result may be added
+        into it, and None returned."""
+        if residual is None:
+            return ctx.ops.linear(x, self.weight, self.bias, out_dtype or ctx.dtype)
+        return ctx.ops.linear(x, self.weight, self.bias, out_dtype or ctx.dtype, residual=residual)

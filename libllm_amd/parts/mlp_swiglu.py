@@ -24,6 +24,8 @@ class SwiGLUSpec(PartSpec):
 @register_feed_forward("swiglu")
 class SwiGLU(FeedForward):
     graph_safe = True      # reads nothing from the host during a step
+    takes_normed = True    # the input goes to a matrix product only
+    adds_to_stream = True  # the output product can add into the residual stream
 
     def __init__(self, spec: SwiGLUSpec):
         if spec.activation != "silu":
@@ -51,6 +53,6 @@ class SwiGLU(FeedForward):
         self.gate_up.bind(torch.cat([gate, up], dim=0))
         self.down.bind(tensors[s.down_name + ".weight"])
 
-    def forward(self, ctx: StepContext, x: torch.Tensor) -> torch.Tensor:
-        h = ctx.ops.linear_swiglu(x, self.gate_up.weight)
-        return self.down(ctx, h)
+    def forward(self, ctx: StepContext, x, residual=None):
+        h = ctx.ops.linear_swiglu(x, self.gate_up.weight, ctx.dtype)
+        return self.down(ctx, h, residual=residual)

@@ -29,7 +29,9 @@ class RMSNorm(Norm):
     def bind(self, tensors, ops, dtype):
         self.weight = tensors["weight"]
 
-    def add_norm(self, ctx: StepContext, stream: Stream, rows=None) -> torch.Tensor:
+    def add_norm(self, ctx: StepContext, stream: Stream, rows=None, lazy=False) -> torch.Tensor:
+        if lazy and stream.delta is None and hasattr(ctx.ops, "normed"):
+            return ctx.ops.normed(stream.res, self.weight, self.eps, rows)
         out = ctx.ops.add_rmsnorm(stream.res, stream.delta, self.weight, self.eps, ctx.dtype, rows)
         stream.delta = None
         return out

@@ -1,1 +1,1 @@
-from .sampler import TOP_K_MAX, Sampler, SamplingParams  # noqa: F401
+from .sampler import TOP_K_MAX, PendingTokens, Sampler, SamplingParams  # noqa: F401

@@ -49,10 +49,63 @@ class SamplingParams:
         return self.temperature == 0.0 or self.top_k == 1
 
 
+class PendingTokens:
+    """Tokens the sampler wrote on the device, on their way to the host on a stream of their own:
+    the device can go on with work queued behind the sampling while the host waits only for the
+    copy.  ``device`` is the int32 tensor; ``tokens()`` waits and returns the list."""
+
+    def __init__(self, device: torch.Tensor, copy_stream):
+        self.device = device
+        self._host = torch.empty(device.shape, dtype=device.dtype, pin_memory=True)
+        ready = torch.cuda.Event()
+        ready.record()
+        with torch.cuda.stream(copy_stream):
+            copy_stream.wait_event(ready)
+            self._host.copy_(device, non_blocking=True)
+            self._done = torch.cuda.Event()
+            self._done.record(copy_stream)
+        self._list = None
+
+    def tokens(self) -> List[int]:
+        if self._list is None:
+            self._done.synchronize()
+            self._list = [int(t) for t in self._host.tolist()]
+        return self._list
+
+    def rows(self, index: Sequence[int]) -> torch.Tensor:
+        """The device tokens of the given rows, in that order."""
+        if list(index) == list(range(self.device.shape[0])):
+            return self.device
+        idx = torch.tensor(list(index), dtype=torch.long).to(self.device.device, non_blocking=True)
+        return self.device.index_select(0, idx)
+
+
 class Sampler:
     def __init__(self, ops, vocab: int):
         self.ops = ops
         self.vocab = vocab
+        self._copy_stream = None
+
+    @property
+    def samples_ahead(self) -> bool:
+        """True if ``sample_device`` can leave the tokens on a GPU."""
+        return getattr(self.ops.device, "type", "cpu") == "cuda"
+
+    def sample_device(self, logits: torch.Tensor, params: SamplingParams, streams: Sequence[int],
+                      counters: Sequence[int]) -> PendingTokens:
+        """As ``sample``, but returns at once: the tokens stay on the device and travel to the
+        host on a side stream."""
+        p = params.validate(self.vocab)
+        if logits.shape[0] != len(streams) or len(streams) != len(counters):
+            raise RequestError("one stream and one counter per row of logits are needed")
+        if p.greedy:
+            out = self.ops.argmax(logits)
+        else:
+            out = self.ops.sample(logits, p.temperature, p.top_k, p.top_p, p.seed,
+                                  list(streams), list(counters))
+        if self._copy_stream is None:
+            self._copy_stream = torch.cuda.Stream(device=out.device)
+        return PendingTokens(out, self._copy_stream)
 
     def sample(self, logits: torch.Tensor, params: SamplingParams, streams: Sequence[int],
                counters: Sequence[int]) -> List[int]:

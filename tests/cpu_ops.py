@@ -26,7 +26,7 @@ class CpuOps:
         inv = torch.rsqrt((x * x).mean(dim=-1, keepdim=True) + eps)
         return (x * weight * inv).to(out_dtype)
 
-    def linear(self, x, w, bias, out_dtype):
+    def linear(self, x, w, bias, out_dtype, residual=None):
         y = x.float() @ w.float().t()
         if bias is not None:
             y = y + bias
@@ -34,7 +34,7 @@ class CpuOps:
             return y.to(torch.bfloat16)
         return y.to(out_dtype)
 
-    def linear_swiglu(self, x, w):
+    def linear_swiglu(self, x, w, dtype=None):
         return self.silu_mul(self.linear(x, w, None, x.dtype))
 
     def silu_mul(self, gu):

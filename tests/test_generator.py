@@ -139,3 +139,57 @@ def test_sampling_params():
     assert Sampler(Ops(), 4).sample(torch.tensor([[0.0, 2.0, 1.0, 2.0]]), SamplingParams(0.0), [0], [0]) == [1]
     with pytest.raises(RequestError):
         Sampler(Ops(), 4).sample(torch.zeros((2, 4)), SamplingParams(0.0), [0], [0])
+
+
+class AheadEngine(ScriptedEngine):
+    """Takes the tokens of a step from a 'device' tensor: the host's ids are placeholders."""
+    takes_device_tokens = True
+
+    def step(self, entries, tokens_device=None):
+        if tokens_device is not None:
+            assert len(tokens_device) == len(entries) and all(list(e.tokens) == [0] for e in entries)
+            entries = [type(e)(e.request, [int(t)], e.want) for e, t in zip(entries, tokens_device)]
+        return super().step(entries)
+
+
+class AheadSampler(ScriptedSampler):
+    samples_ahead = True
+
+    class Pending:
+        def __init__(self, toks):
+            self.toks, self.read = toks, False
+
+        def tokens(self):
+            self.read = True
+            return list(self.toks)
+
+        def rows(self, index):
+            assert not self.read, "the next step is queued before the host reads the tokens"
+            return [self.toks[i] for i in index]
+
+    def sample_device(self, logits, params, streams, counters):
+        return self.Pending(self.sample(logits, params, streams, counters))
+
+
+def test_steps_are_queued_ahead_and_a_stop_token_costs_one_step():
+    scripts = {0: [5, 6, 99, 1, 1], 1: [7, 99, 3], 2: [8, 9, 10, 11, 12]}
+    eng, smp = AheadEngine(scripts), AheadSampler()
+    gen = Generator(eng, smp, (99,), 10000, 1000, 64)
+    out = gen.generate([[1, 2, 3], [4], [5, 6]], SamplingParams(0.0), max_new_tokens=4)
+    assert out == [[5, 6], [7], [8, 9, 10, 11]]            # the same tokens as step by step
+    assert eng.steps[1] == [(0, [5], [0]), (1, [7], [0]), (2, [8], [0])]
+    # sequence 1 drew its stop token in step 1; step 2 was queued before the host saw it
+    assert eng.steps[2] == [(0, [6], [0]), (1, [99], [0]), (2, [9], [0])]
+    assert eng.steps[3] == [(0, [99], [0]), (2, [10], [0])]
+    assert len(eng.steps) == 4                              # the budget is known ahead: no step in vain
+    assert sorted(eng.ended) == [0, 1, 2] and not eng.live
+    # counters of the draws: the tokens drawn before, whether the host has seen them or not
+    assert smp.calls[1] == ([0, 1, 2], [1, 1, 1]) and smp.calls[2] == ([0, 1, 2], [2, 2, 2])
+    assert smp.calls[3] == ([0, 2], [3, 3])
+
+
+def test_queued_ahead_respects_the_position_limit():
+    eng, smp = AheadEngine({0: [5, 6, 7, 8, 9]}), AheadSampler()
+    gen = Generator(eng, smp, (99,), 5, 1000, 64)           # prompt 3 + 2 tokens reach the limit
+    assert gen.generate([[1, 2, 3]], SamplingParams(0.0), max_new_tokens=10) == [[5, 6]]
+    assert [s[0][1] for s in eng.steps] == [[1, 2, 3], [5]]  # no step beyond the limit

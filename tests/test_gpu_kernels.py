@@ -167,8 +167,54 @@ def test_gemm_skinny_refuses(ops):
     out = ops.linear(x, w, None, torch.bfloat16)
     assert close(out, x.double() @ w.double().t(), torch.bfloat16)
     c = torch.empty((2, 16), dtype=torch.bfloat16, device="cuda")
-    st = ops.lib.llm_gemm_skinny_bf16(x.data_ptr(), w.data_ptr(), c.data_ptr(), 1, 2, 16, 12, 0)
+    st = ops.lib.llm_gemm_skinny_bf16(x.data_ptr(), None, None, 0.0, None, w.data_ptr(), c.data_ptr(),
+                                      0, 1, 2, 16, 12, 0)
     assert st == 1                                        # refused, not wrong
+
+
+@pytest.mark.parametrize("m", [1, 5, 16, 40])
+@pytest.mark.parametrize("nk", [(16, 8), (300, 520), (2048, 2048), (72, 4104)])
+def test_gemm_skinny_adds_into_the_stream(ops, m, nk):
+    n, k = nk
+    x = rnd((m, k), torch.bfloat16, 30).cuda()
+    w = rnd((n, k), torch.bfloat16, 31).cuda()
+    res = rnd((m, n), torch.float32, 32, 5.0).cuda()
+    ref = res.double() + x.double() @ w.double().t()
+    assert ops.linear(x, w, None, torch.bfloat16, residual=res) is None
+    assert max_err(res, ref) < 2e-6
+    plain = ops.linear(x, w, None, torch.float32)          # the same sums as the plain product
+    again = rnd((m, n), torch.float32, 32, 5.0).cuda()
+    assert torch.equal(res, again + plain)
+
+
+@pytest.mark.parametrize("m", [1, 3, 8, 16, 20])
+@pytest.mark.parametrize("nk", [(16, 8), (300, 520), (3072, 2048), (72, 1032)])
+@pytest.mark.parametrize("gather", [False, True])
+def test_gemm_skinny_with_fused_norm(ops, m, nk, gather):
+    """A product over rows that are RMS-normalised on the way; beyond 16 rows the norm kernel
+    runs first.  Against the plain formulas, and against the unfused kernels."""
+    n, k = nk
+    stream = rnd((m + 3, k), torch.float32, 33, 7.0).cuda()
+    stream[0] *= 1e-3                                      # rows of very different size
+    wn = (1.0 + 0.3 * rnd((k,), torch.float32, 34)).cuda()
+    w = rnd((n, k), torch.bfloat16, 35).cuda()
+    rows = torch.tensor([(3 * i + 1) % (m + 3) for i in range(m)], dtype=torch.int32, device="cuda") if gather else None
+    src = stream[rows.long()] if gather else stream[:m]
+    sd = src.double()
+    h = sd * wn.double() / torch.sqrt((sd * sd).mean(dim=-1, keepdim=True) + 1e-5)
+    ref = h @ w.double().t()
+    lazy = ops.normed(stream if gather else stream[:m].contiguous(), wn, 1e-5, rows)
+    for out_dtype in DTYPES:
+        out = ops.linear(lazy, w, None, out_dtype)
+        assert out.dtype == out_dtype and tuple(out.shape) == (m, n)
+        assert max_err(out, ref) < (BF16_2ULP if out_dtype == torch.bfloat16 else 2.0 ** -8)
+    hb = ops.add_rmsnorm(stream if gather else stream[:m].contiguous(), None, wn, 1e-5, torch.bfloat16, rows)
+    unfused = ops.linear(hb, w, None, torch.float32)
+    assert max_err(ops.linear(lazy, w, None, torch.float32), unfused) < 2.0 ** -7
+    if n % 32 == 0:
+        g, u = ref[:, :n // 2], ref[:, n // 2:]
+        sw = ops.linear_swiglu(lazy, w, torch.bfloat16)
+        assert max_err(sw, g / (1 + torch.exp(-g)) * u) < 4 * BF16_2ULP
 
 
 def test_large_bf16_product(ops):
