@@ -107,50 +107,233 @@ __device__ __forceinline__ void load_query(const bf16_t* qrow, bool valid, Frag 
 }
 
 // ---------------------------------------------------------------------------------- prompts
-// grid (ceil(max_new / 64), n_heads, sequences), 4 waves, 16 query rows per wave.
+// A block of 4 waves owns 64 consecutive new tokens of one sequence and up to QT query heads that
+// share one kv head; wave w owns rows 16w .. 16w+15 for all those heads (QT tiles of 16 query
+// columns).  The block walks the pages its rows may see; a page's keys and values travel global
+// memory -> registers (issued one page ahead) -> shared memory, where all four waves read their
+// fragments, so a page is fetched once for 64 * QT queries.  16-byte pieces are swizzled in
+// shared memory so that the 16 rows a fragment load touches fall on different banks.
+// Blocks are numbered kv head first, so that the blocks of a kv head run on the same chiplet
+// and share its cache, and long rows first, since later rows see more keys.
 template <int HD>
+struct KeyRow {            // bytes between staged key rows: a power of two of at least 128
+  static constexpr int BYTES = (HD * 2 <= 128) ? 128 : ((HD * 2 <= 256) ? 256 : 512);
+};
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+// A page's keys and values: global memory -> registers (256 threads, 16 bytes each per round).
+template <int HD>
+__device__ __forceinline__ void fetch_page(const bf16_t* __restrict__ k_pages,
+                                           const bf16_t* __restrict__ v_pages, int page, int n_kv,
+                                           int kvh, u32x4 (&kreg)[(8 * HD + 255) / 256],
+                                           u32x4 (&vreg)[(8 * HD + 255) / 256]) {
+  constexpr int PIECES = 8 * HD, LOADS = (PIECES + 255) / 256;
+  const size_t base = ((size_t)page * n_kv + kvh) * PAGE * HD;
+  const u32x4* kp = reinterpret_cast<const u32x4*>(k_pages + base);
+  const u32x4* vp = reinterpret_cast<const u32x4*>(v_pages + base);
+#pragma unroll
+  for (int j = 0; j < LOADS; ++j) {
+    const int ci = threadIdx.x + j * 256;
+    const int cc = (PIECES % 256 == 0 || ci < PIECES) ? ci : 0;     // a piece past the end is not staged
+    kreg[j] = kp[cc];
+    vreg[j] = vp[cc];
+  }
+}
+
+// registers -> shared memory, 16-byte pieces swizzled within groups of 8.
+template <int HD>
+__device__ __forceinline__ void stage_page(unsigned char* k_lds, unsigned char* v_lds,
+                                           const u32x4 (&kreg)[(8 * HD + 255) / 256],
+                                           const u32x4 (&vreg)[(8 * HD + 255) / 256]) {
+  constexpr int PIECES = 8 * HD, LOADS = (PIECES + 255) / 256, KPR = HD / 8, KRB = KeyRow<HD>::BYTES;
+#pragma unroll
+  for (int j = 0; j < LOADS; ++j) {
+    const int ci = threadIdx.x + j * 256;
+    if (PIECES % 256 == 0 || ci < PIECES) {
+      const int krow = ci / KPR, kc = ci % KPR;
+      const int kf = (krow & 3) | (((krow >> 3) & 1) << 2);
+      *reinterpret_cast<u32x4*>(k_lds + krow * KRB + (((kc & ~7) | ((kc & 7) ^ kf)) * 16)) = kreg[j];
+      const int vrow = ci >> 3, vc = ci & 7;
+      *reinterpret_cast<u32x4*>(v_lds + vrow * 128 + ((vc ^ (vrow & 7)) * 16)) = vreg[j];
+    }
+  }
+}
+
+template <int HD, int QT>
 __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ v_pages, const int* __restrict__ table, int table_stride,
     const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_pos0, bf16_t* __restrict__ out, int n_heads, int n_kv,
-    float scale_log2, int window) {
-  const int b = blockIdx.z, h = blockIdx.y;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+    float scale_log2, int window, int n_qblocks, int n_chunks) {
+  constexpr int KS = (HD + 31) / 32, DT = HD / 16, KRB = KeyRow<HD>::BYTES;
+  constexpr int LOADS = (8 * HD + 255) / 256;    // 16-byte pieces of a page per thread
+  __shared__ __attribute__((aligned(16))) unsigned char k_lds[64 * KRB];
+  __shared__ __attribute__((aligned(16))) unsigned char v_lds[HD * 128];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
+  const int n_kvc = n_kv * n_chunks;
+  const int kvc = blockIdx.x % n_kvc, rest = blockIdx.x / n_kvc;
+  const int qb = n_qblocks - 1 - rest % n_qblocks, b = rest / n_qblocks;
+  const int kvh = kvc / n_chunks, chunk = kvc % n_chunks;
+  const int group = n_heads / n_kv;
+  const int per_chunk = (group + n_chunks - 1) / n_chunks;
+  const int h0 = kvh * group + chunk * per_chunk;
+  const int n_h = min(per_chunk, group - chunk * per_chunk);     // heads of this block (<= QT)
   const int start = seq_start[b];
   const int n = seq_start[b + 1] - start;
-  const int q0 = blockIdx.x * 64 + wave * 16;
-  if (q0 >= n) return;                                   // the whole wave leaves; no barriers below
+  const int q0b = qb * 64;
+  if (q0b >= n || n_h <= 0) return;                              // the whole block leaves
   const int pos0 = seq_pos0[b], slot = seq_slot[b];
-  const int kvh = h / (n_heads / n_kv);
-  const int row = q0 + r;
+  const int q0w = q0b + wave * 16;
+  const int row = q0w + r;
   const bool valid = row < n;
-  Frag qf[(HD + 31) / 32];
-  load_query<HD>(q + (size_t)(start + (valid ? row : n - 1)) * q_stride + (size_t)h * HD, valid, qf);
-  const int qpos = pos0 + row;
-  const int kmax = valid ? qpos : -1;
-  const int kmin = !valid ? 0x7fffffff : ((window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0);
-  const int first_pos = pos0 + q0;
-  const int last_pos = pos0 + ((q0 + 15 < n) ? q0 + 15 : n - 1);
-  const int pg_first = (window > 0 && first_pos - window + 1 > 0) ? (first_pos - window + 1) / PAGE : 0;
-  const int pg_last = last_pos / PAGE;
+  const int qpos = pos0 + row;                                   // rows past the end compute and are dropped
+  const int kmax = qpos;
+  const int kmin = (window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
 
-  AttnState<HD> st;
-  attn_init<HD>(st);
-  const int* trow = table + (size_t)slot * table_stride;
-  for (int pg = pg_first; pg <= pg_last; ++pg) {
-    const size_t base = ((size_t)trow[pg] * n_kv + kvh) * PAGE * HD;
-    attn_page<HD>(k_pages + base, v_pages + base, qf, scale_log2, pg * PAGE, kmin, kmax, st);
-  }
-  if (valid) {
-    const float inv = 1.0f / st.l;
-    bf16_t* orow = out + (size_t)(start + row) * n_heads * HD + (size_t)h * HD;
+  Frag qf[QT][KS];
 #pragma unroll
-    for (int dt = 0; dt < HD / 16; ++dt) {
-      uint2 pk;
-      pk.x = (uint32_t)f32_to_bf16(st.o[dt][0] * inv) | ((uint32_t)f32_to_bf16(st.o[dt][1] * inv) << 16);
-      pk.y = (uint32_t)f32_to_bf16(st.o[dt][2] * inv) | ((uint32_t)f32_to_bf16(st.o[dt][3] * inv) << 16);
-      *reinterpret_cast<uint2*>(orow + dt * 16 + 4 * g) = pk;
+  for (int qt = 0; qt < QT; ++qt)
+    load_query<HD>(q + (size_t)(start + (valid ? row : n - 1)) * q_stride + (size_t)(h0 + (qt < n_h ? qt : 0)) * HD,
+                   valid && qt < n_h, qf[qt]);
+
+  // pages of the block, and of this wave
+  const int last_row_b = (q0b + 63 < n) ? q0b + 63 : n - 1;
+  const int pg_first = (window > 0 && pos0 + q0b - window + 1 > 0) ? (pos0 + q0b - window + 1) / PAGE : 0;
+  const int pg_last = (pos0 + last_row_b) / PAGE;
+  const bool wave_live = q0w < n;
+  const int last_row_w = (q0w + 15 < n) ? q0w + 15 : n - 1;
+  const int wpg_first = (window > 0 && pos0 + q0w - window + 1 > 0) ? (pos0 + q0w - window + 1) / PAGE : 0;
+  const int wpg_last = wave_live ? (pos0 + last_row_w) / PAGE : -1;
+
+  f32x4 o[QT][DT], l_acc[QT];           // every row of l_acc holds the running sum of its column
+  float m_run[QT];
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    m_run[qt] = -INFINITY;
+    l_acc[qt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) o[qt][dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  }
+
+  const int* trow = table + (size_t)slot * table_stride;
+  u32x4 kreg[LOADS], vreg[LOADS];
+  fetch_page<HD>(k_pages, v_pages, trow[pg_first], n_kv, kvh, kreg, vreg);
+  for (int pg = pg_first; pg <= pg_last; ++pg) {
+    __syncthreads();                       // every wave is done with the page before
+    stage_page<HD>(k_lds, v_lds, kreg, vreg);
+    __syncthreads();
+    if (pg < pg_last) fetch_page<HD>(k_pages, v_pages, trow[pg + 1], n_kv, kvh, kreg, vreg);
+    if (pg < wpg_first || pg > wpg_last) continue;
+    const int key0 = pg * PAGE;
+
+    // ---- scores S^T[key][query] for 64 keys and QT * 16 queries
+    f32x4 sc[QT][4];
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt)
+#pragma unroll
+      for (int t4 = 0; t4 < 4; ++t4) sc[qt][t4] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t4 = 0; t4 < 4; ++t4) {
+      const int key_row = (t4 >> 1) * 32 + 8 * (r >> 2) + 4 * (t4 & 1) + (r & 3);
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        const int c = ks * 4 + g;
+        Frag a;
+        if (ks * 32 + g * 8 < HD)
+          a.u = *reinterpret_cast<const uint4*>(k_lds + key_row * KRB + (((c & ~7) | ((c & 7) ^ (r & 7))) * 16));
+        else
+          a = frag_zero();
+#pragma unroll
+        for (int qt = 0; qt < QT; ++qt) sc[qt][t4] = mfma_bf16(a, qf[qt][ks], sc[qt][t4]);
+      }
+    }
+    // a page wholly inside every row's view needs no mask
+    const bool mask = (key0 + 63 > pos0 + q0w) || (window > 0 && key0 < pos0 + q0w + 15 - window + 1);
+
+    // ---- running softmax per query column, probabilities as B fragments.  Maxima are taken of
+    // the raw scores (the scale is positive) and the scale goes into the exponent's multiply-add.
+    Frag p[QT][2];
+    float corr[QT];
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+      if (mask) {
+#pragma unroll
+        for (int t4 = 0; t4 < 4; ++t4)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int key = key0 + (t4 >> 1) * 32 + 8 * g + 4 * (t4 & 1) + e;
+            if (key < kmin || key > kmax) sc[qt][t4][e] = -INFINITY;
+          }
+      }
+      float mx = fmaxf(fmaxf(sc[qt][0][0], sc[qt][0][1]), fmaxf(sc[qt][0][2], sc[qt][0][3]));
+#pragma unroll
+      for (int t4 = 1; t4 < 4; ++t4)
+        mx = fmaxf(mx, fmaxf(fmaxf(sc[qt][t4][0], sc[qt][t4][1]), fmaxf(sc[qt][t4][2], sc[qt][t4][3])));
+      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+      const float m_new = fmaxf(m_run[qt], mx * scale_log2);
+      const float m_safe = (m_new > -INFINITY) ? m_new : 0.f;    // nothing seen yet: every p is 2^-inf = 0
+      corr[qt] = fast_exp2(m_run[qt] - m_safe);
+      m_run[qt] = m_new;
+#pragma unroll
+      for (int t4 = 0; t4 < 4; ++t4) {
+        const float p0 = fast_exp2(fmaf(sc[qt][t4][0], scale_log2, -m_safe));
+        const float p1 = fast_exp2(fmaf(sc[qt][t4][1], scale_log2, -m_safe));
+        const float p2 = fast_exp2(fmaf(sc[qt][t4][2], scale_log2, -m_safe));
+        const float p3 = fast_exp2(fmaf(sc[qt][t4][3], scale_log2, -m_safe));
+        uint32_t* dst = reinterpret_cast<uint32_t*>(&p[qt][t4 >> 1].u) + 2 * (t4 & 1);
+        dst[0] = pack2_bf16(p0, p1);
+        dst[1] = pack2_bf16(p2, p3);
+      }
+    }
+
+    // ---- O^T[d][query] += V^T[d][key] P^T[key][query]; a row of ones under V^T sums the rounded
+    // probabilities of each query the same way
+    Frag ones;
+    ones.u = make_uint4(0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u);
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+      f32x4 acc = l_acc[qt];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) acc[e] *= corr[qt];
+      acc = mfma_bf16(ones, p[qt][0], acc);
+      acc = mfma_bf16(ones, p[qt][1], acc);
+      l_acc[qt] = acc;
+    }
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+      const int d = dt * 16 + r;
+      Frag v0, v1;
+      v0.u = *reinterpret_cast<const uint4*>(v_lds + d * 128 + ((g ^ (r & 7)) * 16));
+      v1.u = *reinterpret_cast<const uint4*>(v_lds + d * 128 + (((g + 4) ^ (r & 7)) * 16));
+#pragma unroll
+      for (int qt = 0; qt < QT; ++qt) {
+        f32x4 acc = o[qt][dt];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) acc[e] *= corr[qt];
+        acc = mfma_bf16(v0, p[qt][0], acc);
+        acc = mfma_bf16(v1, p[qt][1], acc);
+        o[qt][dt] = acc;
+      }
+    }
+  }
+
+  if (valid) {
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) {
+      if (qt >= n_h) break;
+      const float inv = 1.0f / l_acc[qt][0];
+      bf16_t* orow = out + (size_t)(start + row) * n_heads * HD + (size_t)(h0 + qt) * HD;
+#pragma unroll
+      for (int dt = 0; dt < DT; ++dt) {
+        uint2 pk;
+        pk.x = (uint32_t)f32_to_bf16(o[qt][dt][0] * inv) | ((uint32_t)f32_to_bf16(o[qt][dt][1] * inv) << 16);
+        pk.y = (uint32_t)f32_to_bf16(o[qt][dt][2] * inv) | ((uint32_t)f32_to_bf16(o[qt][dt][3] * inv) << 16);
+        *reinterpret_cast<uint2*>(orow + dt * 16 + 4 * g) = pk;
+      }
     }
   }
 }
@@ -401,17 +584,26 @@ extern "C" int llm_attention_prefill_bf16(const void* q, int q_stride, const voi
       n_heads > 65535 || n_seqs > 65535)
     return LLM_ERR_ARG;
   const float scale_log2 = scale * 1.4426950408889634f;
-  dim3 grid((max_new + 63) / 64, n_heads, n_seqs);
+  const int group = n_heads / n_kv;
+  // One query head per block measured fastest (more blocks in flight, better balance between
+  // short and long rows) although a page is then staged once per query head of its group.
+  const int n_chunks = group;
+  const int n_qblocks = (max_new + 63) / 64;
+  const long long blocks = (long long)n_qblocks * n_kv * n_chunks * n_seqs;
+  if (blocks > 0x7fffffffLL) return LLM_ERR_ARG;
+#define LAUNCH(D, Q)                                                                              \
+  attn_prefill_kernel<D, Q><<<(unsigned)blocks, 256, 0, stream>>>(                                \
+      (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, table,          \
+      table_stride, seq_start, seq_slot, seq_pos0, (bf16_t*)out, n_heads, n_kv, scale_log2,       \
+      window, n_qblocks, n_chunks)
 #define CASE(D)                                                                                   \
   if (hd == D) {                                                                                  \
-    attn_prefill_kernel<D><<<grid, 256, 0, stream>>>(                                             \
-        (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, table,        \
-        table_stride, seq_start, seq_slot, seq_pos0, (bf16_t*)out, n_heads, n_kv, scale_log2,     \
-        window);                                                                                  \
+    LAUNCH(D, 1);                                                                                 \
     return llm_launch_status();                                                                   \
   }
   FOR_HEAD_DIMS(CASE)
 #undef CASE
+#undef LAUNCH
   return LLM_ERR_ARG;
 }
 

@@ -146,9 +146,40 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
   Conv<T>::store(out + (size_t)m * I + i, u * g / (1.0f + expf(-g)));
 }
 
+// The same for bfloat16 rows whose half width is a multiple of 8: 16 bytes of gate and of up per
+// thread, any number of rows through a grid-stride loop.
+__global__ void silu_mul_vec_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int I,
+                                    size_t total_vec) {
+  const int per_row = I / 8;
+  for (size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x; v < total_vec;
+       v += (size_t)gridDim.x * blockDim.x) {
+    const size_t m = v / per_row;
+    const int i = (int)(v % per_row) * 8;
+    const uint4 g4 = *reinterpret_cast<const uint4*>(gu + m * 2 * I + i);
+    const uint4 u4 = *reinterpret_cast<const uint4*>(gu + m * 2 * I + I + i);
+    const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
+      const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
+      const float r0 = u0 * g0 / (1.0f + expf(-g0)), r1 = u1 * g1 / (1.0f + expf(-g1));
+      ow[j] = (uint32_t)f32_to_bf16(r0) | ((uint32_t)f32_to_bf16(r1) << 16);
+    }
+    *reinterpret_cast<uint4*>(out + m * I + i) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+  }
+}
+
 extern "C" int llm_silu_mul(const void* gu, void* out, int dtype, int M, int I, hipStream_t stream) {
   if (M <= 0) return LLM_OK;
   if (I <= 0 || M > 65535 * 32) return LLM_ERR_ARG;
+  if (dtype == LLM_DTYPE_BF16 && I % 8 == 0 && ((((uintptr_t)gu) | ((uintptr_t)out)) & 15) == 0) {
+    const size_t total_vec = (size_t)M * (I / 8);
+    size_t blocks = (total_vec + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    silu_mul_vec_kernel<<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total_vec);
+    return llm_launch_status();
+  }
   // grid.y is limited to 65535: fold larger M into several launches
   for (int m0 = 0; m0 < M; m0 += 65535) {
     const int mm = (M - m0 < 65535) ? (M - m0) : 65535;

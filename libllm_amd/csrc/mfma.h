@@ -33,3 +33,15 @@ __device__ __forceinline__ Frag frag_load(const bf16_t* p) {
 __device__ __forceinline__ f32x4 mfma_bf16(const Frag& a, const Frag& b, f32x4 c) {
   return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, b.v, c, 0, 0, 0);
 }
+
+// Two floats rounded to bfloat16 (nearest even) by the hardware convert, packed low | high << 16.
+typedef __bf16 bf16x2_hw __attribute__((ext_vector_type(2)));
+typedef float f32x2_hw __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ uint32_t pack2_bf16(float lo, float hi) {
+  const f32x2_hw v = {lo, hi};
+  const bf16x2_hw b = __builtin_convertvector(v, bf16x2_hw);
+  return *reinterpret_cast<const uint32_t*>(&b);
+}
+
+// 2^x by the hardware instruction: results below the normal range become zero.
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
