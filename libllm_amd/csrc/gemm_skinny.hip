@@ -140,7 +140,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
       if (row < 16 * MT) *reinterpret_cast<uint4*>(lds + row * ROW_B + ((x_col ^ (row & 7)) * 16)) = xr[p];
     }
   };
-  Frag a[2][G][2][RT];
+  Frag a[3][G][2][RT];
   auto load_w = [&](int chunk, Frag (&dst)[G][2][RT]) {
 #pragma unroll
     for (int gi = 0; gi < G; ++gi)
@@ -168,28 +168,24 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
       }
   };
 
+  // W fragments are fetched two chunks ahead (three register stages in rotation), X one chunk
   load_x(0);
   load_w(0, a[0]);
-  for (int c = 0; c < n_chunks; c += 2) {
-    // even chunk from a[0], odd chunk from a[1]
-    store_x();
-    __syncthreads();
-    if (c + 1 < n_chunks) {
-      load_x(c + 1);
-      load_w(c + 1, a[1]);
-    }
-    compute(a[0]);
-    __syncthreads();
-    if (c + 1 >= n_chunks) break;
-    store_x();
-    __syncthreads();
-    if (c + 2 < n_chunks) {
-      load_x(c + 2);
-      load_w(c + 2, a[0]);
-    }
-    compute(a[1]);
-    __syncthreads();
+  if (1 < n_chunks) load_w(1, a[1]);
+#define SK_STEP(C, CUR, NXT)                    \
+  store_x();                                    \
+  __syncthreads();                              \
+  if ((C) + 1 < n_chunks) load_x((C) + 1);      \
+  if ((C) + 2 < n_chunks) load_w((C) + 2, NXT); \
+  compute(CUR);                                 \
+  __syncthreads();                              \
+  if ((C) + 1 >= n_chunks) break;
+  for (int c = 0;; c += 3) {
+    SK_STEP(c, a[0], a[2])
+    SK_STEP(c + 1, a[1], a[0])
+    SK_STEP(c + 2, a[2], a[1])
   }
+#undef SK_STEP
 
   if (XNORM) {
     // a wave stages one row per pass: rows (wave / (XV/64)) + p * ROWS_PASS; XV/64 waves share a row
