@@ -343,7 +343,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 // sequences); a wave's 16 query columns are the query heads of the kv head's group (in blocks of 16
 // if the group is larger).  The pages of the sequence are dealt out evenly to all waves of all
 // blocks of a (sequence, kv head); a wave loads a whole page (keys and values) into registers
-// before it computes, and the next page meanwhile.  The waves of a block merge their (O, m, l)
+// before it computes; several blocks share a compute unit, so one's loads overlap another's
+// arithmetic (keeping a second page in flight per wave cost more in occupancy than it gained).
+// The waves of a block merge their (O, m, l)
 // through shared memory; with several blocks each writes its merged partial to global memory and
 // a second kernel merges the partials in block order.
 template <int HD>
@@ -382,7 +384,7 @@ __device__ __forceinline__ void compute_page(const PageFrags<HD>& f, const Frag 
                                              AttnState<HD>& st) {
   constexpr int KS = (HD + 31) / 32;
   const int lane = threadIdx.x & 63, g = lane >> 4;
-  float s[4][4];
+  f32x4 s[4];
 #pragma unroll
   for (int t4 = 0; t4 < 4; ++t4) {
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -391,30 +393,33 @@ __device__ __forceinline__ void compute_page(const PageFrags<HD>& f, const Frag 
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
       const int key = key0 + (t4 >> 1) * 32 + 8 * g + 4 * (t4 & 1) + e;
-      s[t4][e] = (key >= kmin && key <= kmax) ? acc[e] * scale_log2 : -INFINITY;
+      if (key < kmin || key > kmax) acc[e] = -INFINITY;
     }
+    s[t4] = acc;
   }
   float mx = -INFINITY;
 #pragma unroll
   for (int t4 = 0; t4 < 4; ++t4)
-#pragma unroll
-    for (int e = 0; e < 4; ++e) mx = fmaxf(mx, s[t4][e]);
+    mx = fmaxf(mx, fmaxf(fmaxf(s[t4][0], s[t4][1]), fmaxf(s[t4][2], s[t4][3])));
   mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
   mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-  const float m_new = fmaxf(st.m, mx);
-  const bool any = m_new > -INFINITY;
-  const float corr = (st.m > -INFINITY) ? exp2f(st.m - m_new) : 0.f;
+  const float m_new = fmaxf(st.m, mx * scale_log2);
+  const float m_safe = (m_new > -INFINITY) ? m_new : 0.f;      // nothing seen yet: every p is 0
+  const float corr = fast_exp2(st.m - m_safe);
   float sum = 0.f;
   Frag p[2];
 #pragma unroll
-  for (int t4 = 0; t4 < 4; ++t4)
+  for (int t4 = 0; t4 < 4; ++t4) {
+    uint32_t* dst = reinterpret_cast<uint32_t*>(&p[t4 >> 1].u) + 2 * (t4 & 1);
 #pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      const float pv = (any && s[t4][e] > -INFINITY) ? exp2f(s[t4][e] - m_new) : 0.f;
-      const bf16_t pb = f32_to_bf16(pv);
-      p[t4 >> 1].h[4 * (t4 & 1) + e] = pb;
-      sum += bf16_to_f32(pb);          // the sum uses the rounded values that multiply V
+    for (int e = 0; e < 4; e += 2) {
+      const float p0 = fast_exp2(fmaf(s[t4][e], scale_log2, -m_safe));
+      const float p1 = fast_exp2(fmaf(s[t4][e + 1], scale_log2, -m_safe));
+      const uint32_t pk = pack2_bf16(p0, p1);
+      dst[e >> 1] = pk;
+      sum += __uint_as_float(pk << 16) + __uint_as_float(pk & 0xffff0000u);   // the rounded values
     }
+  }
   sum += __shfl_xor(sum, 16, 64);
   sum += __shfl_xor(sum, 32, 64);
   st.l = st.l * corr + sum;
@@ -430,8 +435,8 @@ __device__ __forceinline__ void compute_page(const PageFrags<HD>& f, const Frag 
   }
 }
 
-template <int HD, int WAVES, bool DOUBLE>
-__global__ __launch_bounds__(WAVES * 64, (!DOUBLE && HD <= 128) ? 2 : 1) void attn_decode_kernel(
+template <int HD, int WAVES>
+__global__ __launch_bounds__(WAVES * 64, (HD <= 128) ? 2 : 1) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ v_pages, const int* __restrict__ table, int table_stride,
     const int* __restrict__ seq_slot, const int* __restrict__ seq_pos0, float* __restrict__ part_o,
@@ -459,26 +464,7 @@ __global__ __launch_bounds__(WAVES * 64, (!DOUBLE && HD <= 128) ? 2 : 1) void at
     AttnState<HD> st;
     attn_init<HD>(st);
     const int lo = valid ? kmin : 0x7fffffff, hi = valid ? pos : -1;
-    if (DOUBLE) {
-      PageFrags<HD> f0, f1;
-      if (p0 < p1) {
-        const size_t base = ((size_t)trow[p0] * n_kv + kvh) * PAGE * HD;
-        load_page<HD>(k_pages + base, v_pages + base, f0);
-      }
-      for (int pg = p0; pg < p1; pg += 2) {
-        if (pg + 1 < p1) {
-          const size_t base = ((size_t)trow[pg + 1] * n_kv + kvh) * PAGE * HD;
-          load_page<HD>(k_pages + base, v_pages + base, f1);
-        }
-        compute_page<HD>(f0, qf, scale_log2, pg * PAGE, lo, hi, st);
-        if (pg + 1 >= p1) break;
-        if (pg + 2 < p1) {
-          const size_t base = ((size_t)trow[pg + 2] * n_kv + kvh) * PAGE * HD;
-          load_page<HD>(k_pages + base, v_pages + base, f0);
-        }
-        compute_page<HD>(f1, qf, scale_log2, (pg + 1) * PAGE, lo, hi, st);
-      }
-    } else {
+    {
       for (int pg = p0; pg < p1; ++pg) {
         const size_t base = ((size_t)trow[pg] * n_kv + kvh) * PAGE * HD;
         if (HD <= 128) {
@@ -608,14 +594,12 @@ extern "C" int llm_attention_prefill_bf16(const void* q, int q_stride, const voi
 }
 
 // part_o: [n_seqs, n_heads, n_blocks, hd] float32; part_ml: [n_seqs, n_heads, n_blocks, 2].
-// pages_per_wave: the most pages a wave will get (a hint: above 1 the kernel that keeps a second
-// page in flight is used).
 extern "C" int llm_attention_decode_bf16(const void* q, int q_stride, const void* k_pages,
                                          const void* v_pages, const int* table, int table_stride,
                                          int page_size, const int* seq_slot, const int* seq_pos0,
                                          float* part_o, float* part_ml, void* out,
                                          int n_seqs, int n_heads, int n_kv, int hd, float scale,
-                                         int window, int n_blocks, int pages_per_wave, hipStream_t stream) {
+                                         int window, int n_blocks, hipStream_t stream) {
   if (n_seqs <= 0) return LLM_OK;
   if (page_size != PAGE || !attn_args_ok(q, q_stride, k_pages, v_pages, n_heads, n_kv, hd, window) ||
       n_blocks <= 0 || n_blocks > 1024 || n_kv > 65535 || n_seqs > 65535 || n_heads > 65535 || hd > 256)
@@ -626,16 +610,10 @@ extern "C" int llm_attention_decode_bf16(const void* q, int q_stride, const void
 #define CASE(D)                                                                                   \
   if (hd == D) {                                                                                  \
     constexpr int WAVES = (D > 128) ? 2 : 4;                                                      \
-    if (pages_per_wave > 1 && D <= 64)                                                            \
-      attn_decode_kernel<D, WAVES, true><<<grid, WAVES * 64, 0, stream>>>(                        \
-          (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, table,      \
-          table_stride, seq_slot, seq_pos0, part_o, part_ml, (bf16_t*)out, n_heads, n_kv,         \
-          scale_log2, window);                                                                    \
-    else                                                                                          \
-      attn_decode_kernel<D, WAVES, false><<<grid, WAVES * 64, 0, stream>>>(                       \
-          (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, table,      \
-          table_stride, seq_slot, seq_pos0, part_o, part_ml, (bf16_t*)out, n_heads, n_kv,         \
-          scale_log2, window);                                                                    \
+    attn_decode_kernel<D, WAVES><<<grid, WAVES * 64, 0, stream>>>(                                \
+        (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, table,        \
+        table_stride, seq_slot, seq_pos0, part_o, part_ml, (bf16_t*)out, n_heads, n_kv,           \
+        scale_log2, window);                                                                      \
     if (n_blocks > 1) {                                                                           \
       if (hipGetLastError() != hipSuccess) return LLM_ERR_LAUNCH;                                 \
       attn_decode_combine_kernel<<<dim3(n_heads, n_seqs), ((hd + 63) / 64) * 64, 0, stream>>>(    \

@@ -43,7 +43,7 @@ _SIGNATURES = {
     "llm_attention_prefill_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i,
                                    _i, _i, _f, _i, _vp],
     "llm_attention_decode_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i,
-                                  _i, _i, _i, _f, _i, _i, _i, _vp],
+                                  _i, _i, _i, _f, _i, _i, _vp],
     "llm_attention_decode_waves": [_i],
     "llm_argmax": [_vp, _vp, _vp, _vp, _i, _i, _vp],
     "llm_argmax_parts": [_i],
@@ -343,8 +343,7 @@ class HipOps:
                     qkv.data_ptr(), width, kv.k_pages.data_ptr(), kv.v_pages.data_ptr(),
                     table.data_ptr(), table.shape[1], 64, ctx.seq_slot.data_ptr(),
                     ctx.seq_pos0.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), m, n_heads, n_kv, hd, float(scale),
-                    int(window), n_blocks, -(-pages // (n_blocks * waves)), self._stream()),
-                    "attention_decode_bf16")
+                    int(window), n_blocks, self._stream()), "attention_decode_bf16")
             else:
                 self._check(self.lib.llm_attention_prefill_bf16(
                     qkv.data_ptr(), width, kv.k_pages.data_ptr(), kv.v_pages.data_ptr(),
