@@ -220,6 +220,8 @@ extern "C" int llm_add_bias(void* x, int dtype, const float* b, int M, int N, hi
 // One block per token.  Row layout of qkv: [q heads | k heads | v heads], each head_dim wide.
 //   q, k: o[j] = x[j] c - x[j+r/2] s,  o[j+r/2] = x[j+r/2] c + x[j] s  for j < r/2, r = rot_dim
 //         (rotate-half pairing, src/libllm/llama.cc:151-176); dims >= r pass through.
+//   With `adjacent` the pairs are (2j, 2j+1) instead, still with the angle of pair j: the layout of
+//   a projection whose output rows were reordered so that the two dims of a pair lie side by side.
 //   q is rotated in place; k (rotated) and v go to the sequence's page of the cache:
 //   page = table[slot, pos / PAGE]; keys at [page, kv_head, pos % PAGE, d], values transposed at
 //   [page, kv_head, d, pos % PAGE].
@@ -230,7 +232,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride, const 
                                      const int* __restrict__ tok_pos, const int* __restrict__ tok_seq,
                                      const int* __restrict__ seq_slot, const int* __restrict__ table,
                                      int table_stride, T* __restrict__ k_pages, T* __restrict__ v_pages,
-                                     int write_kv) {
+                                     int write_kv, int adjacent) {
   const int m = blockIdx.x;
   const int pos = tok_pos[m];
   T* row = qkv + (size_t)m * row_stride;
@@ -256,11 +258,12 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride, const 
     const bool is_k = h >= n_heads;
     T* dst = is_k ? k_pages + page_base + (size_t)(h - n_heads) * PAGE * hd : x;
     if (j < half) {
-      float x1 = Conv<T>::load(x + j), x2 = Conv<T>::load(x + j + half);
-      if (b) { x1 += b[j]; x2 += b[j + half]; }
+      const int d1 = adjacent ? 2 * j : j, d2 = adjacent ? 2 * j + 1 : j + half;
+      float x1 = Conv<T>::load(x + d1), x2 = Conv<T>::load(x + d2);
+      if (b) { x1 += b[d1]; x2 += b[d2]; }
       const float cj = c[j], sj = s[j];
-      Conv<T>::store(dst + j, x1 * cj - x2 * sj);
-      Conv<T>::store(dst + j + half, x2 * cj + x1 * sj);
+      Conv<T>::store(dst + d1, x1 * cj - x2 * sj);
+      Conv<T>::store(dst + d2, x2 * cj + x1 * sj);
     } else {
       const int d = rot_dim + (j - half);
       float v = Conv<T>::load(x + d);
@@ -284,7 +287,8 @@ extern "C" int llm_rope_kv_write(void* qkv, int dtype, int row_stride, const flo
                                  int n_kv, int hd, const float* cos_t, const float* sin_t, int rot_dim,
                                  const int* tok_pos, const int* tok_seq, const int* seq_slot,
                                  const int* table, int table_stride, void* k_pages, void* v_pages,
-                                 int page_size, int write_kv, int M, hipStream_t stream) {
+                                 int page_size, int write_kv, int adjacent, int M,
+                                 hipStream_t stream) {
   if (M <= 0) return LLM_OK;
   if (page_size != 64 || hd <= 0 || n_heads <= 0 || n_kv < 0 || rot_dim < 0 || rot_dim > hd ||
       (rot_dim & 1))
@@ -296,11 +300,11 @@ extern "C" int llm_rope_kv_write(void* qkv, int dtype, int row_stride, const flo
   if (dtype == LLM_DTYPE_F32)
     rope_kv_write_kernel<float, 64><<<M, 256, 0, stream>>>(
         (float*)qkv, row_stride, bias, n_heads, n_kv, hd, cos_t, sin_t, rot_dim, tok_pos, tok_seq,
-        seq_slot, table, table_stride, (float*)k_pages, (float*)v_pages, write_kv);
+        seq_slot, table, table_stride, (float*)k_pages, (float*)v_pages, write_kv, adjacent);
   else if (dtype == LLM_DTYPE_BF16)
     rope_kv_write_kernel<bf16_t, 64><<<M, 256, 0, stream>>>(
         (bf16_t*)qkv, row_stride, bias, n_heads, n_kv, hd, cos_t, sin_t, rot_dim, tok_pos, tok_seq,
-        seq_slot, table, table_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, write_kv);
+        seq_slot, table, table_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, write_kv, adjacent);
   else
     return LLM_ERR_ARG;
   return llm_launch_status();

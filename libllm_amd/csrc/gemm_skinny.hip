@@ -16,6 +16,12 @@
 // tile of the same columns, gate and up rounded to the activation dtype first, as the unfused path
 // stores them; or accumulation into a float32 matrix (the residual stream).
 //
+// Rotary epilogue for a stacked q|k|v projection whose q and k rows were reordered so that the two
+// dims of a rotating pair are neighbours (pair j of a head at 2j, 2j+1): bias, rotation at the
+// token's position (src/libllm/llama.cc:151-176 pairs j with j + rot_dim/2; the reordering only
+// moves them side by side), rotated q to the output, rotated k and v to the token's place in the
+// paged cache (keys [page, kv_head, position, dim], values [page, kv_head, dim, position]).
+//
 // Fused RMS norm (up to 16 rows): X is then the float32 residual stream.  Staging multiplies each
 // element by the norm's weight and rounds to bfloat16, and sums the squares of the row on the way
 // (every block stages whole rows); the factor 1/sqrt(mean(x^2) + eps) of a row is applied to its
@@ -27,6 +33,7 @@
 #define SK_EPI_NONE 0
 #define SK_EPI_SWIGLU 1
 #define SK_EPI_ACCUM 2
+#define SK_EPI_ROPE 3
 
 // MT: 16-row tiles of X; RT: 16-row tiles of W per wave; WN: row groups per block; G: granules of
 // 2 steps that a wave takes per chunk (a chunk is 512*G elements of K).
@@ -37,12 +44,26 @@ struct SkinnyNorm {
   float eps;
 };
 
+struct SkinnyRope {
+  const float* bias;       // [N] or null
+  const float* cos_t;      // [positions, rot_dim / 2]
+  const float* sin_t;
+  const int* tok_pos;      // [M] position of each row's token
+  const int* tok_seq;      // [M] its sequence in the step
+  const int* seq_slot;     // [sequences] slot of each sequence
+  const int* table;        // [slots, table_stride] page of (slot, position / 64)
+  bf16_t* k_pages;
+  bf16_t* v_pages;
+  int table_stride, n_heads, n_kv, hd, rot_dim, write_kv;
+};
+
 template <int MT, int RT, int WN, int G, int EPI, bool XNORM, typename OutT>
 __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ X,
                                                                       SkinnyNorm norm,
                                                                       const bf16_t* __restrict__ W,
                                                                       OutT* __restrict__ C, int M,
-                                                                      int N, int K, int n_out) {
+                                                                      int N, int K, int n_out,
+                                                                      SkinnyRope rope) {
   static_assert(!XNORM || (MT == 1 && WN == 1), "the fused norm is built for up to 16 rows");
   constexpr int NT = WN * SK_WK * 64;
   constexpr int CK = 512 * G;                    // elements of K per chunk
@@ -256,6 +277,51 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
       n = ((blockIdx.x * WN + w_n) * RT + ort) * 16 + 4 * (ln >> 4);
     }
     const int m = mt * 16 + (ln & 15);
+    if (EPI == SK_EPI_ROPE) {
+      if (m >= M || n >= N) continue;                 // N, hd are multiples of 16: four outputs, one head
+      if (rope.bias) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += rope.bias[n + e];
+      }
+      const int q_dim = rope.n_heads * rope.hd, kv_dim = rope.n_kv * rope.hd;
+      const int pos = rope.tok_pos[m];
+      const int d = n % rope.hd;
+      if (n < q_dim + kv_dim) {                       // q and k rotate
+        const float* cr = rope.cos_t + (size_t)pos * (rope.rot_dim / 2);
+        const float* sr = rope.sin_t + (size_t)pos * (rope.rot_dim / 2);
+#pragma unroll
+        for (int e = 0; e < 4; e += 2) {
+          if (d + e < rope.rot_dim) {
+            const float c = cr[(d + e) >> 1], sn = sr[(d + e) >> 1];
+            const float x1 = v[e], x2 = v[e + 1];
+            v[e] = x1 * c - x2 * sn;
+            v[e + 1] = x2 * c + x1 * sn;
+          }
+        }
+      }
+      uint2 pk;
+      pk.x = pack2_bf16(v[0], v[1]);
+      pk.y = pack2_bf16(v[2], v[3]);
+      if (n < q_dim) {
+        *reinterpret_cast<uint2*>(C + (size_t)m * q_dim + n) = pk;
+      } else if (rope.write_kv) {
+        const int slot = rope.seq_slot[rope.tok_seq[m]];
+        const int page = rope.table[(size_t)slot * rope.table_stride + pos / 64];
+        const int kn = n - q_dim;
+        if (kn < kv_dim) {
+          const int kvh = kn / rope.hd;
+          *reinterpret_cast<uint2*>(rope.k_pages + (((size_t)page * rope.n_kv + kvh) * 64 + pos % 64) * rope.hd + d) = pk;
+        } else {
+          const int kvh = (kn - kv_dim) / rope.hd;
+          bf16_t* vp = rope.v_pages + (((size_t)page * rope.n_kv + kvh) * rope.hd + d) * 64 + pos % 64;
+          vp[0] = (bf16_t)(pk.x & 0xffffu);
+          vp[64] = (bf16_t)(pk.x >> 16);
+          vp[128] = (bf16_t)(pk.y & 0xffffu);
+          vp[192] = (bf16_t)(pk.y >> 16);
+        }
+      }
+      continue;
+    }
     if (m >= M || n >= ldc) continue;
     OutT* dst = C + (size_t)m * ldc + n;
     if (EPI == SK_EPI_ACCUM) {
@@ -287,6 +353,7 @@ struct SkinnyArgs {
   void* C;
   int M, N, K, n_out;
   hipStream_t stream;
+  SkinnyRope rope;
 };
 
 template <int MT, int RT, int WN, int G, int EPI, bool XNORM, typename OutT>
@@ -296,7 +363,7 @@ static int launch_skinny(const SkinnyArgs& a) {
   constexpr int OUT_RT = (EPI == SK_EPI_SWIGLU) ? RT / 2 : RT;
   const int blocks = (tiles + OUT_RT * WN - 1) / (OUT_RT * WN);
   gemm_skinny_kernel<MT, RT, WN, G, EPI, XNORM, OutT><<<blocks, WN * SK_WK * 64, 0, a.stream>>>(
-      a.X, a.norm, a.W, (OutT*)a.C, a.M, a.N, a.K, a.n_out);
+      a.X, a.norm, a.W, (OutT*)a.C, a.M, a.N, a.K, a.n_out, a.rope);
   return llm_launch_status();
 }
 
@@ -346,6 +413,7 @@ extern "C" int llm_gemm_skinny_bf16(const void* X, const float* norm_x, const fl
   a.K = K;
   a.n_out = N;
   a.stream = stream;
+  a.rope = SkinnyRope{};
   if (epilogue == SK_EPI_NONE) {
     if (out_dtype == LLM_DTYPE_BF16) return pick_shape<SK_EPI_NONE, bf16_t>(a);
     if (out_dtype == LLM_DTYPE_F32) return pick_shape<SK_EPI_NONE, float>(a);
@@ -358,4 +426,58 @@ extern "C" int llm_gemm_skinny_bf16(const void* X, const float* norm_x, const fl
     return pick_shape<SK_EPI_ACCUM, float>(a);
   }
   return LLM_ERR_ARG;
+}
+
+// The stacked q|k|v projection with the rotary epilogue (see the head of this file): rotated q as
+// bfloat16 [M, n_heads * hd] to `q_out`, k and v to the cache if write_kv.  N is
+// (n_heads + 2 n_kv) * hd with write_kv, else n_heads * hd; hd a multiple of 16, rot_dim even.
+extern "C" int llm_gemm_skinny_rope_bf16(const void* X, const float* norm_x, const float* norm_weight,
+                                         float norm_eps, const int* norm_rows, const void* W,
+                                         const float* bias, void* q_out, int M, int K, int n_heads,
+                                         int n_kv, int hd, const float* cos_t, const float* sin_t,
+                                         int rot_dim, const int* tok_pos, const int* tok_seq,
+                                         const int* seq_slot, const int* table, int table_stride,
+                                         void* k_pages, void* v_pages, int page_size, int write_kv,
+                                         hipStream_t stream) {
+  if (M <= 0) return LLM_OK;
+  if (M > 64 || K <= 0 || (K & 7) || n_heads <= 0 || n_kv < 0 || hd <= 0 || (hd & 15) || rot_dim < 0 ||
+      rot_dim > hd || (rot_dim & 1) || page_size != 64)
+    return LLM_ERR_ARG;
+  const void* x = norm_x ? (const void*)norm_x : X;
+  if (x == nullptr || W == nullptr || q_out == nullptr || tok_pos == nullptr) return LLM_ERR_ARG;
+  if ((((uintptr_t)x) | ((uintptr_t)W) | ((uintptr_t)q_out)) & 15) return LLM_ERR_ARG;
+  if (norm_x && (norm_weight == nullptr || (((uintptr_t)norm_weight) & 15) || M > 16)) return LLM_ERR_ARG;
+  if (rot_dim > 0 && (cos_t == nullptr || sin_t == nullptr)) return LLM_ERR_ARG;
+  if (write_kv && (!k_pages || !v_pages || !table || !seq_slot || !tok_seq || n_kv <= 0 ||
+                   ((((uintptr_t)k_pages) | ((uintptr_t)v_pages)) & 7)))
+    return LLM_ERR_ARG;
+  SkinnyArgs a;
+  a.X = (const bf16_t*)X;
+  a.norm.x = norm_x;
+  a.norm.weight = norm_weight;
+  a.norm.rows = norm_rows;
+  a.norm.eps = norm_eps;
+  a.W = (const bf16_t*)W;
+  a.C = q_out;
+  a.M = M;
+  a.N = (n_heads + (write_kv ? 2 * n_kv : 0)) * hd;
+  a.K = K;
+  a.n_out = a.N;
+  a.stream = stream;
+  a.rope.bias = bias;
+  a.rope.cos_t = cos_t;
+  a.rope.sin_t = sin_t;
+  a.rope.tok_pos = tok_pos;
+  a.rope.tok_seq = tok_seq;
+  a.rope.seq_slot = seq_slot;
+  a.rope.table = table;
+  a.rope.k_pages = (bf16_t*)k_pages;
+  a.rope.v_pages = (bf16_t*)v_pages;
+  a.rope.table_stride = table_stride;
+  a.rope.n_heads = n_heads;
+  a.rope.n_kv = n_kv;
+  a.rope.hd = hd;
+  a.rope.rot_dim = rot_dim;
+  a.rope.write_kv = write_kv;
+  return pick_shape<SK_EPI_ROPE, bf16_t>(a);
 }

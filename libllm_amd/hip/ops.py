@@ -34,7 +34,9 @@ _SIGNATURES = {
     "llm_silu_mul": [_vp, _vp, _i, _i, _i, _vp],
     "llm_add_bias": [_vp, _i, _vp, _i, _i, _vp],
     "llm_rope_kv_write": [_vp, _i, _i, _vp, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp,
-                          _vp, _i, _i, _i, _vp],
+                          _vp, _i, _i, _i, _i, _vp],
+    "llm_gemm_skinny_rope_bf16": [_vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i,
+                                  _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _vp],
     "llm_gemm_f32": [_vp, _vp, _vp, _i, _i, _i, _vp],
     "llm_attention_ref": [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
                           _f, _i, _vp],
@@ -268,7 +270,67 @@ class HipOps:
                                           m, two_i // 2, self._stream()), "silu_mul")
         return out
 
-    def rope_kv_write(self, qkv, bias, n_heads, n_kv, hd, cos, sin, rot_dim, ctx, kv, write):
+    # rotating pairs side by side (2j, 2j+1) let the projection's epilogue rotate them: a mixer
+    # that reorders its projection's rows accordingly may pass adjacent=True
+    prefers_adjacent_pairs = True
+
+    def qkv_rope(self, x, w, bias, n_heads, n_kv, hd, cos, sin, rot_dim, ctx, kv, write, adjacent,
+                 dtype):
+        """The stacked q|k|v projection (q alone if not ``write``), bias, rotation of q and k at
+        the tokens' positions, and k and v into the cache.  Returns rows whose first
+        ``n_heads * hd`` columns are the rotated queries.  For few rows in bfloat16 with pairs
+        side by side this is one kernel; otherwise the product and the rotation kernel."""
+        lazy = isinstance(x, NormedRows)
+        m, k = (x.n_rows, x.res.shape[1]) if lazy else x.shape
+        n = (n_heads + (2 * n_kv if write else 0)) * hd
+        if tuple(w.shape) != (n, k):
+            raise KernelError("qkv_rope: the weight is %s, expected %s" % (tuple(w.shape), (n, k)))
+        fused = (dtype == torch.bfloat16 and (adjacent or rot_dim == 0) and hd % 16 == 0
+                 and m <= self.SKINNY_ROWS and m == ctx.n_tokens
+                 and (not write or (kv is not None and kv.k_pages.dtype == torch.bfloat16)))
+        if fused and lazy and not (m <= self.NORM_ROWS and n <= self.NORM_COLS):
+            x, lazy = self._materialise(x, dtype), False
+        if fused and self._skinny_ok(x, w, m, k):
+            self._dev(w, "qkv weight")
+            cptr = sptr = None
+            if rot_dim:
+                if cos is None or cos.shape[1] != rot_dim // 2 or cos.shape != sin.shape:
+                    raise KernelError("qkv_rope: rotary tables do not match rot_dim %d" % rot_dim)
+                if not ctx.captured and ctx.max_ctx > cos.shape[0]:
+                    raise KernelError("qkv_rope: position %d exceeds the rotary table of %d rows"
+                                      % (ctx.max_ctx - 1, cos.shape[0]))
+                cptr, sptr = self._dev(cos, "cos", torch.float32), self._dev(sin, "sin", torch.float32)
+            bptr = None
+            if bias is not None:
+                bptr = self._dev(bias, "qkv bias", torch.float32)
+                if bias.shape[0] < n:
+                    raise KernelError("qkv_rope: the bias is shorter than a row")
+            kptr = vptr = tptr = None
+            stride = 0
+            if write:
+                self._check_kv(kv, n_kv, hd, torch.bfloat16)
+                kptr, vptr, tptr = kv.k_pages.data_ptr(), kv.v_pages.data_ptr(), kv.block_table.data_ptr()
+                stride = kv.block_table.shape[1]
+            if lazy:
+                self._dev(x.res, "residual stream", torch.float32)
+                self._dev(x.weight, "norm weight", torch.float32, (k,))
+                xp, nx, nw, eps = None, x.res.data_ptr(), x.weight.data_ptr(), x.eps
+                rows = None if x.rows is None else x.rows.data_ptr()
+            else:
+                xp, nx, nw, eps, rows = self._dev(x, "qkv input", torch.bfloat16), None, None, 0.0, None
+            q = torch.empty((m, n_heads * hd), dtype=torch.bfloat16, device=self.device)
+            self._check(self.lib.llm_gemm_skinny_rope_bf16(
+                xp, nx, nw, eps, rows, w.data_ptr(), bptr, q.data_ptr(), m, k, n_heads, n_kv, hd,
+                cptr, sptr, rot_dim, ctx.tok_pos.data_ptr(), ctx.tok_seq.data_ptr(),
+                ctx.seq_slot.data_ptr(), tptr, stride, kptr, vptr, 64, 1 if write else 0,
+                self._stream()), "gemm_skinny_rope_bf16")
+            return q
+        qkv = self.linear(x, w, None, dtype)
+        self.rope_kv_write(qkv, bias, n_heads, n_kv, hd, cos, sin, rot_dim, ctx, kv, write, adjacent)
+        return qkv
+
+    def rope_kv_write(self, qkv, bias, n_heads, n_kv, hd, cos, sin, rot_dim, ctx, kv, write,
+                      adjacent=False):
         m, width = qkv.shape
         need = (n_heads + (2 * n_kv if write else 0)) * hd
         if width != need:
@@ -298,7 +360,7 @@ class HipOps:
         self._check(self.lib.llm_rope_kv_write(
             qkv.data_ptr(), _code(qkv.dtype), width, bptr, n_heads, n_kv, hd, cptr, sptr, rot_dim,
             ctx.tok_pos.data_ptr(), ctx.tok_seq.data_ptr(), ctx.seq_slot.data_ptr(), tptr, stride,
-            kptr, vptr, 64, 1 if write else 0, m, self._stream()), "rope_kv_write")
+            kptr, vptr, 64, 1 if write else 0, 1 if adjacent else 0, m, self._stream()), "rope_kv_write")
 
     def _check_kv(self, kv, n_kv, hd, dtype):
         if kv is None:

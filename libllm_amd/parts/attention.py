@@ -60,6 +60,7 @@ class Attention(Mixer):
         self.out = Linear(self.q_dim, spec.width)
         self.cos = self.sin = None
         self.bias = None
+        self.adjacent = False
 
     def cache_need(self):
         s = self.spec
@@ -88,18 +89,45 @@ class Attention(Mixer):
         if s.qkv_bias:
             bias = torch.cat([tensors[n + ".bias"] for n in (s.q_name, s.k_name, s.v_name)]).contiguous()
         w = torch.cat(parts, dim=0)                      # q rows, then k, then v
+        # kernels that rotate inside the projection want the two dims of a pair side by side:
+        # reorder the output rows of q and k (and the bias) once; scores do not change, since
+        # queries and keys are reordered alike
+        self.adjacent = bool(getattr(ops, "prefers_adjacent_pairs", False)) and self.position.rot_dim > 0
+        if self.adjacent:
+            order = self._pair_order(w.device)
+            w = w[order]
+            if bias is not None:
+                bias = bias[order].contiguous()
         self.qkv.bind(w)
         self.q_only.bind(w[:self.q_dim])
         self.bias = bias                                 # added inside the rotation kernel
         self.out.bind(tensors[s.o_name + ".weight"])
         self.cos, self.sin = self.position.tables(w.device)
 
+    def _pair_order(self, device):
+        """Row order of the stacked projection with rotating pairs side by side: in every q and
+        k head dims (j, j + rot_dim/2) move to (2j, 2j+1); other dims and v stay."""
+        s, rot = self.spec, self.position.rot_dim
+        head = torch.arange(s.head_dim)
+        head[0:rot:2] = torch.arange(rot // 2)
+        head[1:rot:2] = torch.arange(rot // 2) + rot // 2
+        n_rot = s.n_heads + s.n_kv_heads
+        qk = (torch.arange(n_rot)[:, None] * s.head_dim + head[None, :]).reshape(-1)
+        v = torch.arange(n_rot * s.head_dim, (n_rot + s.n_kv_heads) * s.head_dim)
+        return torch.cat([qk, v]).to(device)
+
     def forward(self, ctx: StepContext, x, entry, residual=None):
         s = self.spec
         kv = ctx.kv(entry.cache)
-        qkv = self.qkv(ctx, x) if entry.writes else self.q_only(ctx, x)
-        ctx.ops.rope_kv_write(qkv, self.bias, s.n_heads, s.n_kv_heads, s.head_dim, self.cos, self.sin,
-                              self.position.rot_dim, ctx, kv, entry.writes)
+        proj = self.qkv if entry.writes else self.q_only
+        if hasattr(ctx.ops, "qkv_rope"):
+            qkv = ctx.ops.qkv_rope(x, proj.weight, self.bias, s.n_heads, s.n_kv_heads, s.head_dim,
+                                   self.cos, self.sin, self.position.rot_dim, ctx, kv, entry.writes,
+                                   self.adjacent, ctx.dtype)
+        else:
+            qkv = proj(ctx, x)
+            ctx.ops.rope_kv_write(qkv, self.bias, s.n_heads, s.n_kv_heads, s.head_dim, self.cos,
+                                  self.sin, self.position.rot_dim, ctx, kv, entry.writes)
         o = ctx.ops.attention(qkv, s.n_heads, s.n_kv_heads, s.head_dim, ctx, kv,
                               self.scale, s.window)
         return self.out(ctx, o, residual=residual)

@@ -284,6 +284,90 @@ def test_rope_kv_write(ops, dtype, shape, bias):
         o += n
 
 
+def pair_order(n_heads, n_kv, hd, rot):
+    """Rows of a stacked q|k|v projection with the dims of a rotating pair side by side."""
+    head = torch.arange(hd)
+    head[0:rot:2] = torch.arange(rot // 2)
+    head[1:rot:2] = torch.arange(rot // 2) + rot // 2
+    qk = (torch.arange(n_heads + n_kv)[:, None] * hd + head[None, :]).reshape(-1)
+    return torch.cat([qk, torch.arange((n_heads + n_kv) * hd, (n_heads + 2 * n_kv) * hd)])
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("shape", [(4, 2, 16, 16), (6, 3, 48, 24), (32, 8, 64, 64), (3, 1, 32, 0)])
+@pytest.mark.parametrize("bias", [False, True])
+@pytest.mark.parametrize("seqs", [[(2, 0, 5), (0, 61, 9), (1, 130, 1)], [(1, 63, 1), (0, 0, 1), (2, 200, 1)]])
+def test_projection_with_rotation_and_cache_write(ops, dtype, shape, bias, seqs):
+    """The q|k|v projection, rotation and cache write in one call (one kernel for few rows in
+    bfloat16, with and without a fused norm) against the plain formulas on the rows in their
+    natural order; the two pairings hold the same numbers in different places."""
+    n_heads, n_kv, hd, rot = shape
+    k_in = 72
+    ctx = make_ctx(ops, dtype, seqs)
+    m = ctx.n_tokens
+    n = (n_heads + 2 * n_kv) * hd
+    x = rnd((m, k_in), torch.bfloat16, 40)
+    w = rnd((n, k_in), torch.bfloat16, 41, 0.2)
+    b = rnd((n,), torch.float32, 42) if bias else None
+    order = pair_order(n_heads, n_kv, hd, rot) if rot else torch.arange(n)
+    half = rot // 2
+    inv = 1.0 / (10000.0 ** (torch.arange(0, rot, 2, dtype=torch.float64) / max(rot, 1)))
+    ang = torch.arange(300, dtype=torch.float64)[:, None] * inv[None, :]
+    cos, sin = (torch.cos(ang).float().cuda(), torch.sin(ang).float().cuda()) if rot else (None, None)
+    # the plain result, natural order
+    y = x.double() @ w.double().t() + (b.double() if bias else 0)
+    pos = ctx.tok_pos.cpu().long()
+    heads = y[:, :(n_heads + n_kv) * hd].reshape(m, n_heads + n_kv, hd).clone()
+    if rot:
+        c, s_ = torch.cos(ang)[pos][:, None, :], torch.sin(ang)[pos][:, None, :]
+        x1, x2 = heads[..., :half].clone(), heads[..., half:rot].clone()
+        heads[..., :half] = x1 * c - x2 * s_
+        heads[..., half:rot] = x2 * c + x1 * s_
+    v_ref = y[:, (n_heads + n_kv) * hd:].reshape(m, n_kv, hd)
+    head_order = order[:hd]                                    # where each dim of a head went
+    wd = w.cuda().to(dtype)[order.cuda()].contiguous()
+    bd = b.cuda()[order.cuda()].contiguous() if bias else None
+    tol = dict(f32=2e-5, bf16=2 * BF16_2ULP)
+    for lazy in (False, True):
+        kv = make_kv("cuda", dtype, 3, 4, n_kv, hd, seed=1)
+        if lazy:                                               # the input as rows still to be normalised
+            stream = (x.float() * 3.0).cuda()
+            stream[0] *= 50.0
+            wn = (1.0 + 0.3 * rnd((k_in,), torch.float32, 43)).cuda()
+            xin = ops.normed(stream, wn, 1e-5)
+            sd = stream.double().cpu()
+            hn = sd * wn.double().cpu() / torch.sqrt((sd * sd).mean(-1, keepdim=True) + 1e-5)
+            scale = None
+        else:
+            xin = x.cuda().to(dtype)
+        if lazy:
+            y2 = hn @ w.double().t() + (b.double() if bias else 0)
+            heads2 = y2[:, :(n_heads + n_kv) * hd].reshape(m, n_heads + n_kv, hd).clone()
+            if rot:
+                x1, x2 = heads2[..., :half].clone(), heads2[..., half:rot].clone()
+                heads2[..., :half] = x1 * c - x2 * s_
+                heads2[..., half:rot] = x2 * c + x1 * s_
+            want_heads, want_v = heads2, y2[:, (n_heads + n_kv) * hd:].reshape(m, n_kv, hd)
+        else:
+            want_heads, want_v = heads, v_ref
+        out = ops.qkv_rope(xin, wd, bd, n_heads, n_kv, hd, cos, sin, rot, ctx, kv, True, bool(rot), dtype)
+        q = out[:, :n_heads * hd].reshape(m, n_heads, hd)
+        assert close(q, want_heads[:, :n_heads][..., head_order], dtype, **tol)
+        o = 0
+        for slot, p0, n_new in seqs:
+            k_got, v_got = read_kv(kv, slot, p0 + n_new)
+            assert close(k_got[p0:], want_heads[o:o + n_new, n_heads:][..., head_order], dtype, **tol)
+            assert close(v_got[p0:], want_v[o:o + n_new], dtype, **tol)
+            assert torch.count_nonzero(k_got[:p0]) == 0 and torch.count_nonzero(v_got[:p0]) == 0
+            o += n_new
+    # queries alone, for a layer that reads another layer's keys
+    kv = make_kv("cuda", dtype, 3, 4, n_kv, hd, seed=1)
+    q_only = ops.qkv_rope(x.cuda().to(dtype), wd[:n_heads * hd].contiguous(), bd, n_heads, n_kv, hd, cos, sin,
+                          rot, ctx, kv, False, bool(rot), dtype)
+    assert close(q_only[:, :n_heads * hd].reshape(m, n_heads, hd), heads[:, :n_heads][..., head_order], dtype, **tol)
+    assert torch.count_nonzero(kv.k_pages) == 0
+
+
 def test_rope_pairing_and_sign(ops):
     # a unit vector in dimension 0 at position p becomes cos at 0 and +sin at hd/2:
     # o[j] = x[j] c - x[j+hd/2] s, o[j+hd/2] = x[j+hd/2] c + x[j] s   (src/libllm/llama.cc:151-176)
