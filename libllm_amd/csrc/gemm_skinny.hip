@@ -62,8 +62,8 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
                                                                       SkinnyNorm norm,
                                                                       const bf16_t* __restrict__ W,
                                                                       OutT* __restrict__ C, int M,
-                                                                      int N, int K, int n_out,
-                                                                      SkinnyRope rope) {
+                                                                      int N, int K, int ldw,
+                                                                      int n_out, SkinnyRope rope) {
   static_assert(!XNORM || (MT == 1 && WN == 1), "the fused norm is built for up to 16 rows");
   constexpr int NT = WN * SK_WK * 64;
   constexpr int CK = 512 * G;                    // elements of K per chunk
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   for (int rt = 0; rt < RT; ++rt) {
     int n = tile_row[rt] + r;
     if (n > N - 1) n = N - 1;                   // rows past the end read the last row; not stored
-    wp[rt] = W + (size_t)n * K + g * 8;
+    wp[rt] = W + (size_t)n * ldw + g * 8;
   }
 
   f32x4 acc[RT][MT];
@@ -351,7 +351,7 @@ struct SkinnyArgs {
   SkinnyNorm norm;
   const bf16_t* W;
   void* C;
-  int M, N, K, n_out;
+  int M, N, K, ldw, n_out;     // ldw: elements between rows of W (a multiple of 8, at least K)
   hipStream_t stream;
   SkinnyRope rope;
 };
@@ -363,7 +363,7 @@ static int launch_skinny(const SkinnyArgs& a) {
   constexpr int OUT_RT = (EPI == SK_EPI_SWIGLU) ? RT / 2 : RT;
   const int blocks = (tiles + OUT_RT * WN - 1) / (OUT_RT * WN);
   gemm_skinny_kernel<MT, RT, WN, G, EPI, XNORM, OutT><<<blocks, WN * SK_WK * 64, 0, a.stream>>>(
-      a.X, a.norm, a.W, (OutT*)a.C, a.M, a.N, a.K, a.n_out, a.rope);
+      a.X, a.norm, a.W, (OutT*)a.C, a.M, a.N, a.K, a.ldw, a.n_out, a.rope);
   return llm_launch_status();
 }
 
@@ -377,7 +377,10 @@ static int pick_shape(const SkinnyArgs& a) {
     return LLM_ERR_ARG;
   }
   switch (mt) {
-    case 1: return launch_skinny<1, RT, 1, 2, EPI, false, OutT>(a);
+    case 1:
+      // a long K with few rows of W: more of each row in flight per wave
+      if (RT == 1 && a.K >= 4096 && a.N <= 4096) return launch_skinny<1, RT, 1, 4, EPI, false, OutT>(a);
+      return launch_skinny<1, RT, 1, 2, EPI, false, OutT>(a);
     case 2: return launch_skinny<2, RT, 2 / RT, 1, EPI, false, OutT>(a);
     case 3: return launch_skinny<3, RT, 2 / RT, 1, EPI, false, OutT>(a);
     case 4: return launch_skinny<4, RT, 2 / RT, 1, EPI, false, OutT>(a);
@@ -385,16 +388,17 @@ static int pick_shape(const SkinnyArgs& a) {
   return LLM_ERR_ARG;
 }
 
+// Rows of W lie ldw elements apart (ldw >= K, a multiple of 8).
 // C[M, N] (epilogue 0: stored as out_dtype; 2: added into the float32 C) or C[M, N/2] (epilogue 1,
 // SwiGLU over W = [Wg; Wu], N/2 a multiple of 16) from X[M, K] and W[N, K].  X is bfloat16, or,
 // with norm_x given (M <= 16), the rows `norm_rows` of the float32 matrix norm_x, RMS-normalised
 // with norm_weight and norm_eps on the way.
 extern "C" int llm_gemm_skinny_bf16(const void* X, const float* norm_x, const float* norm_weight,
                                     float norm_eps, const int* norm_rows, const void* W, void* C,
-                                    int epilogue, int out_dtype, int M, int N, int K,
+                                    int epilogue, int out_dtype, int M, int N, int K, int ldw,
                                     hipStream_t stream) {
   if (M <= 0 || N <= 0) return LLM_OK;
-  if (M > 64 || K <= 0 || (K & 7)) return LLM_ERR_ARG;
+  if (M > 64 || K <= 0 || (K & 7) || ldw < K || (ldw & 7)) return LLM_ERR_ARG;
   const void* x = norm_x ? (const void*)norm_x : X;
   if (x == nullptr || W == nullptr || C == nullptr) return LLM_ERR_ARG;
   if ((((uintptr_t)x) | ((uintptr_t)W) | ((uintptr_t)C)) & 15) return LLM_ERR_ARG;
@@ -411,6 +415,7 @@ extern "C" int llm_gemm_skinny_bf16(const void* X, const float* norm_x, const fl
   a.M = M;
   a.N = N;
   a.K = K;
+  a.ldw = ldw;
   a.n_out = N;
   a.stream = stream;
   a.rope = SkinnyRope{};
@@ -433,14 +438,14 @@ extern "C" int llm_gemm_skinny_bf16(const void* X, const float* norm_x, const fl
 // (n_heads + 2 n_kv) * hd with write_kv, else n_heads * hd; hd a multiple of 16, rot_dim even.
 extern "C" int llm_gemm_skinny_rope_bf16(const void* X, const float* norm_x, const float* norm_weight,
                                          float norm_eps, const int* norm_rows, const void* W,
-                                         const float* bias, void* q_out, int M, int K, int n_heads,
+                                         const float* bias, void* q_out, int M, int K, int ldw, int n_heads,
                                          int n_kv, int hd, const float* cos_t, const float* sin_t,
                                          int rot_dim, const int* tok_pos, const int* tok_seq,
                                          const int* seq_slot, const int* table, int table_stride,
                                          void* k_pages, void* v_pages, int page_size, int write_kv,
                                          hipStream_t stream) {
   if (M <= 0) return LLM_OK;
-  if (M > 64 || K <= 0 || (K & 7) || n_heads <= 0 || n_kv < 0 || hd <= 0 || (hd & 15) || rot_dim < 0 ||
+  if (M > 64 || K <= 0 || (K & 7) || ldw < K || (ldw & 7) || n_heads <= 0 || n_kv < 0 || hd <= 0 || (hd & 15) || rot_dim < 0 ||
       rot_dim > hd || (rot_dim & 1) || page_size != 64)
     return LLM_ERR_ARG;
   const void* x = norm_x ? (const void*)norm_x : X;
@@ -462,6 +467,7 @@ extern "C" int llm_gemm_skinny_rope_bf16(const void* X, const float* norm_x, con
   a.M = M;
   a.N = (n_heads + (write_kv ? 2 * n_kv : 0)) * hd;
   a.K = K;
+  a.ldw = ldw;
   a.n_out = a.N;
   a.stream = stream;
   a.rope.bias = bias;

@@ -35,12 +35,12 @@ _SIGNATURES = {
     "llm_add_bias": [_vp, _i, _vp, _i, _i, _vp],
     "llm_rope_kv_write": [_vp, _i, _i, _vp, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp,
                           _vp, _i, _i, _i, _i, _vp],
-    "llm_gemm_skinny_rope_bf16": [_vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _i,
+    "llm_gemm_skinny_rope_bf16": [_vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _i,
                                   _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _vp],
     "llm_gemm_f32": [_vp, _vp, _vp, _i, _i, _i, _vp],
     "llm_attention_ref": [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
                           _f, _i, _vp],
-    "llm_gemm_skinny_bf16": [_vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp],
+    "llm_gemm_skinny_bf16": [_vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "llm_attention_mfma_supported": [_i],
     "llm_attention_prefill_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i,
                                    _i, _i, _f, _i, _vp],
@@ -92,6 +92,15 @@ class HipOps:
         if status != 0:
             raise KernelError("%s: %s" % (what, {1: "the kernel refuses these operands",
                                                  2: "the launch failed"}.get(status, "error %d" % status)))
+
+    def _weight(self, w: torch.Tensor, what: str):
+        """A weight matrix: on the device, rows contiguous; rows may lie further apart than
+        their length (a view of some columns of a wider matrix)."""
+        if w.device != self.device:
+            raise KernelError("%s lies on %s, not on %s" % (what, w.device, self.device))
+        if w.dim() != 2 or w.stride(1) != 1 or w.stride(0) < w.shape[1]:
+            raise KernelError("%s must be a matrix with contiguous rows" % what)
+        return w.data_ptr()
 
     def _dev(self, t: torch.Tensor, what: str, dtype=None, shape=None):
         if t.device != self.device:
@@ -165,7 +174,8 @@ class HipOps:
         return x
 
     def _skinny_ok(self, x, w, m, k):
-        if not (self.fast_gemm and w.dtype == torch.bfloat16 and k % 8 == 0 and w.data_ptr() % 16 == 0):
+        if not (self.fast_gemm and w.dtype == torch.bfloat16 and k % 8 == 0 and w.data_ptr() % 16 == 0
+                and w.stride(0) % 8 == 0):
             return False
         if isinstance(x, NormedRows):
             # every block normalises the rows itself: worth it only while the blocks are few
@@ -185,7 +195,7 @@ class HipOps:
         width = n // 2 if epilogue == self._EPI_SWIGLU else n
         self._check(self.lib.llm_gemm_skinny_bf16(
             xp, nx, nw, eps, rows, w.data_ptr(), out.data_ptr() + m0 * width * out.element_size(),
-            epilogue, _code(out.dtype), mm, n, k, self._stream()), "gemm_skinny_bf16")
+            epilogue, _code(out.dtype), mm, n, k, w.stride(0), self._stream()), "gemm_skinny_bf16")
 
     def linear(self, x, w, bias, out_dtype, residual=None):
         """x W^T (+ bias) as ``out_dtype``.  ``x`` is a matrix or a ``normed`` record.  With
@@ -197,7 +207,7 @@ class HipOps:
         n, k2 = w.shape
         if k != k2:
             raise KernelError("linear: x is [%d, %d] but the weight is [%d, %d]" % (m, k, n, k2))
-        self._dev(w, "linear weight")
+        self._weight(w, "linear weight")
         if lazy:
             self._dev(x.res, "residual stream", torch.float32)
             self._dev(x.weight, "norm weight", torch.float32, (k,))
@@ -221,6 +231,8 @@ class HipOps:
             if self._skinny_ok(x, w, m, k) and bias is None:
                 return self.linear(x, w, None, out_dtype, residual)
         if w.dtype == torch.float32:
+            if w.stride(0) != k:
+                raise KernelError("linear: a float32 weight must be contiguous")
             xf = x if x.dtype == torch.float32 else x.float()
             out = torch.empty((m, n), dtype=torch.float32, device=self.device)
             self._check(self.lib.llm_gemm_f32(xf.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k,
@@ -250,7 +262,7 @@ class HipOps:
             raise KernelError("linear_swiglu: x is [%d, %d] but the weight is %s" % (m, k, tuple(w.shape)))
         if (self._skinny_ok(x, w, m, k) and m <= self.SKINNY_ROWS and inter % 16 == 0
                 and dtype == torch.bfloat16):
-            self._dev(w, "linear weight")
+            self._weight(w, "linear weight")
             out = torch.empty((m, inter), dtype=torch.bfloat16, device=self.device)
             self._skinny(x, w, out, self._EPI_SWIGLU, 0, m)
             return out
@@ -291,7 +303,7 @@ class HipOps:
         if fused and lazy and not (m <= self.NORM_ROWS and n <= self.NORM_COLS):
             x, lazy = self._materialise(x, dtype), False
         if fused and self._skinny_ok(x, w, m, k):
-            self._dev(w, "qkv weight")
+            self._weight(w, "qkv weight")
             cptr = sptr = None
             if rot_dim:
                 if cos is None or cos.shape[1] != rot_dim // 2 or cos.shape != sin.shape:
@@ -320,7 +332,7 @@ class HipOps:
                 xp, nx, nw, eps, rows = self._dev(x, "qkv input", torch.bfloat16), None, None, 0.0, None
             q = torch.empty((m, n_heads * hd), dtype=torch.bfloat16, device=self.device)
             self._check(self.lib.llm_gemm_skinny_rope_bf16(
-                xp, nx, nw, eps, rows, w.data_ptr(), bptr, q.data_ptr(), m, k, n_heads, n_kv, hd,
+                xp, nx, nw, eps, rows, w.data_ptr(), bptr, q.data_ptr(), m, k, w.stride(0), n_heads, n_kv, hd,
                 cptr, sptr, rot_dim, ctx.tok_pos.data_ptr(), ctx.tok_seq.data_ptr(),
                 ctx.seq_slot.data_ptr(), tptr, stride, kptr, vptr, 64, 1 if write else 0,
                 self._stream()), "gemm_skinny_rope_bf16")

@@ -99,7 +99,7 @@ class Attention(Mixer):
             if bias is not None:
                 bias = bias[order].contiguous()
         self.qkv.bind(w)
-        self.q_only.bind(w[:self.q_dim])
+        self.q_only.bind(self.qkv.weight[:self.q_dim])    # the same storage, the q rows alone
         self.bias = bias                                 # added inside the rotation kernel
         self.out.bind(tensors[s.o_name + ".weight"])
         self.cos, self.sin = self.position.tables(w.device)

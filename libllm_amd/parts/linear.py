@@ -13,7 +13,7 @@ class Linear:
 
     def bind(self, weight: torch.Tensor, bias: Optional[torch.Tensor] = None):
         assert tuple(weight.shape) == (self.out_features, self.in_features)
-        self.weight = weight.contiguous()
+        self.weight = weight if weight.stride(-1) == 1 else weight.contiguous()
         self.bias = bias
 
     def __call__(self, ctx, x, out_dtype=None, residual=None):

@@ -168,8 +168,31 @@ def test_gemm_skinny_refuses(ops):
     assert close(out, x.double() @ w.double().t(), torch.bfloat16)
     c = torch.empty((2, 16), dtype=torch.bfloat16, device="cuda")
     st = ops.lib.llm_gemm_skinny_bf16(x.data_ptr(), None, None, 0.0, None, w.data_ptr(), c.data_ptr(),
-                                      0, 1, 2, 16, 12, 0)
+                                      0, 1, 2, 16, 12, 12, 0)
     assert st == 1                                        # refused, not wrong
+
+
+def test_weight_rows_may_lie_apart(ops):
+    """A weight that is a view of some columns of a wider matrix: the same bits from every product."""
+    w = rnd((300, 1024), torch.bfloat16, 50).cuda()
+    wide = torch.zeros((300, 1024 + 64), dtype=torch.bfloat16, device="cuda")
+    wide[:, :1024] = w
+    ws = wide[:, :1024]
+    assert ws.stride(0) == 1088 and torch.equal(ws, w)
+    res0 = rnd((9, 300), torch.float32, 53).cuda()
+    for m in (1, 9, 64, 200):                             # skinny and library products
+        x = rnd((m, 1024), torch.bfloat16, 52).cuda()
+        for out_dtype in DTYPES:
+            assert torch.equal(ops.linear(x, ws, None, out_dtype), ops.linear(x, w, None, out_dtype))
+    x = rnd((9, 1024), torch.bfloat16, 52).cuda()
+    a, b = res0.clone(), res0.clone()
+    ops.linear(x, ws, None, torch.bfloat16, residual=a)
+    ops.linear(x, w, None, torch.bfloat16, residual=b)
+    assert torch.equal(a, b)
+    w2 = rnd((320, 1024), torch.bfloat16, 54).cuda()
+    wide2 = torch.zeros((320, 1032), dtype=torch.bfloat16, device="cuda")
+    wide2[:, :1024] = w2
+    assert torch.equal(ops.linear_swiglu(x, wide2[:, :1024]), ops.linear_swiglu(x, w2))
 
 
 @pytest.mark.parametrize("m", [1, 5, 16, 40])
