@@ -39,6 +39,18 @@ FULL = {
 }
 
 
+# the other Llama shapes the reference family covers, for measurements beside the default
+SHAPES = {
+    "1b": {},
+    "3b": {"num_hidden_layers": 28, "hidden_size": 3072, "num_attention_heads": 24, "head_dim": 128},
+    "8b": {"num_hidden_layers": 32, "hidden_size": 4096, "num_attention_heads": 32, "head_dim": 128,
+           "intermediate_size": 14336, "tie_word_embeddings": False,
+           "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
+                            "high_freq_factor": 4.0, "original_max_position_embeddings": 8192}},
+}
+NAMES = {"1b": "Llama-3.2-1B shape", "3b": "Llama-3.2-3B shape", "8b": "Llama-3.1-8B shape"}
+
+
 def log(msg):
     print("[bench] " + msg, file=sys.stderr, flush=True)
 
@@ -134,7 +146,8 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
-    ap.add_argument("--layers", type=int, default=FULL["num_hidden_layers"])
+    ap.add_argument("--shape", default="1b", choices=sorted(SHAPES), help="layer sizes (default: the 1B shape)")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
     ap.add_argument("--batch", type=int, default=8)
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--prefill", type=int, default=2048)
@@ -152,14 +165,18 @@ def main() -> int:
     from libllm_amd.sampling import Sampler, SamplingParams
 
     d = dict(FULL)
-    d["num_hidden_layers"] = args.layers
+    d.update(SHAPES[args.shape])
+    layers_full = d["num_hidden_layers"]
+    if args.layers:
+        d["num_hidden_layers"] = args.layers
+    args.layers = d["num_hidden_layers"]
     cfg = config_from_dict(d)
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     itemsize = 2 if short == "bf16" else 4
     biggest = max(args.batch, 1 if args.no_points else 64)
     max_tokens = biggest * (args.context + 64) + 4096
     log("building %d layers of %d with random weights, cache for %d tokens" %
-        (args.layers, FULL["num_hidden_layers"], max_tokens))
+        (args.layers, layers_full, max_tokens))
     engine = random_engine(cfg, seed=0, dtype=args.dtype, max_tokens=max_tokens)
     sampler = Sampler(engine.ops, cfg.vocab_size)
     params = SamplingParams(temperature=0.0)
@@ -187,17 +204,18 @@ def main() -> int:
             log("decode at batch %d: %.3f ms a step, %.0f tokens/s" % (b, dtb / args.steps * 1e3, b * args.steps / dtb))
 
     out = {
-        "metric": "decode tok/s at batch %d, context %d (Llama-3.2-1B shape)" % (args.batch, args.context),
+        "metric": "decode tok/s at batch %d, context %d (%s)" % (args.batch, args.context, NAMES[args.shape]),
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": round(ms, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": short,
         "data": "synthetic: uniform random token ids, random weights N(0, 0.02)",
         "config": {
-            "model": "Llama-3.2-1B shape", "layers": args.layers, "layers_full": FULL["num_hidden_layers"],
+            "model": NAMES[args.shape], "layers": args.layers, "layers_full": layers_full,
             "hidden": cfg.hidden_size, "heads": cfg.num_attention_heads,
             "kv_heads": cfg.num_key_value_heads, "head_dim": cfg.head_dim,
-            "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size, "tied_head": True,
-            "rope": "theta 5e5, llama3 factor 32", "global_batch": args.batch, "seq_len": args.context,
+            "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
+            "tied_head": cfg.tie_word_embeddings,
+            "rope": "theta 5e5, llama3 factor %g" % cfg.rope_scaling["factor"], "global_batch": args.batch, "seq_len": args.context,
             "prefill_tokens": args.prefill, "sampling": "greedy", "parallelism": "single GPU",
         },
         "prefill": {"value": round(args.prefill / pre_s, 1), "tokens": args.prefill,
