@@ -381,9 +381,16 @@ static int pick_shape(const SkinnyArgs& a) {
       // a long K with few rows of W: more of each row in flight per wave
       if (RT == 1 && a.K >= 4096 && a.N <= 4096) return launch_skinny<1, RT, 1, 4, EPI, false, OutT>(a);
       return launch_skinny<1, RT, 1, 2, EPI, false, OutT>(a);
-    case 2: return launch_skinny<2, RT, 2 / RT, 1, EPI, false, OutT>(a);
-    case 3: return launch_skinny<3, RT, 2 / RT, 1, EPI, false, OutT>(a);
-    case 4: return launch_skinny<4, RT, 2 / RT, 1, EPI, false, OutT>(a);
+    // two row groups per block only where W has rows enough to fill the GPU with such blocks
+    case 2:
+      if (RT == 1 && a.N < 8192) return launch_skinny<2, 1, 1, 1, EPI, false, OutT>(a);
+      return launch_skinny<2, RT, 2 / RT, 1, EPI, false, OutT>(a);
+    case 3:
+      if (RT == 1 && a.N < 8192) return launch_skinny<3, 1, 1, 1, EPI, false, OutT>(a);
+      return launch_skinny<3, RT, 2 / RT, 1, EPI, false, OutT>(a);
+    case 4:
+      if (RT == 1 && a.N < 8192) return launch_skinny<4, 1, 1, 1, EPI, false, OutT>(a);
+      return launch_skinny<4, RT, 2 / RT, 1, EPI, false, OutT>(a);
   }
   return LLM_ERR_ARG;
 }
