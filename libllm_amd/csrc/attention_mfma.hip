@@ -518,10 +518,42 @@ __global__ __launch_bounds__(WAVES * 64, (HD <= 128) ? 2 : 1) void attn_decode_k
 }
 
 // out[b, h, :] = sum_s O_s 2^(m_s - m) / sum_s l_s 2^(m_s - m) over the blocks' partials, in block
-// order; grid (n_heads, sequences), one thread per dimension.
+// order; grid (n_heads, sequences), one thread per dimension.  Up to NB partials (the template's
+// bound) are all fetched before any is used, so the kernel waits for memory once.
+template <int NB>
 __global__ void attn_decode_combine_kernel(const float* __restrict__ part_o,
                                            const float* __restrict__ part_ml,
                                            bf16_t* __restrict__ out, int n_heads, int hd, int n_blk) {
+  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  const size_t idx0 = ((size_t)b * n_heads + h) * n_blk;
+  const bool live = d < hd;
+  float ms[NB], ls[NB], os[NB];
+#pragma unroll
+  for (int s = 0; s < NB; ++s) {
+    const bool in = s < n_blk;
+    const float2 ml = in ? *reinterpret_cast<const float2*>(part_ml + (idx0 + s) * 2) : make_float2(-INFINITY, 0.f);
+    ms[s] = ml.x;
+    ls[s] = ml.y;
+    os[s] = (in && live) ? part_o[(idx0 + s) * hd + d] : 0.f;
+  }
+  float m = ms[0];
+#pragma unroll
+  for (int s = 1; s < NB; ++s) m = fmaxf(m, ms[s]);
+  float l = 0.f, o = 0.f;
+#pragma unroll
+  for (int s = 0; s < NB; ++s) {
+    const float w = (ms[s] > -INFINITY) ? exp2f(ms[s] - m) : 0.f;
+    l += ls[s] * w;
+    o += os[s] * w;
+  }
+  if (live) out[((size_t)b * n_heads + h) * hd + d] = f32_to_bf16(o / l);
+}
+
+// The same for any number of partials.
+__global__ void attn_decode_combine_loop_kernel(const float* __restrict__ part_o,
+                                                const float* __restrict__ part_ml,
+                                                bf16_t* __restrict__ out, int n_heads, int hd,
+                                                int n_blk) {
   __shared__ float s_w[1024];
   const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
   const size_t idx0 = ((size_t)b * n_heads + h) * n_blk;
@@ -616,8 +648,20 @@ extern "C" int llm_attention_decode_bf16(const void* q, int q_stride, const void
         scale_log2, window);                                                                      \
     if (n_blocks > 1) {                                                                           \
       if (hipGetLastError() != hipSuccess) return LLM_ERR_LAUNCH;                                 \
-      attn_decode_combine_kernel<<<dim3(n_heads, n_seqs), ((hd + 63) / 64) * 64, 0, stream>>>(    \
-          part_o, part_ml, (bf16_t*)out, n_heads, hd, n_blocks);                                  \
+      const dim3 cgrid(n_heads, n_seqs);                                                          \
+      const int cthreads = ((hd + 63) / 64) * 64;                                                 \
+      if (n_blocks <= 8)                                                                          \
+        attn_decode_combine_kernel<8><<<cgrid, cthreads, 0, stream>>>(part_o, part_ml,            \
+                                                                     (bf16_t*)out, n_heads, hd,   \
+                                                                     n_blocks);                   \
+      else if (n_blocks <= 32)                                                                    \
+        attn_decode_combine_kernel<32><<<cgrid, cthreads, 0, stream>>>(part_o, part_ml,           \
+                                                                      (bf16_t*)out, n_heads, hd,  \
+                                                                      n_blocks);                  \
+      else                                                                                        \
+        attn_decode_combine_loop_kernel<<<cgrid, cthreads, 0, stream>>>(part_o, part_ml,          \
+                                                                       (bf16_t*)out, n_heads, hd, \
+                                                                       n_blocks);                 \
     }                                                                                             \
     return llm_launch_status();                                                                   \
   }

@@ -486,6 +486,16 @@ def test_attention_far_key_stands_out(ops, dtype, far):
         assert max_err(out, ref) < (1e-5 if dtype == torch.float32 else BF16_2ULP)
 
 
+@pytest.mark.parametrize("ctx_len,far", [(2100, 5), (9000, 4321), (9000, 8999)])
+def test_attention_decode_over_many_pages(ops, ctx_len, far):
+    """A decoded token over thousands of keys: the pages are dealt out to many blocks whose
+    partial results a second kernel merges (through each of its variants); one far key dominates."""
+    out, ref = run_attention(ops, torch.bfloat16, 8, 2, 64, [(0, ctx_len, 1)], seed=3, boost=(far, 12.0))
+    assert max_err(out, ref) < BF16_2ULP
+    out, ref = run_attention(ops, torch.bfloat16, 4, 1, 128, [(1, ctx_len // 2, 1), (0, ctx_len, 1)], seed=4)
+    assert max_err(out, ref) < BF16_2ULP
+
+
 def test_attention_single_token_is_value(ops):
     # one query, no past: the output is the value itself
     out, ref = run_attention(ops, torch.float32, 4, 4, 32, [(0, 0, 1)])
