@@ -549,28 +549,47 @@ __global__ void attn_decode_combine_kernel(const float* __restrict__ part_o,
   if (live) out[((size_t)b * n_heads + h) * hd + d] = f32_to_bf16(o / l);
 }
 
-// The same for any number of partials.
+// The same for any number of partials: block (dims, 8 groups); group g merges partials g, g+8, ...
+// as they come (a running maximum), then the 8 groups are merged through shared memory.
 __global__ void attn_decode_combine_loop_kernel(const float* __restrict__ part_o,
                                                 const float* __restrict__ part_ml,
                                                 bf16_t* __restrict__ out, int n_heads, int hd,
                                                 int n_blk) {
-  __shared__ float s_w[1024];
-  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x;
+  __shared__ float s_m[8], s_l[8], s_o[8][256];
+  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x, grp = threadIdx.y;
   const size_t idx0 = ((size_t)b * n_heads + h) * n_blk;
-  float m = -INFINITY;
-  for (int s = 0; s < n_blk; ++s) m = fmaxf(m, part_ml[(idx0 + s) * 2]);
-  for (int s = d; s < n_blk; s += blockDim.x) {
-    const float ms = part_ml[(idx0 + s) * 2];
-    s_w[s] = (ms > -INFINITY) ? exp2f(ms - m) : 0.f;
+  const bool live = d < hd;
+  float m = -INFINITY, l = 0.f, o = 0.f;
+#pragma unroll 4
+  for (int s = grp; s < n_blk; s += 8) {
+    const float2 ml = *reinterpret_cast<const float2*>(part_ml + (idx0 + s) * 2);
+    const float ov = live ? part_o[(idx0 + s) * hd + d] : 0.f;
+    if (ml.x > -INFINITY) {
+      const float m_new = fmaxf(m, ml.x);
+      const float c_old = exp2f(m - m_new), c_new = exp2f(ml.x - m_new);   // exp2(-inf) = 0 at first
+      l = l * c_old + ml.y * c_new;
+      o = o * c_old + ov * c_new;
+      m = m_new;
+    }
   }
+  if (d == 0) {
+    s_m[grp] = m;
+    s_l[grp] = l;
+  }
+  s_o[grp][d] = o;
   __syncthreads();
-  float l = 0.f, o = 0.f;
-  for (int s = 0; s < n_blk; ++s) {
-    const float w = s_w[s];
-    l += part_ml[(idx0 + s) * 2 + 1] * w;
-    if (d < hd) o += part_o[(idx0 + s) * hd + d] * w;
+  if (grp != 0 || !live) return;
+  float mm = s_m[0];
+#pragma unroll
+  for (int g = 1; g < 8; ++g) mm = fmaxf(mm, s_m[g]);
+  float lt = 0.f, ot = 0.f;
+#pragma unroll
+  for (int g = 0; g < 8; ++g) {
+    const float w = (s_m[g] > -INFINITY) ? exp2f(s_m[g] - mm) : 0.f;
+    lt += s_l[g] * w;
+    ot += s_o[g][d] * w;
   }
-  if (d < hd) out[((size_t)b * n_heads + h) * hd + d] = f32_to_bf16(o / l);
+  out[((size_t)b * n_heads + h) * hd + d] = f32_to_bf16(ot / lt);
 }
 
 // ---------------------------------------------------------------------------------- entry points
@@ -659,9 +678,8 @@ extern "C" int llm_attention_decode_bf16(const void* q, int q_stride, const void
                                                                       (bf16_t*)out, n_heads, hd,  \
                                                                       n_blocks);                  \
       else                                                                                        \
-        attn_decode_combine_loop_kernel<<<cgrid, cthreads, 0, stream>>>(part_o, part_ml,          \
-                                                                       (bf16_t*)out, n_heads, hd, \
-                                                                       n_blocks);                 \
+        attn_decode_combine_loop_kernel<<<cgrid, dim3(cthreads, 8), 0, stream>>>(                 \
+            part_o, part_ml, (bf16_t*)out, n_heads, hd, n_blocks);                                \
     }                                                                                             \
     return llm_launch_status();                                                                   \
   }
