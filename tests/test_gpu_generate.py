@@ -61,7 +61,7 @@ def test_sampled_generation_and_stop_tokens(model_b):
     from libllm_amd import Model
     path, cfg, weights = model_b
     rng = np.random.default_rng(3)
-    prompts = [rng.integers(10, cfg.vocab, size=n).tolist() for n in (1, 17, 40, 70)]   # BASELINE's tiny B workload
+    prompts = [rng.integers(10, cfg.vocab, size=n).tolist() for n in (1, 17, 40, 70)]   # a lone token, short and longer prompts
     model = Model(path, dtype="float32", max_tokens=1024)
     got = model.generate(prompts, max_new_tokens=12, temperature=0.8, top_k=50, top_p=0.8, seed=4)
     want = [sampling.generate(cfg, weights, p, 12, 0.8, 50, 0.8, seed=4, stream=i) for i, p in enumerate(prompts)]
