@@ -188,6 +188,35 @@ def test_toy_mixer_registers_builds_and_steps(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_routed_feed_forward_and_position_encoding(ops, dtype):
+    """A feed-forward with routing and a position encoding of another kind, both defined in
+    tests/toy.py, chosen for one layer each: whole prompts and cut ones agree with the plain
+    restatement (rows whose routing is a near tie aside, in bfloat16)."""
+    cfg = llama.PlainConfig(TINY_A)
+    model = DecoderModel(toy.toys_spec(config_from_dict(TINY_A)))
+    assert "model.layers.1.moe.experts.w_in" in model.declared()
+    t = random_tensors(model.declared(), 21, std=0.1, norm_std=0.2)
+    model.bind({k: v.to("cuda", torch.float32 if (dtype == torch.float32 or v.dim() == 1) else dtype)
+                for k, v in t.items()}, ops, dtype)
+    engine = Engine(model, ops, dtype, max_tokens=512)
+    assert not engine.use_graphs                          # the routed part reads on the host
+    w = {k: v.double().numpy() for k, v in t.items()}
+    ids = np.random.default_rng(8).integers(0, 256, size=100).tolist()
+    ref, margin = toy.toys_oracle(cfg, w, ids)
+    whole = engine.step([StepEntry("a", ids, list(range(100)))]).double().cpu().numpy()
+    engine.end(["a"])
+    cut = torch.cat([engine.step([StepEntry("b", ids[:70], list(range(70)))]).clone()] +
+                    [engine.step([StepEntry("b", [x], [0])]).clone() for x in ids[70:]]).double().cpu().numpy()
+    engine.end(["b"])
+    clear = margin > (1e-6 if dtype == torch.float32 else 0.05)
+    assert clear.sum() > 80
+    # the routed layer is the last one: a near tie at one row does not touch the other rows
+    assert_logits_close(whole[clear], ref[clear], dtype, "whole")
+    assert_logits_close(cut[clear], ref[clear], dtype, "cut")
+    engine.cache.check()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_schedule_and_mixed_layers_on_the_gpu(ops, dtype):
     """A layer run twice, a run that reads another run's keys, and a layer with a window and
     another grouping: whole prompts and single tokens agree."""

@@ -75,3 +75,124 @@ def toy_oracle(cfg, weights, toy_weight, ids, decay=0.5):
         x = x + np.stack(mixed)
         x = x + llama.mlp(cfg, weights, layer, llama.rms_norm(x, weights[p + "post_attention_layernorm.weight"], cfg.eps))
     return llama.lm_head(cfg, weights, llama.rms_norm(x, weights["model.norm.weight"], cfg.eps))
+
+
+# ---------------------------------------------------------------------------------------------
+# A feed-forward with routing and a position encoding of another kind, both defined here: they
+# are registered, chosen per layer in a model record, bound and stepped like the built-in parts.
+from libllm_amd.parts import FeedForward, register_feed_forward, register_position  # noqa: E402
+
+
+@dataclass
+class TopOneSpec(PartSpec):
+    width: int = 0
+    inner: int = 0
+    n_experts: int = 2
+
+
+@register_feed_forward("top1_experts")
+class TopOneExperts(FeedForward):
+    """Each row goes to the one expert whose router logit (in 32-bit) is largest:
+    y = W_out[e] relu(W_in[e] x)."""
+    graph_safe = False               # the rows of an expert are picked on the host's say
+
+    def __init__(self, spec: TopOneSpec):
+        self.spec = spec
+
+    def weights(self):
+        s = self.spec
+        return {"router.weight": WeightDecl((s.n_experts, s.width)),
+                "experts.w_in": WeightDecl((s.n_experts, s.inner, s.width)),
+                "experts.w_out": WeightDecl((s.n_experts, s.width, s.inner))}
+
+    def bind(self, tensors, ops, dtype):
+        self.router = tensors["router.weight"].float()
+        self.w_in, self.w_out = tensors["experts.w_in"], tensors["experts.w_out"]
+
+    def forward(self, ctx, x):
+        choice = (x.float() @ self.router.t()).argmax(dim=-1)
+        out = torch.zeros_like(x)
+        for e in range(self.spec.n_experts):
+            rows = (choice == e).nonzero().flatten()
+            if rows.numel():
+                h = torch.relu(x[rows].float() @ self.w_in[e].float().t())
+                out[rows] = (h @ self.w_out[e].float().t()).to(x.dtype)
+        return out
+
+
+@dataclass
+class ClockSpec(PartSpec):
+    rot_dim: int = 0
+    max_position: int = 0
+    step: float = 0.05
+
+
+@register_position("clock")
+class ClockPosition:
+    """Pair j of the first rot_dim dims turns by position * (j + 1) * step."""
+
+    def __init__(self, spec: ClockSpec):
+        self.spec, self.rot_dim = spec, spec.rot_dim
+
+    def angles(self):
+        pos = torch.arange(self.spec.max_position, dtype=torch.float64)
+        return pos[:, None] * (torch.arange(self.rot_dim // 2, dtype=torch.float64) + 1.0) * self.spec.step
+
+    def tables(self, device):
+        a = self.angles()
+        return torch.cos(a).float().to(device), torch.sin(a).float().to(device)
+
+
+def toys_spec(base_config):
+    """The Llama model as data with layer 0's position encoding and layer 1's feed-forward
+    replaced by the toys above."""
+    spec = base_config.to_spec()
+    spec.layers[0].mixer.position = ClockSpec(kind="clock", rot_dim=spec.layers[0].mixer.head_dim // 2,
+                                              max_position=spec.max_position)
+    spec.layers[1].feed_forward = TopOneSpec(kind="top1_experts", width=spec.width, inner=48, n_experts=3)
+    spec.layers[1].prefixes["feed_forward"] = "model.layers.1.moe."
+    return spec
+
+
+def toys_oracle(cfg, weights, ids, step=0.05):
+    """The same model through the plain functions, the two toys restated in numpy."""
+    import numpy as np
+
+    from plain import llama
+    t = len(ids)
+    x = llama.embedding(weights["model.embed_tokens.weight"], ids)
+    positions = np.arange(t)
+    # layer 0: attention with the clock rotation on the first half of every head
+    p = "model.layers.0."
+    h = llama.rms_norm(x, weights[p + "input_layernorm.weight"], cfg.eps)
+    wqkv, _ = llama.fused_qkv(weights, p + "self_attn.")
+    qkv = llama.linear(h, wqkv)
+    qd, kd, hd = cfg.n_heads * cfg.head_dim, cfg.n_kv * cfg.head_dim, cfg.head_dim
+    q = qkv[:, :qd].reshape(t, cfg.n_heads, hd)
+    k = qkv[:, qd:qd + kd].reshape(t, cfg.n_kv, hd)
+    v = qkv[:, qd + kd:].reshape(t, cfg.n_kv, hd)
+    rot = hd // 2
+    ang = positions[:, None] * (np.arange(rot // 2) + 1.0) * step
+    cos, sin = np.cos(ang)[:, None, :], np.sin(ang)[:, None, :]
+
+    def turn(a):
+        a = a.copy()
+        a1, a2 = a[..., :rot // 2].copy(), a[..., rot // 2:rot].copy()
+        a[..., :rot // 2] = a1 * cos - a2 * sin
+        a[..., rot // 2:rot] = a2 * cos + a1 * sin
+        return a
+    o = llama.attention(turn(q).transpose(1, 0, 2), turn(k).transpose(1, 0, 2), v.transpose(1, 0, 2), True)
+    x = x + llama.linear(o.transpose(1, 0, 2).reshape(t, qd), weights[p + "self_attn.o_proj.weight"])
+    x = x + llama.mlp(cfg, weights, 0, llama.rms_norm(x, weights[p + "post_attention_layernorm.weight"], cfg.eps))
+    # layer 1: plain attention, routed feed-forward
+    p = "model.layers.1."
+    x = x + llama.attention_block(cfg, weights, 1, llama.rms_norm(x, weights[p + "input_layernorm.weight"], cfg.eps), positions)
+    h = llama.rms_norm(x, weights[p + "post_attention_layernorm.weight"], cfg.eps)
+    logits = h @ weights[p + "moe.router.weight"].T
+    choice = logits.argmax(-1)
+    margin = np.sort(logits, axis=-1)
+    y = np.stack([weights[p + "moe.experts.w_out"][e] @ np.maximum(weights[p + "moe.experts.w_in"][e] @ row, 0.0)
+                  for row, e in zip(h, choice)])
+    x = x + y
+    out = llama.lm_head(cfg, weights, llama.rms_norm(x, weights["model.norm.weight"], cfg.eps))
+    return out, margin[:, -1] - margin[:, -2]
