@@ -1,4 +1,4 @@
-// Arg-max and temperature / top-k / top-p sampling over float32 logits, one block per row.
+// Arg-max and temperature / top-k / top-p sampling over float32 logits.
 //
 // Order of operations as in the reference (src/libllm/generator.cc:197-214, 47-113):
 // z = logits / temperature, p = softmax(z) over the whole vocabulary, the top_k largest sorted
@@ -132,108 +132,243 @@ __device__ __forceinline__ T block_inclusive_scan(T v, T* buf, T* total) {
   return v + before;
 }
 
-template <int NT, int KMAX>
-__global__ __launch_bounds__(NT) void sample_kernel(const float* __restrict__ logits, int V,
-                                                     float inv_temp, int top_k, float top_p,
-                                                     uint64_t seed, const long long* __restrict__ streams,
-                                                     const long long* __restrict__ counters,
-                                                     int* __restrict__ out) {
-  __shared__ float fbuf[NT / 64];
-  __shared__ int ibuf[NT / 64];
-  __shared__ unsigned int hist[256];
-  __shared__ unsigned long long cand[KMAX];
-  __shared__ unsigned int sh_prefix, sh_need, sh_count;
-  __shared__ int sh_result;
+// The radix-selection step over a histogram of 256 bins: the bin in which the `need`-th largest
+// key lies, and how many keys of that bin are still needed.  Threads 0..255 take part (the block
+// has at least 256); bins are scanned from 255 down by a parallel prefix sum.  `wsum` needs 4
+// entries.  All threads of the block must call it; the results are in sh_bin / sh_rest after it.
+__device__ __forceinline__ void select_bin(const unsigned int* hist, unsigned need, unsigned* wsum,
+                                           unsigned* sh_bin, unsigned* sh_rest) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  unsigned v = 0, inc = 0;
+  if (tid < 256) {
+    v = hist[255 - tid];
+    inc = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const unsigned o = __shfl_up(inc, off, 64);
+      if (lane >= off) inc += o;
+    }
+    if (lane == 63) wsum[wave] = inc;
+  }
+  __syncthreads();
+  if (tid < 256) {
+    unsigned before = 0;
+    for (int w = 0; w < wave; ++w) before += wsum[w];
+    inc += before;
+    // the first bin (from the top) at which the running count reaches `need`; if the counts never
+    // reach it (cannot happen when need <= number of keys) the lowest bin takes the rest
+    const bool here = (inc >= need && inc - v < need) || (tid == 255 && inc < need);
+    if (here) {
+      *sh_bin = 255u - (unsigned)tid;
+      *sh_rest = need - (inc - v);
+    }
+  }
+  __syncthreads();
+}
 
+// Sampling in two stages, so that one row still uses many compute units.
+//
+// Stage 1, grid (parts, rows): a block owns a contiguous slice of at most SP_PER logits.  It
+// writes the slice's maximum of z and its sum of exp(z - maximum), and, with top_k > 0, the
+// slice's min(top_k, size) largest logits as 64-bit keys (order key << 32 | ~index: a larger key
+// is a larger logit or, between equal logits, a lower index), found by radix selection over the
+// slice held in shared memory.
+// Stage 2, one block a row: the normaliser from the parts; with top_k > 0 the top_k largest of all
+// candidate keys by radix selection over the 64-bit keys (they are distinct, so no ties remain),
+// sorted, then nucleus and draw sequentially; with top_k == 0 the part and then the element at
+// which the running sum in index order passes u * Z.
+#define SP_PER 4096          // most logits of a stage-1 slice
+#define SP_NT 512            // threads of a stage-1 block
+#define SP_KMAX 1024         // most candidates kept
+
+struct SampleParts {
+  float* part_max;            // [rows, parts]
+  float* part_sum;            // [rows, parts]
+  unsigned long long* cand;   // [rows, parts, k_part]
+};
+
+__global__ __launch_bounds__(SP_NT) void sample_part_kernel(const float* __restrict__ logits, int V,
+                                                             int per, float inv_temp, int k_part,
+                                                             SampleParts out) {
+  __shared__ float vals[SP_PER];
+  __shared__ float fbuf[SP_NT / 64];
+  __shared__ int ibuf[SP_NT / 64];
+  __shared__ unsigned int hist[256], wsum[4];
+  __shared__ unsigned int sh_prefix, sh_need, sh_count, sh_bin, sh_rest;
+  const int part = blockIdx.x, row = blockIdx.y, parts = gridDim.x, tid = threadIdx.x;
+  const int lo = part * per;
+  const int n = min(per, V - lo);                       // >= 1 by the choice of parts
+  const float* x = logits + (size_t)row * V + lo;
+  float mx = -INFINITY;
+  for (int i = tid; i < n; i += SP_NT) {
+    const float v = x[i];
+    vals[i] = v;
+    mx = fmaxf(mx, v * inv_temp);
+  }
+  mx = block_max<SP_NT>(mx, fbuf);                      // also orders the writes to vals
+  float sum = 0.f;
+  for (int i = tid; i < n; i += SP_NT) sum += expf(vals[i] * inv_temp - mx);
+  sum = block_sum<SP_NT>(sum, fbuf);
+  if (tid == 0) {
+    out.part_max[row * parts + part] = mx;
+    out.part_sum[row * parts + part] = sum;
+  }
+  if (k_part <= 0) return;
+  unsigned long long* cand = out.cand + ((size_t)row * parts + part) * k_part;
+  const int k = min(k_part, n);
+  for (int i = k + tid; i < k_part; i += SP_NT) cand[i] = 0ull;       // a short slice: empty places
+
+  // ---- the k-th largest key of the slice by radix selection, 8 bits a pass
+  if (tid == 0) { sh_prefix = 0; sh_need = (unsigned)k; }
+  __syncthreads();
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+    for (int b = tid; b < 256; b += SP_NT) hist[b] = 0;
+    __syncthreads();
+    const unsigned prefix = sh_prefix;
+    for (int i = tid; i < n; i += SP_NT) {
+      const uint32_t key = order_key(vals[i]);
+      if (pass == 0 || (key >> (shift + 8)) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+    }
+    __syncthreads();
+    select_bin(hist, sh_need, wsum, &sh_bin, &sh_rest);
+    if (tid == 0) {
+      sh_need = sh_rest;
+      sh_prefix = (prefix << 8) | sh_bin;
+    }
+    __syncthreads();
+  }
+  const uint32_t kth = sh_prefix;
+  const int need_eq = (int)sh_need;          // how many logits equal to the k-th are taken: the lowest indices
+  const int n_gt = k - need_eq;
+  if (tid == 0) sh_count = 0;
+  __syncthreads();
+  // contiguous chunks per thread, so that equal keys are ranked by index
+  const int chunk = (n + SP_NT - 1) / SP_NT;
+  const int c0 = min(n, tid * chunk), c1 = min(n, c0 + chunk);
+  int eq_mine = 0;
+  for (int i = c0; i < c1; ++i) {
+    const uint32_t key = order_key(vals[i]);
+    if (key > kth) {
+      const unsigned p = atomicAdd(&sh_count, 1u);
+      cand[p] = ((unsigned long long)key << 32) | (0xffffffffu - (uint32_t)(lo + i));
+    } else if (key == kth) {
+      ++eq_mine;
+    }
+  }
+  int eq_total;
+  const int eq_inc = block_inclusive_scan<int, SP_NT>(eq_mine, ibuf, &eq_total);
+  int rank = eq_inc - eq_mine;
+  if (eq_mine > 0 && rank < need_eq) {
+    for (int i = c0; i < c1 && rank < need_eq; ++i) {
+      if (order_key(vals[i]) == kth) {
+        cand[n_gt + rank] = ((unsigned long long)kth << 32) | (0xffffffffu - (uint32_t)(lo + i));
+        ++rank;
+      }
+    }
+  }
+}
+
+template <int NT>
+__global__ __launch_bounds__(NT) void sample_final_kernel(const float* __restrict__ logits, int V,
+                                                           int per, int parts, float inv_temp,
+                                                           int top_k, int k_part, float top_p,
+                                                           uint64_t seed,
+                                                           const long long* __restrict__ streams,
+                                                           const long long* __restrict__ counters,
+                                                           SampleParts in, int* __restrict__ out) {
+  __shared__ float fbuf[NT / 64];
+  __shared__ unsigned int hist[256], wsum[4];
+  __shared__ unsigned long long cand[SP_KMAX];
+  __shared__ unsigned long long sh_prefix;
+  __shared__ unsigned int sh_need, sh_count, sh_bin, sh_rest;
+  __shared__ int sh_result, sh_part;
+  __shared__ float sh_before;
   const int row = blockIdx.x, tid = threadIdx.x;
   const float* x = logits + (size_t)row * V;
   const float u = counter_uniform(seed, (uint64_t)streams[row], (uint64_t)counters[row]);
+  const float* pm = in.part_max + (size_t)row * parts;
+  const float* ps = in.part_sum + (size_t)row * parts;
 
-  // max and normaliser of softmax(z), z = x * inv_temp
+  // the row's maximum and normaliser from the parts, in part order
   float mx = -INFINITY;
-  for (int i = tid; i < V; i += NT) mx = fmaxf(mx, x[i] * inv_temp);
-  mx = block_max<NT>(mx, fbuf);
-
-  const int chunk = (V + NT - 1) / NT;
-  const int c0 = min(V, tid * chunk), c1 = min(V, c0 + chunk);
-  float part = 0.f;
-  for (int i = c0; i < c1; ++i) part += expf(x[i] * inv_temp - mx);
-  float Z;
-  const float inc = block_inclusive_scan<float, NT>(part, fbuf, &Z);
-
-  if (tid == 0) sh_result = V - 1;
-  __syncthreads();
+  for (int p = 0; p < parts; ++p) mx = fmaxf(mx, pm[p]);
+  float Z = 0.f;
+  for (int p = 0; p < parts; ++p) Z += ps[p] * expf(pm[p] - mx);
 
   if (top_k <= 0) {
-    // nothing is cut: walk the vocabulary in index order
+    // nothing is cut: the part, then the element, where the running sum passes r
     const float r = u * Z;
-    const float lo = inc - part;          // running sum before this thread's chunk
-    if (c1 > c0 && r >= lo && r < inc) {
-      float run = lo;
-      int pick = c1 - 1;
+    if (tid == 0) {
+      float run = 0.f;
+      int p = 0;
+      for (; p < parts - 1; ++p) {
+        const float next = run + ps[p] * expf(pm[p] - mx);
+        if (r < next) break;
+        run = next;
+      }
+      sh_part = p;
+      sh_before = run;
+    }
+    __syncthreads();
+    const int lo = sh_part * per;
+    const int n = min(per, V - lo);
+    const int chunk = (n + NT - 1) / NT;
+    const int c0 = min(n, tid * chunk), c1 = min(n, c0 + chunk);
+    float part = 0.f;
+    for (int i = c0; i < c1; ++i) part += expf(x[lo + i] * inv_temp - mx);
+    float total;
+    const float inc = sh_before + block_inclusive_scan<float, NT>(part, fbuf, &total);
+    if (tid == 0) sh_result = lo + n - 1;               // rounding left r beyond the part's end
+    __syncthreads();
+    const float before = inc - part;
+    if (c1 > c0 && r >= before && r < inc) {
+      float run = before;
+      int pick = lo + c1 - 1;
       for (int i = c0; i < c1; ++i) {
-        run += expf(x[i] * inv_temp - mx);
-        if (r < run) { pick = i; break; }
+        run += expf(x[lo + i] * inv_temp - mx);
+        if (r < run) { pick = lo + i; break; }
       }
       sh_result = pick;
+    } else if (tid == 0 && r < sh_before) {
+      sh_result = lo;
     }
     __syncthreads();
     if (tid == 0) out[row] = sh_result;
     return;
   }
 
-  // ---- the top_k-th largest key by radix selection, 8 bits a pass
-  if (tid == 0) { sh_prefix = 0; sh_need = (unsigned)top_k; }
+  // ---- the top_k largest candidate keys: radix selection over 64 bits, 8 bits a pass
+  const unsigned long long* all = in.cand + (size_t)row * parts * k_part;
+  const int C = parts * k_part;
+  if (tid == 0) { sh_prefix = 0ull; sh_need = (unsigned)top_k; }
   __syncthreads();
-  for (int pass = 0; pass < 4; ++pass) {
-    const int shift = 24 - 8 * pass;
+  for (int pass = 0; pass < 8; ++pass) {
+    const int shift = 56 - 8 * pass;
     for (int b = tid; b < 256; b += NT) hist[b] = 0;
     __syncthreads();
-    const unsigned prefix = sh_prefix;
-    for (int i = tid; i < V; i += NT) {
-      const uint32_t key = order_key(x[i]);
-      if (pass == 0 || (key >> (shift + 8)) == prefix) atomicAdd(&hist[(key >> shift) & 255u], 1u);
+    const unsigned long long prefix = sh_prefix;
+    for (int i = tid; i < C; i += NT) {
+      const unsigned long long key = all[i];
+      if (pass == 0 || (key >> (shift + 8)) == prefix) atomicAdd(&hist[(unsigned)(key >> shift) & 255u], 1u);
     }
     __syncthreads();
+    select_bin(hist, sh_need, wsum, &sh_bin, &sh_rest);
     if (tid == 0) {
-      unsigned need = sh_need, cum = 0;
-      int b = 255;
-      for (; b > 0; --b) {
-        if (cum + hist[b] >= need) break;
-        cum += hist[b];
-      }
-      sh_need = need - cum;               // still to take inside bin b
-      sh_prefix = (prefix << 8) | (unsigned)b;
+      sh_need = sh_rest;
+      sh_prefix = (prefix << 8) | (unsigned long long)sh_bin;
     }
     __syncthreads();
   }
-  const uint32_t kth = sh_prefix;         // key of the top_k-th largest logit
-  const int need_eq = (int)sh_need;       // how many logits equal to it are taken (lowest indices)
-  const int n_gt = top_k - need_eq;
-
-  // ---- collect: everything above the threshold, then the first need_eq equal ones by index
+  const unsigned long long kth = sh_prefix;             // the top_k-th largest key; keys are distinct
   if (tid == 0) sh_count = 0;
-  for (int i = tid; i < KMAX; i += NT) cand[i] = 0ull;
+  for (int i = tid; i < SP_KMAX; i += NT) cand[i] = 0ull;
   __syncthreads();
-  int eq_mine = 0;
-  for (int i = c0; i < c1; ++i) {
-    const uint32_t key = order_key(x[i]);
-    if (key > kth) {
+  for (int i = tid; i < C; i += NT) {
+    const unsigned long long key = all[i];
+    if (key >= kth && key != 0ull) {
       const unsigned p = atomicAdd(&sh_count, 1u);
-      if (p < (unsigned)KMAX) cand[p] = ((unsigned long long)key << 32) | (0xffffffffu - (uint32_t)i);
-    } else if (key == kth) {
-      ++eq_mine;
-    }
-  }
-  int eq_total;
-  const int eq_inc = block_inclusive_scan<int, NT>(eq_mine, ibuf, &eq_total);
-  int rank = eq_inc - eq_mine;
-  if (eq_mine > 0 && rank < need_eq) {
-    for (int i = c0; i < c1 && rank < need_eq; ++i) {
-      if (order_key(x[i]) == kth) {
-        cand[n_gt + rank] = ((unsigned long long)kth << 32) | (0xffffffffu - (uint32_t)i);
-        ++rank;
-      }
+      if (p < (unsigned)SP_KMAX) cand[p] = key;
     }
   }
   __syncthreads();
@@ -243,48 +378,77 @@ __global__ __launch_bounds__(NT) void sample_kernel(const float* __restrict__ lo
   while (P < top_k) P <<= 1;
   for (int k = 2; k <= P; k <<= 1) {
     for (int j = k >> 1; j > 0; j >>= 1) {
-      if (tid < P) {
-        const int other = tid ^ j;
-        if (other > tid) {
-          const unsigned long long a = cand[tid], b = cand[other];
-          const bool desc = (tid & k) == 0;
-          if (desc ? (a < b) : (a > b)) { cand[tid] = b; cand[other] = a; }
+      for (int t = tid; t < P; t += NT) {
+        const int other = t ^ j;
+        if (other > t) {
+          const unsigned long long a = cand[t], b = cand[other];
+          const bool desc = (t & k) == 0;
+          if (desc ? (a < b) : (a > b)) { cand[t] = b; cand[other] = a; }
         }
       }
       __syncthreads();
     }
   }
 
-  // ---- nucleus and draw, sequentially in candidate order
+  // ---- nucleus and draw, sequentially in candidate order; the probabilities are fetched by all
+  // threads first, so that the walk waits for memory once
+  __shared__ float prob[SP_KMAX];
+  for (int i = tid; i < top_k; i += NT) {
+    const int idx = (int)(0xffffffffu - (uint32_t)(cand[i] & 0xffffffffull));
+    prob[i] = expf(x[idx] * inv_temp - mx) / Z;
+  }
+  __syncthreads();
   if (tid == 0) {
     float kept = 0.f;
     int n = 0;
     for (int i = 0; i < top_k; ++i) {
-      const int idx = (int)(0xffffffffu - (uint32_t)(cand[i] & 0xffffffffull));
-      kept += expf(x[idx] * inv_temp - mx) / Z;
+      kept += prob[i];
       ++n;
       if (kept >= top_p) break;
     }
     const float r = u * kept;
     float run = 0.f;
-    int pick = (int)(0xffffffffu - (uint32_t)(cand[n - 1] & 0xffffffffull));
+    int pick = n - 1;
     for (int i = 0; i < n; ++i) {
-      const int idx = (int)(0xffffffffu - (uint32_t)(cand[i] & 0xffffffffull));
-      run += expf(x[idx] * inv_temp - mx) / Z;
-      if (r < run) { pick = idx; break; }
+      run += prob[i];
+      if (r < run) { pick = i; break; }
     }
-    out[row] = pick;
+    out[row] = (int)(0xffffffffu - (uint32_t)(cand[pick] & 0xffffffffull));
   }
+}
+
+// Parts a row of V logits is cut into, and candidates kept per part: the scratch arrays hold
+// rows * parts floats each and rows * parts * k_part keys.
+extern "C" int llm_sample_parts(int V) {
+  const int parts = (V + SP_PER - 1) / SP_PER;
+  return parts < 1 ? 1 : parts;
+}
+
+extern "C" int llm_sample_k_part(int V, int top_k) {
+  if (top_k <= 0) return 0;
+  const int parts = llm_sample_parts(V);
+  const int per = (V + parts - 1) / parts;
+  return top_k < per ? top_k : per;
 }
 
 extern "C" int llm_sample(const float* logits, int* out, int R, int V, float temperature, int top_k,
                           float top_p, unsigned long long seed, const long long* streams,
-                          const long long* counters, hipStream_t stream) {
+                          const long long* counters, float* part_max, float* part_sum,
+                          unsigned long long* cand, hipStream_t stream) {
   if (R <= 0) return LLM_OK;
-  if (V <= 0 || !(temperature > 0.f) || top_k < 0 || top_k > 1024 || top_k > V ||
-      !(top_p > 0.f && top_p <= 1.f) || (top_k == 0 && top_p < 1.f))
+  if (V <= 0 || R > 65535 || !(temperature > 0.f) || top_k < 0 || top_k > SP_KMAX || top_k > V ||
+      !(top_p > 0.f && top_p <= 1.f) || (top_k == 0 && top_p < 1.f) || !part_max || !part_sum ||
+      (top_k > 0 && !cand))
     return LLM_ERR_ARG;
-  sample_kernel<1024, 1024><<<R, 1024, 0, stream>>>(logits, V, 1.0f / temperature, top_k, top_p,
-                                                    (uint64_t)seed, streams, counters, out);
+  const int parts = llm_sample_parts(V);
+  if (parts > 65535) return LLM_ERR_ARG;
+  const int per = (V + parts - 1) / parts;
+  const int k_part = llm_sample_k_part(V, top_k);
+  SampleParts sp{part_max, part_sum, cand};
+  const float inv_temp = 1.0f / temperature;
+  sample_part_kernel<<<dim3(parts, R), SP_NT, 0, stream>>>(logits, V, per, inv_temp, k_part, sp);
+  if (hipGetLastError() != hipSuccess) return LLM_ERR_LAUNCH;
+  sample_final_kernel<1024><<<R, 1024, 0, stream>>>(logits, V, per, parts, inv_temp, top_k, k_part,
+                                                    top_p, (uint64_t)seed, streams, counters, sp, out);
   return llm_launch_status();
 }

@@ -49,7 +49,9 @@ _SIGNATURES = {
     "llm_attention_decode_waves": [_i],
     "llm_argmax": [_vp, _vp, _vp, _vp, _i, _i, _vp],
     "llm_argmax_parts": [_i],
-    "llm_sample": [_vp, _vp, _i, _i, _f, _i, _f, _u64, _vp, _vp, _vp],
+    "llm_sample": [_vp, _vp, _i, _i, _f, _i, _f, _u64, _vp, _vp, _vp, _vp, _vp, _vp],
+    "llm_sample_parts": [_i],
+    "llm_sample_k_part": [_i, _i],
 }
 
 
@@ -452,7 +454,13 @@ class HipOps:
             raise KernelError("sample: one stream and counter per row are needed")
         keys = torch.tensor([streams, counters], dtype=torch.int64).to(self.device)
         out = torch.empty((r,), dtype=torch.int32, device=self.device)
+        parts = self.lib.llm_sample_parts(v)
+        k_part = self.lib.llm_sample_k_part(v, int(top_k))
+        part_max = torch.empty((r * parts,), dtype=torch.float32, device=self.device)
+        part_sum = torch.empty((r * parts,), dtype=torch.float32, device=self.device)
+        cand = torch.empty((max(1, r * parts * k_part),), dtype=torch.int64, device=self.device)
         self._check(self.lib.llm_sample(logits.data_ptr(), out.data_ptr(), r, v, float(temperature),
                                         int(top_k), float(top_p), int(seed) & (2**64 - 1),
-                                        keys[0].data_ptr(), keys[1].data_ptr(), self._stream()), "sample")
+                                        keys[0].data_ptr(), keys[1].data_ptr(), part_max.data_ptr(),
+                                        part_sum.data_ptr(), cand.data_ptr(), self._stream()), "sample")
         return out
