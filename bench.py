@@ -141,6 +141,63 @@ def time_prefill(engine, torch, tokens, vocab, reps):
     return best
 
 
+def run_workload(args, torch):
+    """The two generation workloads beside the headline: 16 prompts of unequal lengths (uniform in
+    [64, 2048]) with 256 tokens each, or 64 prompts of 1,024 tokens with 512 tokens each, through
+    the generation loop (greedy, no stop token)."""
+    import numpy as np
+
+    from libllm_amd.cache import PAGE
+    from libllm_amd.config import config_from_dict
+    from libllm_amd.engine import Generator
+    from libllm_amd.runtime import random_engine
+    from libllm_amd.sampling import Sampler, SamplingParams
+    d = dict(FULL)
+    d.update(SHAPES[args.shape])
+    d["eos_token_id"] = None
+    cfg = config_from_dict(d)
+    rng = np.random.default_rng(0)
+    if args.workload == "batch64":
+        prompts = [rng.integers(0, cfg.vocab_size, size=1024).tolist() for _ in range(64)]
+        new = 512
+    else:
+        prompts = [rng.integers(0, cfg.vocab_size, size=int(n)).tolist()
+                   for n in rng.integers(64, 2049, size=16)]
+        new = 256
+    need = sum((len(p) + new + PAGE) // PAGE * PAGE for p in prompts) + 4096
+    engine = random_engine(cfg, seed=0, dtype=args.dtype, max_tokens=need)
+    gen = Generator(engine, Sampler(engine.ops, cfg.vocab_size), (), cfg.max_position_embeddings,
+                    engine.cache.n_pages, PAGE, max_batch=64)
+    result = None
+    for rep in range(2):                                   # the first run warms up and captures graphs
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        first = []
+
+        def on_token(i, tok):
+            if not first:
+                torch.cuda.synchronize()
+                first.append(time.perf_counter() - t0)
+        out = gen.generate(prompts, SamplingParams(temperature=0.0), max_new_tokens=new, on_token=on_token)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        n_prompt, n_out = sum(len(p) for p in prompts), sum(len(o) for o in out)
+        result = {
+            "metric": "generated tok/s, %s workload (%s)" % (args.workload, NAMES[args.shape]),
+            "value": round((n_out - len(prompts)) / (dt - first[0]), 1), "unit": "tokens/s", "n_gpus": 1,
+            "steps": new - 1, "warmup": 0, "ms_per_step": round((dt - first[0]) / (new - 1) * 1e3, 3),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+            "data": "synthetic: uniform random token ids, random weights N(0, 0.02)",
+            "config": {"model": NAMES[args.shape], "layers": cfg.num_hidden_layers, "prompts": len(prompts),
+                       "prompt_tokens": n_prompt, "new_tokens_each": new, "sampling": "greedy"},
+            "prefill": {"value": round(n_prompt / first[0], 1), "tokens": n_prompt, "ms": round(first[0] * 1e3, 2)},
+        }
+        log("run %d: first tokens after %.1f ms, then %.2f ms a step" % (rep, first[0] * 1e3, result["ms_per_step"]))
+    print(json.dumps(result), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -153,12 +210,17 @@ def main() -> int:
     ap.add_argument("--prefill", type=int, default=2048)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64")
+    ap.add_argument("--workload", choices=["unequal16", "batch64"],
+                    help="run a generation workload through the generation loop instead")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this library does not run on several (--gpus %d)" % args.gpus)
         return 2
 
     import torch
+
+    if args.workload:
+        return run_workload(args, torch)
 
     from libllm_amd.config import config_from_dict
     from libllm_amd.runtime import random_engine
