@@ -97,9 +97,15 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   const bf16_t* wp[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    int n = tile_row[rt] + r;
-    if (n > N - 1) n = N - 1;                   // rows past the end read the last row; not stored
-    wp[rt] = W + (size_t)n * ldw + g * 8;
+    if (ldw == 0) {                             // tiled for the matrix cores: see llm_pack_weight
+      int t = tile_row[rt] / 16;
+      if (t > (N - 1) / 16) t = (N - 1) / 16;
+      wp[rt] = W + ((size_t)t * n_steps * 64 + lane) * 8;
+    } else {
+      int n = tile_row[rt] + r;
+      if (n > N - 1) n = N - 1;                 // rows past the end read the last row; not stored
+      wp[rt] = W + (size_t)n * ldw + g * 8;
+    }
   }
 
   f32x4 acc[RT][MT];
@@ -161,6 +167,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
       if (row < 16 * MT) *reinterpret_cast<uint4*>(lds + row * ROW_B + ((x_col ^ (row & 7)) * 16)) = xr[p];
     }
   };
+  const int wstep = (ldw == 0) ? 512 : 32;       // elements between a lane's fragments of consecutive steps
   Frag a[3][G][2][RT];
   auto load_w = [&](int chunk, Frag (&dst)[G][2][RT]) {
 #pragma unroll
@@ -170,7 +177,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
         const int s = chunk * (CK / 32) + gi * 16 + wk * 2 + u;
         const bool in = s < n_steps && (s * 32 + g * 8) < K;
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) dst[gi][u][rt] = in ? frag_load(wp[rt] + s * 32) : frag_zero();
+        for (int rt = 0; rt < RT; ++rt) dst[gi][u][rt] = in ? frag_load(wp[rt] + (size_t)s * wstep) : frag_zero();
       }
   };
   auto compute = [&](Frag (&src)[G][2][RT]) {
@@ -395,7 +402,8 @@ static int pick_shape(const SkinnyArgs& a) {
   return LLM_ERR_ARG;
 }
 
-// Rows of W lie ldw elements apart (ldw >= K, a multiple of 8).
+// Rows of W lie ldw elements apart (ldw >= K, a multiple of 8); ldw == 0 says that W is the
+// tiled copy that llm_pack_weight makes.
 // C[M, N] (epilogue 0: stored as out_dtype; 2: added into the float32 C) or C[M, N/2] (epilogue 1,
 // SwiGLU over W = [Wg; Wu], N/2 a multiple of 16) from X[M, K] and W[N, K].  X is bfloat16, or,
 // with norm_x given (M <= 16), the rows `norm_rows` of the float32 matrix norm_x, RMS-normalised
@@ -405,7 +413,7 @@ extern "C" int llm_gemm_skinny_bf16(const void* X, const float* norm_x, const fl
                                     int epilogue, int out_dtype, int M, int N, int K, int ldw,
                                     hipStream_t stream) {
   if (M <= 0 || N <= 0) return LLM_OK;
-  if (M > 64 || K <= 0 || (K & 7) || ldw < K || (ldw & 7)) return LLM_ERR_ARG;
+  if (M > 64 || K <= 0 || (K & 7) || (ldw != 0 && (ldw < K || (ldw & 7)))) return LLM_ERR_ARG;
   const void* x = norm_x ? (const void*)norm_x : X;
   if (x == nullptr || W == nullptr || C == nullptr) return LLM_ERR_ARG;
   if ((((uintptr_t)x) | ((uintptr_t)W) | ((uintptr_t)C)) & 15) return LLM_ERR_ARG;
@@ -452,7 +460,7 @@ extern "C" int llm_gemm_skinny_rope_bf16(const void* X, const float* norm_x, con
                                          void* k_pages, void* v_pages, int page_size, int write_kv,
                                          hipStream_t stream) {
   if (M <= 0) return LLM_OK;
-  if (M > 64 || K <= 0 || (K & 7) || ldw < K || (ldw & 7) || n_heads <= 0 || n_kv < 0 || hd <= 0 || (hd & 15) || rot_dim < 0 ||
+  if (M > 64 || K <= 0 || (K & 7) || (ldw != 0 && (ldw < K || (ldw & 7))) || n_heads <= 0 || n_kv < 0 || hd <= 0 || (hd & 15) || rot_dim < 0 ||
       rot_dim > hd || (rot_dim & 1) || page_size != 64)
     return LLM_ERR_ARG;
   const void* x = norm_x ? (const void*)norm_x : X;
@@ -493,4 +501,31 @@ extern "C" int llm_gemm_skinny_rope_bf16(const void* X, const float* norm_x, con
   a.rope.rot_dim = rot_dim;
   a.rope.write_kv = write_kv;
   return pick_shape<SK_EPI_ROPE, bf16_t>(a);
+}
+
+// W[N, K] (rows ldw apart) into the layout the skinny product streams best: for every tile of 16
+// rows and every step of 32 elements of K, the 64 fragments of 8 elements in lane order
+// (lane l: row l % 16, elements 8 * (l / 16) .. + 7), so that a wave's load is 1 KiB in a row.
+// Rows and elements past the end are zero.  out holds ceil(N/16) * ceil(K/32) * 512 elements.
+__global__ void pack_weight_kernel(const bf16_t* __restrict__ W, bf16_t* __restrict__ out, int N, int K,
+                                   int ldw) {
+  const int n_steps = (K + 31) / 32;
+  const int t = blockIdx.x, lane = threadIdx.x & 63;
+  const int r = lane & 15, g = lane >> 4;
+  const int n = t * 16 + r;
+  for (int s = blockIdx.y * (blockDim.x >> 6) + (threadIdx.x >> 6); s < n_steps; s += gridDim.y * (blockDim.x >> 6)) {
+    const int k = s * 32 + g * 8;
+    uint4 v = make_uint4(0u, 0u, 0u, 0u);
+    if (n < N && k < K) v = *reinterpret_cast<const uint4*>(W + (size_t)n * ldw + k);   // K is a multiple of 8
+    *reinterpret_cast<uint4*>(out + (((size_t)t * n_steps + s) * 64 + lane) * 8) = v;
+  }
+}
+
+extern "C" int llm_pack_weight(const void* W, void* out, int N, int K, int ldw, hipStream_t stream) {
+  if (N <= 0 || K <= 0) return LLM_OK;
+  if ((K & 7) || ldw < K || (ldw & 7) || ((((uintptr_t)W) | ((uintptr_t)out)) & 15)) return LLM_ERR_ARG;
+  const int tiles = (N + 15) / 16;
+  dim3 grid(tiles, 8);
+  pack_weight_kernel<<<grid, 256, 0, stream>>>((const bf16_t*)W, (bf16_t*)out, N, K, ldw);
+  return llm_launch_status();
 }

@@ -85,6 +85,9 @@ class DecoderModel:
                     part.bind({}, ops, dtype)
         self.embed_table = tensors[s.embedding.tensor]
         self.head_weight = self.embed_table if s.head.tied else tensors[s.head.tensor]
+        self.head_prepared = self.head_weight
+        if hasattr(ops, "prepare_weight"):
+            self.head_prepared = ops.prepare_weight(self.head_weight)
 
     # ---- what the cache has to hold
     def cache_needs(self):
@@ -121,7 +124,7 @@ class DecoderModel:
         if want_rows is None or want_rows.numel() == 0:
             return None
         h = self.final_norm.add_norm(ctx, stream, rows=want_rows, lazy=True)
-        return ctx.ops.linear(h, self.head_weight, None, torch.float32)
+        return ctx.ops.linear(h, self.head_prepared, None, torch.float32)
 
 
 def declared_weights(spec: ModelSpec) -> Dict[str, WeightDecl]:

@@ -37,6 +37,7 @@ _SIGNATURES = {
                           _vp, _i, _i, _i, _i, _vp],
     "llm_gemm_skinny_rope_bf16": [_vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _i,
                                   _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _vp],
+    "llm_pack_weight": [_vp, _vp, _i, _i, _i, _vp],
     "llm_gemm_f32": [_vp, _vp, _vp, _i, _i, _i, _vp],
     "llm_attention_ref": [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
                           _f, _i, _vp],
@@ -64,6 +65,15 @@ class NormedRows:
         self.n_rows = res.shape[0] if rows is None else rows.shape[0]
 
 
+class PreparedWeight:
+    """A weight matrix ``w`` and its copy ``tiled`` for the matrix cores: what
+    ``HipOps.prepare_weight`` returns and every product takes in place of the matrix."""
+
+    def __init__(self, w, tiled):
+        self.w, self.tiled = w, tiled
+        self.shape, self.dtype = w.shape, w.dtype
+
+
 class HipOps:
     supports_graphs = True
 
@@ -83,6 +93,7 @@ class HipOps:
             fn.restype = _i
         torch.backends.cuda.matmul.allow_tf32 = False
         self.fast_attention = True
+        self.pack_weights = True
         self.fast_gemm = True
 
     # ---- helpers
@@ -165,6 +176,37 @@ class HipOps:
     DECODE_BLOCKS = 4096    # blocks of the decode attention grid beyond which sequences are not split further
     _EPI_NONE, _EPI_SWIGLU, _EPI_ACCUM = 0, 1, 2
 
+    def prepare_weight(self, w: torch.Tensor, like=None):
+        """Called once for a weight matrix that products will stream many times.  Returns what
+        the products take in place of ``w``: ``w`` itself, or a record that holds, beside ``w``,
+        a copy tiled for the matrix cores, which the products for few rows read instead (a wave
+        then loads 1 KiB in a row rather than 16 pieces of 64 bytes); the library product for
+        many rows goes on reading ``w``.  ``like``: the record of a matrix of which ``w`` is the
+        leading rows (a multiple of 16 of them); its tiled copy then serves ``w`` too."""
+        if isinstance(like, PreparedWeight) and w.shape[0] % 16 == 0 and w.data_ptr() == like.w.data_ptr() \
+                and w.shape[1] == like.w.shape[1] and w.shape[0] <= like.w.shape[0]:
+            return PreparedWeight(w, like.tiled)
+        if (not self.pack_weights or w.dtype != torch.bfloat16 or w.dim() != 2 or w.shape[1] % 8
+                or w.stride(1) != 1 or w.stride(0) % 8 or w.data_ptr() % 16 or w.device != self.device):
+            return w
+        n, k = w.shape
+        tiled = torch.empty((-(-n // 16) * -(-k // 32) * 512,), dtype=torch.bfloat16, device=self.device)
+        self._check(self.lib.llm_pack_weight(w.data_ptr(), tiled.data_ptr(), n, k, w.stride(0),
+                                             self._stream()), "pack_weight")
+        return PreparedWeight(w, tiled)
+
+    @staticmethod
+    def _plain(w):
+        return w.w if isinstance(w, PreparedWeight) else w
+
+    @staticmethod
+    def _streamed(w):
+        """(pointer, row stride) the skinny product reads a weight through: its tiled copy if it
+        has one (row stride 0 says so), else the matrix itself."""
+        if isinstance(w, PreparedWeight):
+            return w.tiled.data_ptr(), 0
+        return w.data_ptr(), w.stride(0)
+
     def normed(self, res, weight, eps, rows=None):
         """Rows of the float32 stream ``res`` that are to be RMS-normalised: a record that
         ``linear`` and ``linear_swiglu`` take in place of a matrix, fusing the norm into the
@@ -177,6 +219,7 @@ class HipOps:
         return x
 
     def _skinny_ok(self, x, w, m, k):
+        w = self._plain(w)
         if not (self.fast_gemm and w.dtype == torch.bfloat16 and k % 8 == 0 and w.data_ptr() % 16 == 0
                 and w.stride(0) % 8 == 0):
             return False
@@ -196,9 +239,10 @@ class HipOps:
         else:
             xp, nx, nw, eps, rows = x.data_ptr() + m0 * k * 2, None, None, 0.0, None
         width = n // 2 if epilogue == self._EPI_SWIGLU else n
+        wptr, ldw = self._streamed(w)
         self._check(self.lib.llm_gemm_skinny_bf16(
-            xp, nx, nw, eps, rows, w.data_ptr(), out.data_ptr() + m0 * width * out.element_size(),
-            epilogue, _code(out.dtype), mm, n, k, w.stride(0), self._stream()), "gemm_skinny_bf16")
+            xp, nx, nw, eps, rows, wptr, out.data_ptr() + m0 * width * out.element_size(),
+            epilogue, _code(out.dtype), mm, n, k, ldw, self._stream()), "gemm_skinny_bf16")
 
     def linear(self, x, w, bias, out_dtype, residual=None):
         """x W^T (+ bias) as ``out_dtype``.  ``x`` is a matrix or a ``normed`` record.  With
@@ -210,7 +254,7 @@ class HipOps:
         n, k2 = w.shape
         if k != k2:
             raise KernelError("linear: x is [%d, %d] but the weight is [%d, %d]" % (m, k, n, k2))
-        self._weight(w, "linear weight")
+        self._weight(self._plain(w), "linear weight")
         if lazy:
             self._dev(x.res, "residual stream", torch.float32)
             self._dev(x.weight, "norm weight", torch.float32, (k,))
@@ -233,6 +277,7 @@ class HipOps:
             x = self._materialise(x, torch.float32 if w.dtype == torch.float32 else torch.bfloat16)
             if self._skinny_ok(x, w, m, k) and bias is None:
                 return self.linear(x, w, None, out_dtype, residual)
+        w = self._plain(w)
         if w.dtype == torch.float32:
             if w.stride(0) != k:
                 raise KernelError("linear: a float32 weight must be contiguous")
@@ -265,7 +310,7 @@ class HipOps:
             raise KernelError("linear_swiglu: x is [%d, %d] but the weight is %s" % (m, k, tuple(w.shape)))
         if (self._skinny_ok(x, w, m, k) and m <= self.SKINNY_ROWS and inter % 16 == 0
                 and dtype == torch.bfloat16):
-            self._weight(w, "linear weight")
+            self._weight(self._plain(w), "linear weight")
             out = torch.empty((m, inter), dtype=torch.bfloat16, device=self.device)
             self._skinny(x, w, out, self._EPI_SWIGLU, 0, m)
             return out
@@ -306,7 +351,7 @@ class HipOps:
         if fused and lazy and not (m <= self.NORM_ROWS and n <= self.NORM_COLS):
             x, lazy = self._materialise(x, dtype), False
         if fused and self._skinny_ok(x, w, m, k):
-            self._weight(w, "qkv weight")
+            self._weight(self._plain(w), "qkv weight")
             cptr = sptr = None
             if rot_dim:
                 if cos is None or cos.shape[1] != rot_dim // 2 or cos.shape != sin.shape:
@@ -334,8 +379,9 @@ class HipOps:
             else:
                 xp, nx, nw, eps, rows = self._dev(x, "qkv input", torch.bfloat16), None, None, 0.0, None
             q = torch.empty((m, n_heads * hd), dtype=torch.bfloat16, device=self.device)
+            wptr, ldw = self._streamed(w)
             self._check(self.lib.llm_gemm_skinny_rope_bf16(
-                xp, nx, nw, eps, rows, w.data_ptr(), bptr, q.data_ptr(), m, k, w.stride(0), n_heads, n_kv, hd,
+                xp, nx, nw, eps, rows, wptr, bptr, q.data_ptr(), m, k, ldw, n_heads, n_kv, hd,
                 cptr, sptr, rot_dim, ctx.tok_pos.data_ptr(), ctx.tok_seq.data_ptr(),
                 ctx.seq_slot.data_ptr(), tptr, stride, kptr, vptr, 64, 1 if write else 0,
                 self._stream()), "gemm_skinny_rope_bf16")

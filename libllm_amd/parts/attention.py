@@ -98,10 +98,10 @@ class Attention(Mixer):
             w = w[order]
             if bias is not None:
                 bias = bias[order].contiguous()
-        self.qkv.bind(w)
-        self.q_only.bind(self.qkv.weight[:self.q_dim])    # the same storage, the q rows alone
+        self.qkv.bind(w, ops=ops)
+        self.q_only.bind(self.qkv.weight[:self.q_dim], ops=ops, like=self.qkv.prepared)    # the same storage
         self.bias = bias                                 # added inside the rotation kernel
-        self.out.bind(tensors[s.o_name + ".weight"])
+        self.out.bind(tensors[s.o_name + ".weight"], ops=ops)
         self.cos, self.sin = self.position.tables(w.device)
 
     def _pair_order(self, device):
@@ -121,7 +121,7 @@ class Attention(Mixer):
         kv = ctx.kv(entry.cache)
         proj = self.qkv if entry.writes else self.q_only
         if hasattr(ctx.ops, "qkv_rope"):
-            qkv = ctx.ops.qkv_rope(x, proj.weight, self.bias, s.n_heads, s.n_kv_heads, s.head_dim,
+            qkv = ctx.ops.qkv_rope(x, proj.prepared, self.bias, s.n_heads, s.n_kv_heads, s.head_dim,
                                    self.cos, self.sin, self.position.rot_dim, ctx, kv, entry.writes,
                                    self.adjacent, ctx.dtype)
         else:

@@ -50,9 +50,9 @@ class SwiGLU(FeedForward):
         gate, up = tensors[s.gate_name + ".weight"], tensors[s.up_name + ".weight"]
         if gate.dtype != up.dtype:
             gate, up = gate.float(), up.float()
-        self.gate_up.bind(torch.cat([gate, up], dim=0))
-        self.down.bind(tensors[s.down_name + ".weight"])
+        self.gate_up.bind(torch.cat([gate, up], dim=0), ops=ops)
+        self.down.bind(tensors[s.down_name + ".weight"], ops=ops)
 
     def forward(self, ctx: StepContext, x, residual=None):
-        h = ctx.ops.linear_swiglu(x, self.gate_up.weight, ctx.dtype)
+        h = ctx.ops.linear_swiglu(x, self.gate_up.prepared, ctx.dtype)
         return self.down(ctx, h, residual=residual)

@@ -172,6 +172,38 @@ def test_gemm_skinny_refuses(ops):
     assert st == 1                                        # refused, not wrong
 
 
+@pytest.mark.parametrize("nk", [(16, 8), (300, 520), (2050, 264), (3072, 2048), (40, 4104)])
+def test_prepared_weight_gives_the_same_bits(ops, nk):
+    """The copy tiled for the matrix cores holds the same numbers: every product for few rows
+    returns the same bits from it as from the matrix, and the product for many rows reads the matrix."""
+    from libllm_amd.hip.ops import PreparedWeight
+    n, k = nk
+    w = rnd((n, k), torch.bfloat16, 60).cuda()
+    pw = ops.prepare_weight(w)
+    assert isinstance(pw, PreparedWeight) and tuple(pw.shape) == (n, k)
+    for m in (1, 9, 40, 130):
+        x = rnd((m, k), torch.bfloat16, 61).cuda()
+        for out_dtype in DTYPES:
+            assert torch.equal(ops.linear(x, pw, None, out_dtype), ops.linear(x, w, None, out_dtype))
+    x = rnd((9, k), torch.bfloat16, 61).cuda()
+    a, b = torch.ones((9, n), device="cuda"), torch.ones((9, n), device="cuda")
+    ops.linear(x, pw, None, torch.bfloat16, residual=a)
+    ops.linear(x, w, None, torch.bfloat16, residual=b)
+    assert torch.equal(a, b)
+    if n % 32 == 0:
+        assert torch.equal(ops.linear_swiglu(x, pw), ops.linear_swiglu(x, w))
+        head = w[:n // 2]                                   # the leading rows share the tiled copy
+        ph = ops.prepare_weight(head, like=pw)
+        assert ph.tiled is pw.tiled
+        assert torch.equal(ops.linear(x, ph, None, torch.float32), ops.linear(x, head.contiguous(), None, torch.float32))
+    stream = rnd((9, k), torch.float32, 62, 3.0).cuda()
+    wn = (1.0 + 0.2 * rnd((k,), torch.float32, 63)).cuda()
+    lazy = ops.normed(stream, wn, 1e-5)
+    assert torch.equal(ops.linear(lazy, pw, None, torch.bfloat16), ops.linear(lazy, w, None, torch.bfloat16))
+    w32 = rnd((24, 40), torch.float32, 64).cuda()
+    assert ops.prepare_weight(w32) is w32                   # a 32-bit matrix is left as it is
+
+
 def test_weight_rows_may_lie_apart(ops):
     """A weight that is a view of some columns of a wider matrix: the same bits from every product."""
     w = rnd((300, 1024), torch.bfloat16, 50).cuda()
