@@ -69,7 +69,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   constexpr int CK = 512 * G;                    // elements of K per chunk
   constexpr int ROW_B = CK * 2;                  // bytes of a staged row; 16-byte pieces are swizzled
   constexpr int X_BYTES = 16 * MT * ROW_B;
-  constexpr int RED_BYTES = SK_WK * WN * RT * MT * 1024;
+  constexpr int RED_BYTES = SK_WK * WN * ((EPI == SK_EPI_SWIGLU) ? 2 : 1) * MT * 1024;
   constexpr int LDS_BYTES = X_BYTES > RED_BYTES ? X_BYTES : RED_BYTES;
   constexpr int XV = CK / 8;                     // 16-byte pieces of a staged row
   constexpr int ROWS_PASS = NT / XV;             // rows staged per pass of the block
@@ -233,23 +233,28 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
     }
   }
 
-  // ---- add the partial sums of the 8 waves in order, apply the epilogue, store
+  // ---- add the partial sums of the 8 waves in order, apply the epilogue, store: one output tile
+  // of every row group a round (a gate and its up tile together), so that the buffer stays small
   float* red = reinterpret_cast<float*>(lds);
+  constexpr int RPR = (EPI == SK_EPI_SWIGLU) ? 2 : 1;    // W tiles of a row group per round
+  constexpr int OUT_RT = RT / RPR;
+  constexpr int ITEMS = WN * MT * 64;
+  const int ldc = (EPI == SK_EPI_SWIGLU) ? n_out : N;
 #pragma unroll
-  for (int rt = 0; rt < RT; ++rt)
+  for (int ort = 0; ort < OUT_RT; ++ort) {
+  if (ort > 0) __syncthreads();                          // the round before has been read
+#pragma unroll
+  for (int j = 0; j < RPR; ++j)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt)
-      *reinterpret_cast<float4*>(red + ((((wk * WN + wn) * RT + rt) * MT + mt) * 64 + lane) * 4) =
-          make_float4(acc[rt][mt][0], acc[rt][mt][1], acc[rt][mt][2], acc[rt][mt][3]);
+      *reinterpret_cast<float4*>(red + ((((wk * WN + wn) * RPR + j) * MT + mt) * 64 + lane) * 4) =
+          make_float4(acc[ort * RPR + j][mt][0], acc[ort * RPR + j][mt][1], acc[ort * RPR + j][mt][2],
+                      acc[ort * RPR + j][mt][3]);
   __syncthreads();
-  constexpr int OUT_RT = (EPI == SK_EPI_SWIGLU) ? RT / 2 : RT;
-  constexpr int ITEMS = WN * OUT_RT * MT * 64;
-  const int ldc = (EPI == SK_EPI_SWIGLU) ? n_out : N;
   for (int it = tid; it < ITEMS; it += NT) {
     const int ln = it & 63;
     const int mt = (it >> 6) % MT;
-    const int ort = (it / (64 * MT)) % OUT_RT;
-    const int w_n = it / (64 * MT * OUT_RT);
+    const int w_n = it / (64 * MT);
     float v[4];
     int n;
     if (EPI == SK_EPI_SWIGLU) {
@@ -257,9 +262,9 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
 #pragma unroll
       for (int w = 0; w < SK_WK; ++w) {
         const float4 pg = *reinterpret_cast<const float4*>(
-            red + ((((w * WN + w_n) * RT + 2 * ort) * MT + mt) * 64 + ln) * 4);
+            red + ((((w * WN + w_n) * RPR + 0) * MT + mt) * 64 + ln) * 4);
         const float4 pu = *reinterpret_cast<const float4*>(
-            red + ((((w * WN + w_n) * RT + 2 * ort + 1) * MT + mt) * 64 + ln) * 4);
+            red + ((((w * WN + w_n) * RPR + 1) * MT + mt) * 64 + ln) * 4);
         gsum[0] += pg.x; gsum[1] += pg.y; gsum[2] += pg.z; gsum[3] += pg.w;
         usum[0] += pu.x; usum[1] += pu.y; usum[2] += pu.z; usum[3] += pu.w;
       }
@@ -275,7 +280,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
 #pragma unroll
       for (int w = 0; w < SK_WK; ++w) {
         const float4 p = *reinterpret_cast<const float4*>(
-            red + ((((w * WN + w_n) * RT + ort) * MT + mt) * 64 + ln) * 4);
+            red + (((w * WN + w_n) * MT + mt) * 64 + ln) * 4);
         sum[0] += p.x; sum[1] += p.y; sum[2] += p.z; sum[3] += p.w;
       }
       const float scale = XNORM ? s_inv[mt * 16 + (ln & 15)] : 1.0f;
@@ -351,6 +356,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
         if (n + e < ldc) Conv<OutT>::store(dst + e, v[e]);
     }
   }
+  }
 }
 
 struct SkinnyArgs {
@@ -374,6 +380,18 @@ static int launch_skinny(const SkinnyArgs& a) {
   return llm_launch_status();
 }
 
+template <int MT, int EPI, typename OutT>
+static int pick_rows(const SkinnyArgs& a) {
+  if constexpr (EPI == SK_EPI_SWIGLU) {
+    if (a.n_out >= 8192) return launch_skinny<MT, 4, 1, 1, EPI, false, OutT>(a);
+    return launch_skinny<MT, 2, 1, 1, EPI, false, OutT>(a);
+  } else {
+    if (a.N >= 8192) return launch_skinny<MT, 2, 2, 1, EPI, false, OutT>(a);
+    if (a.N >= 6144) return launch_skinny<MT, 2, 1, 1, EPI, false, OutT>(a);
+    return launch_skinny<MT, 1, 1, 1, EPI, false, OutT>(a);
+  }
+}
+
 template <int EPI, typename OutT>
 static int pick_shape(const SkinnyArgs& a) {
   constexpr int RT = (EPI == SK_EPI_SWIGLU) ? 2 : 1;
@@ -388,16 +406,11 @@ static int pick_shape(const SkinnyArgs& a) {
       // a long K with few rows of W: more of each row in flight per wave
       if (RT == 1 && a.K >= 4096 && a.N <= 4096) return launch_skinny<1, RT, 1, 4, EPI, false, OutT>(a);
       return launch_skinny<1, RT, 1, 2, EPI, false, OutT>(a);
-    // two row groups per block only where W has rows enough to fill the GPU with such blocks
-    case 2:
-      if (RT == 1 && a.N < 8192) return launch_skinny<2, 1, 1, 1, EPI, false, OutT>(a);
-      return launch_skinny<2, RT, 2 / RT, 1, EPI, false, OutT>(a);
-    case 3:
-      if (RT == 1 && a.N < 8192) return launch_skinny<3, 1, 1, 1, EPI, false, OutT>(a);
-      return launch_skinny<3, RT, 2 / RT, 1, EPI, false, OutT>(a);
-    case 4:
-      if (RT == 1 && a.N < 8192) return launch_skinny<4, 1, 1, 1, EPI, false, OutT>(a);
-      return launch_skinny<4, RT, 2 / RT, 1, EPI, false, OutT>(a);
+    // More rows of W per block where W has rows enough to fill the GPU with such blocks: the rows
+    // of X are then staged once for 64 rows of W instead of 16.
+    case 2: return pick_rows<2, EPI, OutT>(a);
+    case 3: return pick_rows<3, EPI, OutT>(a);
+    case 4: return pick_rows<4, EPI, OutT>(a);
   }
   return LLM_ERR_ARG;
 }
