@@ -128,6 +128,47 @@ def build(force: bool = True, verbose: bool = True) -> str:
     return os.path.join(target, LIB_NAME)
 
 
+CAPI_NAME = "libllm.so"
+
+
+def build_capi(force: bool = True, verbose: bool = True) -> str:
+    """Compiles the C API (csrc/capi: host code only, against this interpreter's headers and
+    library) and returns the path of libllm.so."""
+    import sysconfig
+    src = os.path.join(CSRC, "capi", "llm_capi.cc")
+    h = hashlib.sha256()
+    for path in (src, os.path.join(CSRC, "capi", "llm.h")):
+        with open(path, "rb") as f:
+            h.update(f.read())
+    want = h.hexdigest()[:20]
+    for d in _lib_dirs():
+        so, stamp = os.path.join(d, CAPI_NAME), os.path.join(d, CAPI_NAME + ".hash")
+        if not force and os.path.isfile(so) and os.path.isfile(stamp) and open(stamp).read().strip() == want:
+            return so
+    cxx = os.environ.get("CXX") or shutil.which("g++") or shutil.which("c++") or _hipcc()
+    if cxx is None:
+        raise KernelError("the C API is not built and no C++ compiler was found")
+    target = next((d for d in _lib_dirs() if _writable(d)), None)
+    if target is None:
+        raise KernelError("no writable folder for the C API library (tried %s)" % ", ".join(_lib_dirs()))
+    root = os.path.dirname(os.path.dirname(_HERE))
+    libdir = sysconfig.get_config_var("LIBDIR") or "/usr/lib"
+    pylib = "python" + sysconfig.get_config_var("LDVERSION")
+    tmp_so = os.path.join(target, CAPI_NAME + ".tmp-%d" % os.getpid())
+    cmd = [cxx, "-O2", "-fPIC", "-shared", "-std=c++17", "-I", sysconfig.get_paths()["include"],
+           "-DLIBLLM_AMD_ROOT=\"%s\"" % root, src, "-o", tmp_so,
+           "-L", libdir, "-Wl,-rpath," + libdir, "-l" + pylib, "-ldl"]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise KernelError("compiling the C API failed:\n%s" % proc.stdout[-4000:])
+    os.replace(tmp_so, os.path.join(target, CAPI_NAME))
+    with open(os.path.join(target, CAPI_NAME + ".hash"), "w") as f:
+        f.write(want)
+    if verbose:
+        _say("built %s" % CAPI_NAME)
+    return os.path.join(target, CAPI_NAME)
+
+
 def load() -> ctypes.CDLL:
     """The kernel library; built first if no current build exists."""
     global _lib
