@@ -283,6 +283,108 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride, const 
   }
 }
 
+// The same for bfloat16 with neighbouring pairs, a tile of 64 rows and one head per block
+// (grid: row tiles x (q heads + k heads + v heads)).  q and k move as 16-byte vectors (four pairs
+// and their four angles at a time).  v is transposed through LDS, so that consecutive lanes write
+// consecutive positions of a page: rows of a prompt lie in order, and a wave's 64 stores of two
+// bytes then fall into one line instead of 64.  Needs hd and rot_dim in multiples of 8.
+template <int PAGE>
+__global__ __launch_bounds__(256) void rope_kv_write_tile_kernel(
+    bf16_t* __restrict__ qkv, int row_stride, const float* __restrict__ bias, int n_heads, int n_kv, int hd,
+    const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot_dim,
+    const int* __restrict__ tok_pos, const int* __restrict__ tok_seq, const int* __restrict__ seq_slot,
+    const int* __restrict__ table, int table_stride, bf16_t* __restrict__ k_pages,
+    bf16_t* __restrict__ v_pages, int M) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char tile_raw[];
+  __shared__ int s_pos[64], s_page[64];
+  const int tid = threadIdx.x, m0 = blockIdx.x * 64, h = blockIdx.y;
+  const bool is_q = h < n_heads, is_k = !is_q && h < n_heads + n_kv;
+  if (tid < 64) {
+    const int m = m0 + tid;
+    int pos = 0, page = 0;
+    if (m < M) {
+      pos = tok_pos[m];
+      if (!is_q) page = table[(size_t)seq_slot[tok_seq[m]] * table_stride + pos / PAGE];
+    }
+    s_pos[tid] = pos;
+    s_page[tid] = page;
+  }
+  __syncthreads();
+  const int vecs = hd / 8, half = rot_dim / 2;
+  const float* b = bias ? bias + (size_t)h * hd : nullptr;
+  if (is_q || is_k) {
+    for (int it = tid; it < 64 * vecs; it += 256) {
+      const int r = it / vecs, d = (it % vecs) * 8, m = m0 + r;
+      if (m >= M) continue;
+      bf16_t* src = qkv + (size_t)m * row_stride + (size_t)h * hd + d;
+      const uint4 raw = *reinterpret_cast<const uint4*>(src);
+      const uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+      float x[8];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        x[2 * e] = bf16_to_f32((bf16_t)(w[e] & 0xffffu));
+        x[2 * e + 1] = bf16_to_f32((bf16_t)(w[e] >> 16));
+      }
+      if (b) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) x[e] += b[d + e];
+      }
+      const int pos = s_pos[r];
+      if (d < rot_dim) {
+        const float4 c4 = *reinterpret_cast<const float4*>(cos_t + (size_t)pos * half + d / 2);
+        const float4 s4 = *reinterpret_cast<const float4*>(sin_t + (size_t)pos * half + d / 2);
+        const float c[4] = {c4.x, c4.y, c4.z, c4.w}, sn[4] = {s4.x, s4.y, s4.z, s4.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float x1 = x[2 * e], x2 = x[2 * e + 1];
+          x[2 * e] = x1 * c[e] - x2 * sn[e];
+          x[2 * e + 1] = x2 * c[e] + x1 * sn[e];
+        }
+      }
+      uint4 out;
+      out.x = (uint32_t)f32_to_bf16(x[0]) | ((uint32_t)f32_to_bf16(x[1]) << 16);
+      out.y = (uint32_t)f32_to_bf16(x[2]) | ((uint32_t)f32_to_bf16(x[3]) << 16);
+      out.z = (uint32_t)f32_to_bf16(x[4]) | ((uint32_t)f32_to_bf16(x[5]) << 16);
+      out.w = (uint32_t)f32_to_bf16(x[6]) | ((uint32_t)f32_to_bf16(x[7]) << 16);
+      bf16_t* dst = is_q ? src
+                         : k_pages + (((size_t)s_page[r] * n_kv + (h - n_heads)) * PAGE + pos % PAGE) * hd + d;
+      *reinterpret_cast<uint4*>(dst) = out;
+    }
+    return;
+  }
+  // a v head: rows of the tile into LDS (a row takes hd + 2 values, an odd number of words, so that
+  // a column is read without bank conflicts), then one dim a wave at a time, a row a lane
+  const int kvh = h - n_heads - n_kv;
+  uint32_t* tile = reinterpret_cast<uint32_t*>(tile_raw);
+  const int row_w = hd / 2 + 1;                                    // words per row of the tile
+  for (int it = tid; it < 64 * vecs; it += 256) {
+    const int r = it / vecs, d = (it % vecs) * 8, m = m0 + r;
+    uint4 raw = make_uint4(0u, 0u, 0u, 0u);
+    if (m < M) raw = *reinterpret_cast<const uint4*>(qkv + (size_t)m * row_stride + (size_t)h * hd + d);
+    uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
+    if (b) {
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float lo = bf16_to_f32((bf16_t)(w[e] & 0xffffu)) + b[d + 2 * e];
+        const float hi = bf16_to_f32((bf16_t)(w[e] >> 16)) + b[d + 2 * e + 1];
+        w[e] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
+      }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) tile[r * row_w + d / 2 + e] = w[e];
+  }
+  __syncthreads();
+  const int lane = tid & 63, wave = tid >> 6;
+  if (m0 + lane < M) {
+    const int pos = s_pos[lane];
+    bf16_t* dst = v_pages + ((size_t)s_page[lane] * n_kv + kvh) * hd * PAGE + pos % PAGE;
+    for (int d = wave; d < hd; d += 4) {
+      const uint32_t w = tile[lane * row_w + d / 2];
+      dst[(size_t)d * PAGE] = (bf16_t)((d & 1) ? (w >> 16) : (w & 0xffffu));
+    }
+  }
+}
+
 extern "C" int llm_rope_kv_write(void* qkv, int dtype, int row_stride, const float* bias, int n_heads,
                                  int n_kv, int hd, const float* cos_t, const float* sin_t, int rot_dim,
                                  const int* tok_pos, const int* tok_seq, const int* seq_slot,
@@ -297,6 +399,18 @@ extern "C" int llm_rope_kv_write(void* qkv, int dtype, int row_stride, const flo
   const int width = (n_heads + (write_kv ? 2 * n_kv : 0)) * hd;
   if (row_stride < width) return LLM_ERR_ARG;
   if (write_kv && (!k_pages || !v_pages || !table || !seq_slot || !tok_seq)) return LLM_ERR_ARG;
+  const bool vec_ok = dtype == LLM_DTYPE_BF16 && (adjacent || rot_dim == 0) && hd % 8 == 0 && hd <= 256 &&
+                      rot_dim % 8 == 0 && row_stride % 8 == 0 && ((uintptr_t)qkv & 15) == 0 &&
+                      ((uintptr_t)cos_t & 15) == 0 && ((uintptr_t)sin_t & 15) == 0 &&
+                      (!write_kv || ((uintptr_t)k_pages & 15) == 0) && M >= 64;
+  if (vec_ok) {
+    const dim3 grid((M + 63) / 64, n_heads + (write_kv ? 2 * n_kv : 0));
+    const size_t lds = write_kv ? (size_t)64 * (hd / 2 + 1) * 4 : 0;
+    rope_kv_write_tile_kernel<64><<<grid, 256, lds, stream>>>(
+        (bf16_t*)qkv, row_stride, bias, n_heads, n_kv, hd, cos_t, sin_t, rot_dim, tok_pos, tok_seq, seq_slot,
+        table, table_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, M);
+    return llm_launch_status();
+  }
   if (dtype == LLM_DTYPE_F32)
     rope_kv_write_kernel<float, 64><<<M, 256, 0, stream>>>(
         (float*)qkv, row_stride, bias, n_heads, n_kv, hd, cos_t, sin_t, rot_dim, tok_pos, tok_seq,

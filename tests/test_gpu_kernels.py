@@ -423,6 +423,58 @@ def test_projection_with_rotation_and_cache_write(ops, dtype, shape, bias, seqs)
     assert torch.count_nonzero(kv.k_pages) == 0
 
 
+@pytest.mark.parametrize("shape", [(4, 2, 16, 16), (6, 3, 48, 24), (5, 1, 64, 64), (8, 2, 128, 128), (2, 2, 256, 64),
+                                   (3, 1, 32, 0)])
+@pytest.mark.parametrize("bias", [False, True])
+def test_rope_kv_write_on_many_rows(ops, shape, bias):
+    """Prompts of many rows in bfloat16 with neighbouring pairs take a kernel of their own (tiles
+    of 64 rows, v transposed through LDS): several sequences that cross page borders, a last tile
+    that is not full, partial rotation; and nothing beside the new positions is written."""
+    n_heads, n_kv, hd, rot = shape
+    dtype = torch.bfloat16
+    seqs = [(2, 0, 70), (0, 61, 9), (1, 130, 50), (3, 5, 31)]      # 160 rows: two tiles and a half
+    ctx = make_ctx(ops, dtype, seqs)
+    m = ctx.n_tokens
+    width = (n_heads + 2 * n_kv) * hd
+    nat = rnd((m, width), dtype, 50)                                # rows in their natural order
+    b_nat = rnd((width,), torch.float32, 51) if bias else None
+    order = pair_order(n_heads, n_kv, hd, rot) if rot else torch.arange(width)
+    head_order = order[:hd]
+    half = rot // 2
+    inv = 1.0 / (10000.0 ** (torch.arange(0, rot, 2, dtype=torch.float64) / max(rot, 1)))
+    ang = torch.arange(300, dtype=torch.float64)[:, None] * inv[None, :]
+    cos, sin = (torch.cos(ang).float().cuda(), torch.sin(ang).float().cuda()) if rot else (None, None)
+    x = nat.double() + (b_nat.double() if bias else 0)
+    pos = ctx.tok_pos.cpu().long()
+    heads = x[:, :(n_heads + n_kv) * hd].reshape(m, n_heads + n_kv, hd).clone()
+    if rot:
+        c, s_ = torch.cos(ang)[pos][:, None, :], torch.sin(ang)[pos][:, None, :]
+        x1, x2 = heads[..., :half].clone(), heads[..., half:rot].clone()
+        heads[..., :half] = x1 * c - x2 * s_
+        heads[..., half:rot] = x2 * c + x1 * s_
+    v_ref = x[:, (n_heads + n_kv) * hd:].reshape(m, n_kv, hd)
+    for write in (True, False):
+        kv = make_kv("cuda", dtype, 4, 4, n_kv, hd, seed=1)
+        cols = width if write else n_heads * hd                     # queries alone when nothing is written
+        qkv = nat[:, order][:, :cols].contiguous().cuda()
+        bd = b_nat[order][:cols].contiguous().cuda() if bias else None
+        ops.rope_kv_write(qkv, bd, n_heads, n_kv, hd, cos, sin, rot, ctx, kv, write, adjacent=bool(rot))
+        q = qkv[:, :n_heads * hd].reshape(m, n_heads, hd)
+        assert close(q, heads[:, :n_heads][..., head_order], dtype)
+        if not write:
+            assert torch.count_nonzero(kv.k_pages) == 0 and torch.count_nonzero(kv.v_pages) == 0
+            continue
+        o = 0
+        for slot, p0, n_new in seqs:
+            k_got, v_got = read_kv(kv, slot, p0 + n_new)
+            assert close(k_got[p0:], heads[o:o + n_new, n_heads:][..., head_order], dtype)
+            assert close(v_got[p0:], v_ref[o:o + n_new], dtype)
+            assert torch.count_nonzero(k_got[:p0]) == 0 and torch.count_nonzero(v_got[:p0]) == 0
+            o += n_new
+        written = sum(n for _, _, n in seqs) * n_kv * hd
+        assert torch.count_nonzero(kv.k_pages) <= written and torch.count_nonzero(kv.v_pages) <= written
+
+
 def test_rope_pairing_and_sign(ops):
     # a unit vector in dimension 0 at position p becomes cos at 0 and +sin at hd/2:
     # o[j] = x[j] c - x[j+hd/2] s, o[j+hd/2] = x[j+hd/2] c + x[j] s   (src/libllm/llama.cc:151-176)
