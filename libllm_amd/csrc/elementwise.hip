@@ -148,25 +148,36 @@ __global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, i
 
 // The same for bfloat16 rows whose half width is a multiple of 8: 16 bytes of gate and of up per
 // thread, any number of rows through a grid-stride loop.
+__device__ __forceinline__ uint4 silu_mul_8(const uint4 g4, const uint4 u4) {
+  const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
+  uint32_t ow[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
+    const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
+    const float r0 = u0 * g0 / (1.0f + expf(-g0)), r1 = u1 * g1 / (1.0f + expf(-g1));
+    ow[j] = (uint32_t)f32_to_bf16(r0) | ((uint32_t)f32_to_bf16(r1) << 16);
+  }
+  return make_uint4(ow[0], ow[1], ow[2], ow[3]);
+}
+
+// Two vectors a thread and round (the second half a grid apart), all four loads asked for before
+// the first is used.
 __global__ void silu_mul_vec_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int I,
                                     size_t total_vec) {
   const int per_row = I / 8;
-  for (size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x; v < total_vec;
-       v += (size_t)gridDim.x * blockDim.x) {
-    const size_t m = v / per_row;
-    const int i = (int)(v % per_row) * 8;
-    const uint4 g4 = *reinterpret_cast<const uint4*>(gu + m * 2 * I + i);
-    const uint4 u4 = *reinterpret_cast<const uint4*>(gu + m * 2 * I + I + i);
-    const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
-    uint32_t ow[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
-      const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
-      const float r0 = u0 * g0 / (1.0f + expf(-g0)), r1 = u1 * g1 / (1.0f + expf(-g1));
-      ow[j] = (uint32_t)f32_to_bf16(r0) | ((uint32_t)f32_to_bf16(r1) << 16);
-    }
-    *reinterpret_cast<uint4*>(out + m * I + i) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+  const size_t span = (size_t)gridDim.x * blockDim.x;
+  for (size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x; v < total_vec; v += 2 * span) {
+    const size_t v2 = v + span;
+    const bool two = v2 < total_vec;
+    const size_t m = v / per_row, m2 = two ? v2 / per_row : m;
+    const int i = (int)(v % per_row) * 8, i2 = two ? (int)(v2 % per_row) * 8 : i;
+    const uint4 ga = *reinterpret_cast<const uint4*>(gu + m * 2 * I + i);
+    const uint4 ua = *reinterpret_cast<const uint4*>(gu + m * 2 * I + I + i);
+    const uint4 gb = *reinterpret_cast<const uint4*>(gu + m2 * 2 * I + i2);
+    const uint4 ub = *reinterpret_cast<const uint4*>(gu + m2 * 2 * I + I + i2);
+    *reinterpret_cast<uint4*>(out + m * I + i) = silu_mul_8(ga, ua);
+    if (two) *reinterpret_cast<uint4*>(out + m2 * I + i2) = silu_mul_8(gb, ub);
   }
 }
 
@@ -175,8 +186,9 @@ extern "C" int llm_silu_mul(const void* gu, void* out, int dtype, int M, int I, 
   if (I <= 0 || M > 65535 * 32) return LLM_ERR_ARG;
   if (dtype == LLM_DTYPE_BF16 && I % 8 == 0 && ((((uintptr_t)gu) | ((uintptr_t)out)) & 15) == 0) {
     const size_t total_vec = (size_t)M * (I / 8);
-    size_t blocks = (total_vec + 255) / 256;
+    size_t blocks = (total_vec + 511) / 512;                      // two vectors a thread
     if (blocks > 65536) blocks = 65536;
+    if (blocks == 0) blocks = 1;
     silu_mul_vec_kernel<<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total_vec);
     return llm_launch_status();
   }

@@ -301,6 +301,20 @@ def test_silu_mul_limits(ops):
     assert abs(out[0, 2]) < 1e-10
 
 
+def test_silu_mul_limits_bfloat16_vectors(ops):
+    # the vector kernel computes 1 / (1 + 2^(-g log2 e)) with the hardware's exp2 and reciprocal:
+    # a gate far below zero overflows the power to infinity, and the product must be 0, not NaN
+    gates = [0.0, 30.0, -30.0, 5.0, -100.0, -1000.0, 100.0, 1.0]
+    ups = [3.0, 2.0, 7.0, 11.0, 5.0, 5.0, 0.5, -4.0]
+    gu = torch.tensor([gates + ups], device="cuda", dtype=torch.bfloat16)
+    out = ops.silu_mul(gu).float().cpu()[0]
+    assert torch.isfinite(out).all()
+    assert out[0] == 0.0 and out[2].abs() < 1e-9 and out[4] == 0.0 and out[5] == 0.0
+    assert out[1] == 60.0 and out[6] == 50.0
+    g, u = torch.tensor(gates, dtype=torch.float64), torch.tensor(ups, dtype=torch.float64)
+    assert close(out, g / (1 + torch.exp(-g)) * u, torch.bfloat16)
+
+
 # ------------------------------------------------------------------------------- rotation + cache write
 @pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("shape", [(4, 2, 16, 16), (6, 1, 32, 32), (6, 3, 48, 24), (5, 5, 80, 80), (32, 8, 64, 0)])
