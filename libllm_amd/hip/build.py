@@ -129,21 +129,25 @@ def build(force: bool = True, verbose: bool = True) -> str:
 
 
 CAPI_NAME = "libllm.so"
+CLI_NAME = "llm"                 # the command line over the C API, beside the library
 
 
 def build_capi(force: bool = True, verbose: bool = True) -> str:
     """Compiles the C API (csrc/capi: host code only, against this interpreter's headers and
-    library) and returns the path of libllm.so."""
+    library) and the ``llm`` program over it; returns the path of libllm.so (the program lies
+    beside it)."""
     import sysconfig
     src = os.path.join(CSRC, "capi", "llm_capi.cc")
     h = hashlib.sha256()
-    for path in (src, os.path.join(CSRC, "capi", "llm.h")):
+    main_src = os.path.join(CSRC, "capi", "llm_main.cc")
+    for path in (src, os.path.join(CSRC, "capi", "llm.h"), main_src):
         with open(path, "rb") as f:
             h.update(f.read())
     want = h.hexdigest()[:20]
     for d in _lib_dirs():
         so, stamp = os.path.join(d, CAPI_NAME), os.path.join(d, CAPI_NAME + ".hash")
-        if not force and os.path.isfile(so) and os.path.isfile(stamp) and open(stamp).read().strip() == want:
+        if (not force and os.path.isfile(so) and os.path.isfile(os.path.join(d, CLI_NAME))
+                and os.path.isfile(stamp) and open(stamp).read().strip() == want):
             return so
     cxx = os.environ.get("CXX") or shutil.which("g++") or shutil.which("c++") or _hipcc()
     if cxx is None:
@@ -162,6 +166,13 @@ def build_capi(force: bool = True, verbose: bool = True) -> str:
     if proc.returncode != 0:
         raise KernelError("compiling the C API failed:\n%s" % proc.stdout[-4000:])
     os.replace(tmp_so, os.path.join(target, CAPI_NAME))
+    tmp_exe = os.path.join(target, CLI_NAME + ".tmp-%d" % os.getpid())
+    cmd = [cxx, "-O2", "-std=c++17", "-I", os.path.join(CSRC, "capi"), main_src, "-o", tmp_exe,
+           os.path.join(target, CAPI_NAME), "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + libdir]
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if proc.returncode != 0:
+        raise KernelError("compiling the llm program failed:\n%s" % proc.stdout[-4000:])
+    os.replace(tmp_exe, os.path.join(target, CLI_NAME))
     with open(os.path.join(target, CAPI_NAME + ".hash"), "w") as f:
         f.write(want)
     if verbose:

@@ -80,16 +80,44 @@ def test_sampled_generation_and_stop_tokens(model_b):
     assert [c.token_id for c in chunks if c.token_id is not None] == sampling.generate(cfg, weights, prompts[1], 5)
 
 
-def test_command_line(model_b):
+def programs():
+    """The Python command line and the C++ one over the C API: same flags, same messages."""
+    from libllm_amd.hip import build as hip_build
+    native = os.path.join(os.path.dirname(hip_build.build_capi(force=False, verbose=False)), hip_build.CLI_NAME)
+    return {"python": [sys.executable, os.path.join(ROOT, "bin", "llm")], "native": [native]}
+
+
+@pytest.mark.parametrize("program", ["python", "native"])
+def test_command_line(model_b, program):
     path, cfg, weights = model_b
     prompt = [11, 12, 13, 14]
     want = sampling.generate(cfg, weights, prompt, 6)
-    proc = subprocess.run([sys.executable, os.path.join(ROOT, "bin", "llm"), "chat", "-m", path, "-device", "auto",
-                           "-dtype", "float32", "-ids", "-temperature", "0", "-max_new_tokens", "6"],
+    proc = subprocess.run(programs()[program] + ["chat", "-m", path, "-device", "auto",
+                           "-dtype", "float32", "-ids", "-temperature", "0", "--max-new-tokens", "6"],
                           input=" ".join(map(str, prompt)) + "\n:new\n\n", capture_output=True, text=True, timeout=120)
     assert proc.returncode == 0, proc.stderr
     assert " ".join(map(str, want)) in proc.stdout
     assert "tokens, time=" in proc.stdout and "ms per token" in proc.stdout
+    assert "===== new session =====" in proc.stdout
+
+
+def test_command_lines_agree_on_a_text_session(model_b):
+    """A session in text (bytes as token ids, since the model folder has no tokenizer): a system
+    prompt, quotes, a backslash and characters beyond ASCII in the questions, a second turn that
+    continues the first, a new session.  Both programs print the same, the timing line aside."""
+    path, _, _ = model_b
+    session = ':sys be "brief"\nwhat is C:\\temp?\nund jetzt: \u00e4\u00f6\u00fc \u4e2d\u6587 \U0001f600\n:new\nagain\n'
+    outs = {}
+    for name, cmd in programs().items():
+        proc = subprocess.run(cmd + ["chat", "-m", path, "-dtype", "float32", "-temperature", "0.8", "-top_k", "20",
+                                     "-seed", "5", "-max_new_tokens", "9"],
+                              input=session.encode("utf-8"), capture_output=True, timeout=120)
+        assert proc.returncode == 0, proc.stderr.decode("utf-8", "replace")
+        lines = proc.stdout.decode("utf-8", "replace").splitlines()
+        outs[name] = [l for l in lines if "ms per token" not in l]
+        assert sum("ms per token" in l for l in lines) == 3
+    assert outs["python"] == outs["native"]
+    assert any("===== new session =====" in l for l in outs["native"])
 
 
 def test_smoke_entry():
