@@ -404,7 +404,9 @@ static int pick_shape(const SkinnyArgs& a) {
   switch (mt) {
     case 1:
       // a long K with few rows of W: more of each row in flight per wave
-      if (RT == 1 && a.K >= 4096 && a.N <= 4096) return launch_skinny<1, RT, 1, 4, EPI, false, OutT>(a);
+      if constexpr (RT == 1) {
+        if (a.K >= 4096 && a.N <= 4096) return launch_skinny<1, RT, 1, 4, EPI, false, OutT>(a);
+      }
       return launch_skinny<1, RT, 1, 2, EPI, false, OutT>(a);
     // More rows of W per block where W has rows enough to fill the GPU with such blocks: the rows
     // of X are then staged once for 64 rows of W instead of 16.
