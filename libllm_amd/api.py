@@ -15,7 +15,8 @@ from typing import Iterable, List, Optional, Sequence, Union
 from .cache import PAGE
 from .engine import Generator, StepEntry
 from .errors import ConfigError, RequestError
-from .runtime import load_engine
+from .config import config_from_dir
+from .runtime import load_engine, random_engine
 from .sampling import Sampler, SamplingParams
 
 
@@ -25,6 +26,16 @@ class Device(IntEnum):
     CUDA = 0x0100
     GPU = 0x0100
     AUTO = 0x1f00
+
+
+def parse_device(device) -> Device:
+    """A Device, or its name: cpu, cuda (hip and gpu mean the same) or auto (src/libllm/llm.cc:154-168)."""
+    if isinstance(device, str):
+        names = {"cpu": Device.CPU, "cuda": Device.CUDA, "hip": Device.CUDA, "gpu": Device.CUDA, "auto": Device.AUTO}
+        if device.lower() not in names:
+            raise ConfigError("invalid device name: must be one of \"cpu\", \"cuda\" or \"auto\"")
+        return names[device.lower()]
+    return Device(int(device))
 
 
 class ControlToken:
@@ -96,15 +107,22 @@ class Completion:
 
 
 class Model:
-    def __init__(self, config_file: str, device: Device = Device.AUTO, dtype: str = "bfloat16",
-                 max_tokens: int = 8192, max_batch: int = 64, ops=None, use_graphs: bool = True) -> None:
-        """``config_file``: the model folder, or the config.json inside it."""
-        if int(device) == int(Device.CPU):
+    def __init__(self, config_file: str, device: Union[Device, str] = Device.AUTO, dtype: str = "bfloat16",
+                 max_tokens: int = 8192, max_batch: int = 64, ops=None, use_graphs: bool = True,
+                 random_weights: bool = False, seed: int = 0) -> None:
+        """``config_file``: the model folder, or the config.json inside it.  ``device``: a Device
+        or one of "auto", "cuda", "hip", "cpu".  With ``random_weights`` only config.json is read
+        and every tensor is drawn from ``seed``."""
+        if int(parse_device(device)) == int(Device.CPU):
             raise ConfigError("this library has no CPU path; use Device.AUTO or Device.GPU")
         model_dir = os.path.dirname(config_file) if os.path.isfile(config_file) else config_file
         self.model_dir = model_dir
-        self.engine = load_engine(model_dir, dtype=dtype, max_tokens=max_tokens, ops=ops,
-                                  use_graphs=use_graphs)
+        if random_weights:
+            self.engine = random_engine(config_from_dir(model_dir), seed=seed, dtype=dtype,
+                                        max_tokens=max_tokens, ops=ops, use_graphs=use_graphs)
+        else:
+            self.engine = load_engine(model_dir, dtype=dtype, max_tokens=max_tokens, ops=ops,
+                                      use_graphs=use_graphs)
         self.config = self.engine.config
         spec = self.engine.model.spec
         self._sampler = Sampler(self.engine.ops, spec.vocab)

@@ -12,7 +12,9 @@ from typing import Iterator, Optional
 
 from .errors import ConfigError, RequestError
 
-_LOAD_KEYS = {"filename", "device", "dtype", "max_tokens", "max_batch"}
+_LOAD_KEYS = {"filename", "device", "dtype", "max_tokens", "max_batch", "random_weights", "seed"}
+_GENERATE_KEYS = {"prompts", "max_new_tokens", "temperature", "top_k", "top_p", "seed", "stop_tokens"}
+_STEP_KEYS = {"step", "entries", "end"}
 _COMPLETE_KEYS = {"messages", "token_ids", "temperature", "top_k", "top_p", "max_new_tokens", "seed"}
 
 
@@ -23,8 +25,9 @@ def parse(text: str) -> str:
 
 def load(kwargs_json: str):
     """``filename``: the model folder or its config.json; ``device``: cpu, cuda or auto
-    (src/libllm/llm.cc:154-168, 206-236).  Ours: ``dtype``, ``max_tokens``, ``max_batch``."""
-    from .api import Device, Model
+    (src/libllm/llm.cc:154-168, 206-236).  Ours: ``dtype``, ``max_tokens``, ``max_batch``, and
+    ``random_weights`` with ``seed`` (only config.json is then read)."""
+    from .api import Model, parse_device
     kw = json.loads(kwargs_json)
     if not isinstance(kw, dict):
         raise ConfigError("kwargs must be a JSON object")
@@ -33,12 +36,9 @@ def load(kwargs_json: str):
             raise ConfigError("unexpected key in kwargs: %s" % key)
     if "filename" not in kw:
         raise ConfigError("key \"filename\" is required")
-    device = str(kw.get("device", "auto")).lower()
-    if device not in ("cpu", "cuda", "auto"):
-        raise ConfigError("invalid device: %s" % device)
-    dev = {"cpu": Device.CPU, "cuda": Device.CUDA, "auto": Device.AUTO}[device]
-    return Model(kw["filename"], dev, dtype=kw.get("dtype", "bfloat16"),
-                 max_tokens=int(kw.get("max_tokens", 8192)), max_batch=int(kw.get("max_batch", 64)))
+    return Model(kw["filename"], parse_device(str(kw.get("device", "auto"))), dtype=kw.get("dtype", "bfloat16"),
+                 max_tokens=int(kw.get("max_tokens", 8192)), max_batch=int(kw.get("max_batch", 64)),
+                 random_weights=bool(kw.get("random_weights", False)), seed=int(kw.get("seed", 0)))
 
 
 def info(model) -> str:
@@ -82,3 +82,50 @@ def next_chunk(chunks: Iterator) -> Optional[str]:
     for chunk in chunks:
         return json.dumps({"text": chunk.text, "token_id": chunk.token_id})
     return None
+
+
+def generate(model, kwargs_json: str) -> str:
+    """Batches of prompts of token ids, as ``Model.generate``: ``{"prompts": [[...], ...]}`` with
+    ``max_new_tokens``, ``temperature``, ``top_k``, ``top_p``, ``seed``, ``stop_tokens``; returns
+    ``{"tokens": [[...], ...]}``.  No counterpart in the reference's C API."""
+    kw = json.loads(kwargs_json)
+    if not isinstance(kw, dict) or "prompts" not in kw:
+        raise RequestError("key \"prompts\" is required")
+    for key in kw:
+        if key not in _GENERATE_KEYS:
+            raise RequestError("unexpected key in kwargs: %s" % key)
+    prompts = [[int(t) for t in p] for p in kw["prompts"]]
+    out = model.generate(prompts, max_new_tokens=int(kw.get("max_new_tokens", 256)),
+                         temperature=float(kw.get("temperature", 1.0)), top_k=int(kw.get("top_k", 50)),
+                         top_p=float(kw.get("top_p", 0.8)), seed=int(kw.get("seed", 0)),
+                         stop_tokens=kw.get("stop_tokens"))
+    return json.dumps({"tokens": out})
+
+
+def step(model, kwargs_json: str, address: int, capacity: int) -> int:
+    """One call of the step function, in the words of a trace line: ``{"entries": [{"id", "tokens",
+    "want"}], "end": [...]}``.  The float32 logits at the wanted places, [wanted, vocab], are
+    written to ``capacity`` floats at ``address``; returns the number of wanted rows, or minus
+    the number of floats needed if they do not fit (nothing has run then).  No counterpart in the
+    reference's C API."""
+    import ctypes
+    from .engine import StepEntry
+    kw = json.loads(kwargs_json)
+    if not isinstance(kw, dict) or "entries" not in kw:
+        raise RequestError("key \"entries\" is required")
+    for key in kw:
+        if key not in _STEP_KEYS:
+            raise RequestError("unexpected key in kwargs: %s" % key)
+    entries = [StepEntry(e["id"], [int(t) for t in e["tokens"]], [int(w) for w in e.get("want", [])])
+               for e in kw["entries"]]
+    wanted = sum(len(e.want) for e in entries)
+    vocab = model.engine.vocab
+    if wanted * vocab > capacity:
+        return -(wanted * vocab)
+    logits = model.step(entries) if entries else None     # a line may only end requests
+    if wanted:
+        host = logits.float().cpu().contiguous().numpy()
+        ctypes.memmove(address, host.ctypes.data, host.nbytes)
+    if kw.get("end"):
+        model.end(list(kw["end"]))
+    return wanted

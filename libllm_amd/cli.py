@@ -36,23 +36,25 @@ def _model_args(prog):
     ap = argparse.ArgumentParser(prog=prog, allow_abbrev=False)
     _flag(ap, "m", action="append", default=[], metavar="MODEL",
           help="the model folder (config.json and model.safetensors)")
-    _flag(ap, "device", default="auto", help="inference device, either cpu, cuda or auto")
-    _flag(ap, "dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    _flag(ap, "device", default="auto", help="inference device, either cpu, cuda (or hip) or auto")
+    _flag(ap, "dtype", default="bfloat16", choices=["bfloat16", "float32", "bf16", "fp32"])
+    _flag(ap, "random_weights", action="store_true",
+          help="read only config.json from the model folder and draw the weights from -seed")
     _flag(ap, "max_tokens", type=int, default=8192, help="tokens the cache holds")
     return ap
 
 
 def _load(args, ap):
     device = args.device.lower()
-    if device not in ("cpu", "cuda", "auto"):
+    if device not in ("cpu", "cuda", "hip", "auto"):
         ap.error('invalid device name: must be one of "cpu", "cuda" or "auto"')
     if len(args.m) == 0:
         ap.error("model name (-m) is empty.")
     if len(args.m) != 1:
         ap.error("only 1 model (-m) is expected")
-    from .api import Device, Model
-    dev = {"cpu": Device.CPU, "cuda": Device.CUDA, "auto": Device.AUTO}[device]
-    return Model(args.m[0], dev, dtype=args.dtype, max_tokens=args.max_tokens)
+    from .api import Model
+    return Model(args.m[0], device, dtype=args.dtype, max_tokens=args.max_tokens,
+                 random_weights=args.random_weights, seed=getattr(args, "seed", 0))
 
 
 def chat_main(argv) -> int:
@@ -60,7 +62,7 @@ def chat_main(argv) -> int:
     _flag(ap, "temperature", type=float, default=1.0)
     _flag(ap, "top_k", type=int, default=50)
     _flag(ap, "top_p", type=float, default=0.8)
-    _flag(ap, "seed", type=int, default=0)
+    _flag(ap, "seed", type=int, default=0, help="seed of the sampler (and of -random_weights)")
     _flag(ap, "max_new_tokens", type=int, default=256)
     _flag(ap, "ids", action="store_true", help="lines are token ids; replies are printed as ids")
     args = ap.parse_args(argv)
@@ -163,7 +165,7 @@ def main(argv=None) -> int:
     try:
         if command == "chat":
             return chat_main(rest)
-        if command == "benchmark":
+        if command in ("benchmark", "bench"):
             return benchmark_main(rest)
     except LlmError as e:
         sys.stderr.write("llm: %s\n" % e)

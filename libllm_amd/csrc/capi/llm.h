@@ -40,7 +40,8 @@ int32_t llm_json_destroy(llm_json_t *j);
 int32_t llm_json_parse(llm_json_t *j, const char *json_str);
 int32_t llm_json_dump(llm_json_t *j, char *buf, int64_t buf_size);
 
-/* model: kwargs of load {"filename", "device"} (ours: "dtype", "max_tokens", "max_batch");
+/* model: kwargs of load {"filename", "device"} (ours: "dtype", "max_tokens", "max_batch",
+ * "random_weights", "seed");
  * info {"name", ...}; kwargs of complete {"messages" or "token_ids", "temperature", "top_k",
  * "top_p"} (ours: "max_new_tokens", "seed") */
 int32_t llm_model_init(llm_model_t *m);
@@ -48,6 +49,20 @@ int32_t llm_model_destroy(llm_model_t *m);
 int32_t llm_model_load(llm_model_t *m, llm_json_t *kwargs);
 int32_t llm_model_get_info(llm_model_t *m, llm_json_t *info);
 int32_t llm_model_complete(llm_model_t *m, llm_json_t *kwargs, llm_completion_t *comp);
+
+/* Two calls without a counterpart in the reference's C API, for what this library has beside
+ * single completions.
+ * generate: batches of prompts of token ids, unequal lengths, as many batches as the cache needs:
+ *   kwargs {"prompts": [[1, 2, 3], [4, 5]], "max_new_tokens", "temperature", "top_k", "top_p",
+ *   "seed", "stop_tokens"}; result {"tokens": [[...], [...]]}.
+ * step: one call of the step function, in the words of a line of a trace:
+ *   kwargs {"entries": [{"id": "a", "tokens": [5, 17, 3], "want": [0, 2]}], "end": []};
+ *   the float32 logits at the wanted places, [wanted, vocab] (vocab_size of get_info), go to
+ *   `logits`, which holds `capacity` floats; *n_rows is the number of wanted rows.  If they do not
+ *   fit, nothing runs, *n_rows is the number of floats needed and LLM_ERROR_INSUFFICIENT_BUFFER is
+ *   returned. */
+int32_t llm_model_generate(llm_model_t *m, llm_json_t *kwargs, llm_json_t *result);
+int32_t llm_model_step(llm_model_t *m, llm_json_t *kwargs, float *logits, int64_t capacity, int64_t *n_rows);
 
 /* completion: chunk {"text", "token_id"}; LLM_ERROR_EOF after the last one */
 int32_t llm_completion_init(llm_completion_t *c);

@@ -226,6 +226,40 @@ int32_t llm_model_complete(llm_model_t *m, llm_json_t *kwargs, llm_completion_t 
   return 0;
 }
 
+int32_t llm_model_generate(llm_model_t *m, llm_json_t *kwargs, llm_json_t *result) {
+  if (m == nullptr || *m == nullptr || (*m)->model == nullptr)
+    return fail(LLM_ERROR_INVALID_ARG, "invalid argument: m");
+  if (kwargs == nullptr || *kwargs == nullptr) return fail(LLM_ERROR_INVALID_ARG, "invalid argument: kwargs");
+  if (result == nullptr || *result == nullptr) return fail(LLM_ERROR_INVALID_ARG, "invalid argument: result");
+  Gil gil;
+  PyObject *out = call("generate", Py_BuildValue("(Os)", (*m)->model, (*kwargs)->text.c_str()));
+  if (out == nullptr) return LLM_ERROR_ABORTED;
+  const char *c = PyUnicode_AsUTF8(out);
+  if (c != nullptr) (*result)->text = c;
+  Py_DECREF(out);
+  return 0;
+}
+
+int32_t llm_model_step(llm_model_t *m, llm_json_t *kwargs, float *logits, int64_t capacity, int64_t *n_rows) {
+  if (m == nullptr || *m == nullptr || (*m)->model == nullptr)
+    return fail(LLM_ERROR_INVALID_ARG, "invalid argument: m");
+  if (kwargs == nullptr || *kwargs == nullptr) return fail(LLM_ERROR_INVALID_ARG, "invalid argument: kwargs");
+  if (n_rows == nullptr) return fail(LLM_ERROR_INVALID_ARG, "invalid argument: n_rows");
+  if (capacity < 0 || (capacity > 0 && logits == nullptr)) return fail(LLM_ERROR_INVALID_ARG, "invalid argument: logits");
+  Gil gil;
+  PyObject *out = call("step", Py_BuildValue("(OsKL)", (*m)->model, (*kwargs)->text.c_str(),
+                                             (unsigned long long)(uintptr_t)logits, (long long)capacity));
+  if (out == nullptr) return LLM_ERROR_ABORTED;
+  const long long rows = PyLong_AsLongLong(out);
+  Py_DECREF(out);
+  if (rows < 0) {
+    *n_rows = -rows;
+    return fail(LLM_ERROR_INSUFFICIENT_BUFFER, "insufficient buffer for the logits");
+  }
+  *n_rows = rows;
+  return 0;
+}
+
 int32_t llm_completion_init(llm_completion_t *c) {
   if (c == nullptr) return fail(LLM_ERROR_INVALID_ARG, "invalid argument: c");
   *c = new llm_completion_impl_t();

@@ -1,8 +1,9 @@
 // The `llm` program over the C API (llm.h), as the reference's command line is a program over its
 // C API (go/bin/main.go:27-54, go/bin/args.go:54-91, go/bin/chat.go:44-132):
 //
-//   llm chat -m MODEL [-device cpu|cuda|auto] [-dtype bfloat16|float32] [-max_tokens N]
+//   llm chat -m MODEL [-device cpu|cuda|hip|auto] [-dtype bfloat16|float32] [-max_tokens N]
 //            [-temperature T] [-top_k K] [-top_p P] [-seed S] [-max_new_tokens N] [-ids]
+//            [-random_weights]
 //
 // A prompt loop with `:new` (clear the history), `:sys <prompt>` (set the system prompt and clear),
 // empty lines ignored, end of input leaving; after each reply `(N tokens, time=..s, ..ms per token)`.
@@ -38,7 +39,8 @@ void usage() {
 void chat_usage() {
   std::fprintf(stderr,
                "usage: llm chat -m MODEL [-device DEVICE] [-dtype {bfloat16,float32}] [-max_tokens N]\n"
-               "                [-temperature T] [-top_k K] [-top_p P] [-seed S] [-max_new_tokens N] [-ids]\n");
+               "                [-temperature T] [-top_k K] [-top_p P] [-seed S] [-max_new_tokens N] [-ids]\n"
+               "                [-random_weights]\n");
 }
 
 [[noreturn]] void arg_error(const std::string &msg) {
@@ -150,7 +152,7 @@ int chat_main(int argc, char **argv) {
   std::string device = "auto", dtype = "bfloat16";
   long max_tokens = 8192, top_k = 50, seed = 0, max_new = 256;
   double temperature = 1.0, top_p = 0.8;
-  bool ids = false;
+  bool ids = false, random_weights = false;
   for (int i = 0; i < argc; ++i) {
     std::string flag = argv[i];
     if (flag.size() < 2 || flag[0] != '-') arg_error("unrecognized arguments: " + flag);
@@ -158,6 +160,7 @@ int chat_main(int argc, char **argv) {
     for (char &c : flag) if (c == '-') c = '_';
     if (flag == "h" || flag == "help") { chat_usage(); return 0; }
     if (flag == "ids") { ids = true; continue; }
+    if (flag == "random_weights") { random_weights = true; continue; }
     if (i + 1 >= argc) arg_error("argument -" + flag + ": expected one argument");
     const std::string value = argv[++i];
     char *end = nullptr;
@@ -174,9 +177,9 @@ int chat_main(int argc, char **argv) {
     else if (flag == "max_new_tokens") max_new = as_long();
     else arg_error("unrecognized arguments: -" + flag);
   }
-  if (device != "cpu" && device != "cuda" && device != "auto")
+  if (device != "cpu" && device != "cuda" && device != "hip" && device != "auto")
     arg_error("invalid device name: must be one of \"cpu\", \"cuda\" or \"auto\"");
-  if (dtype != "bfloat16" && dtype != "float32") arg_error("argument -dtype: invalid choice: '" + dtype + "'");
+  if (dtype != "bfloat16" && dtype != "float32" && dtype != "bf16" && dtype != "fp32") arg_error("argument -dtype: invalid choice: '" + dtype + "'");
   if (models.empty()) arg_error("model name (-m) is empty.");
   if (models.size() != 1) arg_error("only 1 model (-m) is expected");
 
@@ -191,7 +194,8 @@ int chat_main(int argc, char **argv) {
   {
     std::ostringstream js;
     js << "{\"filename\": " << quoted(models[0]) << ", \"device\": " << quoted(device) << ", \"dtype\": "
-       << quoted(dtype) << ", \"max_tokens\": " << max_tokens << "}";
+       << quoted(dtype) << ", \"max_tokens\": " << max_tokens << ", \"random_weights\": "
+       << (random_weights ? "true" : "false") << ", \"seed\": " << seed << "}";
     CHECK(llm_json_parse(&kwargs, js.str().c_str()));
     CHECK(llm_model_load(&model, &kwargs));
   }

@@ -71,6 +71,11 @@ def test_argument_checks_and_load_errors(lib, tmp_path):
                          ('{"filename": "%s", "device": "auto"}' % tmp_path, b"config.json")):
         assert lib.llm_model_load(ctypes.byref(m), ctypes.byref(new_json(lib, kwargs))) == ABORTED
         assert word in lib.llm_get_last_error_message(), lib.llm_get_last_error_message()
+    # generate and step need a loaded model, a result and a place for the count
+    n = ctypes.c_int64()
+    assert lib.llm_model_generate(ctypes.byref(m), ctypes.byref(new_json(lib, "{}")), ctypes.byref(new_json(lib))) == INVALID_ARG
+    assert lib.llm_model_step(ctypes.byref(m), ctypes.byref(new_json(lib, "{}")), None, ctypes.c_int64(0),
+                              ctypes.byref(n)) == INVALID_ARG
     assert lib.llm_model_destroy(ctypes.byref(m)) == 0 and m.value is None
     assert lib.llm_completion_destroy(ctypes.byref(c)) == 0 and c.value is None
 
@@ -136,3 +141,81 @@ def test_completion_from_a_c_program(lib, tiny_model, tmp_path):
     got = [t for t in got if t is not None]
     assert got == want
     assert lines[-1] == "end"
+
+
+@pytest.mark.gpu
+def test_generate_and_step_from_c(lib, tiny_model):
+    """Batches of unequal prompts and the step function through the C API, against the plain
+    implementation; a buffer that is too small is refused before anything runs."""
+    path, cfg, weights = tiny_model
+    rng = np.random.default_rng(12)
+    prompts = [rng.integers(3, cfg.vocab, size=k).tolist() for k in (3, 9, 1)]
+    m = ctypes.c_void_p()
+    assert lib.llm_model_init(ctypes.byref(m)) == 0
+    kwargs = new_json(lib, json.dumps({"filename": path, "device": "hip", "dtype": "fp32", "max_tokens": 1024}))
+    assert lib.llm_model_load(ctypes.byref(m), ctypes.byref(kwargs)) == 0, lib.llm_get_last_error_message()
+    # generate
+    result = new_json(lib)
+    ask = new_json(lib, json.dumps({"prompts": prompts, "max_new_tokens": 5, "temperature": 0.0}))
+    assert lib.llm_model_generate(ctypes.byref(m), ctypes.byref(ask), ctypes.byref(result)) == 0, \
+        lib.llm_get_last_error_message()
+    got = json.loads(dump(lib, result)[1])["tokens"]
+    assert got == [sampling.generate(cfg, weights, p, 5, temperature=0.0) for p in prompts]
+    bad = new_json(lib, json.dumps({"prompts": prompts, "beams": 4}))
+    assert lib.llm_model_generate(ctypes.byref(m), ctypes.byref(bad), ctypes.byref(result)) == ABORTED
+    assert b"beams" in lib.llm_get_last_error_message()
+    # step: two prompts at once, then one token each; the shorter request ends first
+    lib.llm_model_step.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+    n = ctypes.c_int64()
+    a, b = prompts[0], prompts[1]
+    line = {"entries": [{"id": "a", "tokens": a, "want": [0, len(a) - 1]}, {"id": "b", "tokens": b, "want": [len(b) - 1]}]}
+    small = (ctypes.c_float * 8)()
+    rc = lib.llm_model_step(ctypes.byref(m), ctypes.byref(new_json(lib, json.dumps(line))), small, 8, ctypes.byref(n))
+    assert rc == INSUFFICIENT_BUFFER and n.value == 3 * cfg.vocab         # nothing ran: the same step goes again
+    buf = (ctypes.c_float * (3 * cfg.vocab))()
+    rc = lib.llm_model_step(ctypes.byref(m), ctypes.byref(new_json(lib, json.dumps(line))), buf, 3 * cfg.vocab, ctypes.byref(n))
+    assert rc == 0 and n.value == 3, lib.llm_get_last_error_message()
+    out = np.ctypeslib.as_array(buf).reshape(3, cfg.vocab).copy()
+    la, lb = llama.logits_all(cfg, weights, a), llama.logits_all(cfg, weights, b)
+    ref = np.stack([la[0], la[-1], lb[-1]])
+    assert np.abs(out - ref).max() < 2e-4 * max(1.0, np.abs(ref).max())
+    line = {"entries": [{"id": "a", "tokens": [7], "want": [0]}, {"id": "b", "tokens": [9], "want": []}], "end": ["b"]}
+    rc = lib.llm_model_step(ctypes.byref(m), ctypes.byref(new_json(lib, json.dumps(line))), buf, 3 * cfg.vocab, ctypes.byref(n))
+    assert rc == 0 and n.value == 1
+    out = np.ctypeslib.as_array(buf)[:cfg.vocab].copy()
+    ref = llama.logits_all(cfg, weights, a + [7])[-1]
+    assert np.abs(out - ref).max() < 2e-4 * max(1.0, np.abs(ref).max())
+    rc = lib.llm_model_step(ctypes.byref(m), ctypes.byref(new_json(lib, '{"entries": [], "end": ["a"]}')), None, 0, ctypes.byref(n))
+    assert rc == 0 and n.value == 0
+    rc = lib.llm_model_step(ctypes.byref(m), ctypes.byref(new_json(lib, '{"entries": [], "end": ["a"]}')), None, 0, ctypes.byref(n))
+    assert rc == ABORTED                                                   # released twice
+    assert lib.llm_model_destroy(ctypes.byref(m)) == 0
+
+
+@pytest.mark.gpu
+def test_random_weights_from_c(lib, tiny_model, tmp_path):
+    """A folder with config.json alone and "random_weights": the same seed gives the same model."""
+    import shutil
+    path, cfg, _ = tiny_model
+    shutil.copy(os.path.join(path, "config.json"), tmp_path / "config.json")
+    lib.llm_model_step.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int64, ctypes.c_void_p]
+    outs = []
+    for seed in (3, 3, 4):
+        m = ctypes.c_void_p()
+        assert lib.llm_model_init(ctypes.byref(m)) == 0
+        kwargs = new_json(lib, json.dumps({"filename": str(tmp_path), "random_weights": True, "seed": seed,
+                                           "dtype": "float32", "max_tokens": 256}))
+        assert lib.llm_model_load(ctypes.byref(m), ctypes.byref(kwargs)) == 0, lib.llm_get_last_error_message()
+        # logits, not greedy tokens: a random model with tied embeddings repeats its last token
+        buf, n = (ctypes.c_float * cfg.vocab)(), ctypes.c_int64()
+        line = new_json(lib, json.dumps({"entries": [{"id": 0, "tokens": [5, 6, 7], "want": [2]}], "end": [0]}))
+        assert lib.llm_model_step(ctypes.byref(m), ctypes.byref(line), buf, cfg.vocab, ctypes.byref(n)) == 0
+        outs.append(np.ctypeslib.as_array(buf).copy())
+        assert lib.llm_model_destroy(ctypes.byref(m)) == 0
+    assert np.isfinite(outs[0]).all() and outs[0].std() > 0
+    assert np.array_equal(outs[0], outs[1]) and not np.allclose(outs[0], outs[2])
+    kwargs = new_json(lib, json.dumps({"filename": str(tmp_path)}))       # without the flag the tensors are missed
+    m = ctypes.c_void_p()
+    assert lib.llm_model_init(ctypes.byref(m)) == 0
+    assert lib.llm_model_load(ctypes.byref(m), ctypes.byref(kwargs)) == ABORTED
+    assert lib.llm_model_destroy(ctypes.byref(m)) == 0

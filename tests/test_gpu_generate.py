@@ -101,6 +101,28 @@ def test_command_line(model_b, program):
     assert "===== new session =====" in proc.stdout
 
 
+@pytest.mark.parametrize("program", ["python", "native"])
+def test_command_line_random_weights_and_aliases(model_b, program, tmp_path):
+    """-random_weights reads config.json alone; hip names the GPU, fp32 the dtype; two dashes work."""
+    import shutil
+    path, _, _ = model_b
+    shutil.copy(os.path.join(path, "config.json"), tmp_path / "config.json")
+    outs = []
+    for seed in ("3", "3"):
+        proc = subprocess.run(programs()[program] + ["chat", "-m", str(tmp_path), "--device", "hip", "-dtype", "fp32",
+                                                     "--random-weights", "-seed", seed, "-ids", "-temperature", "0",
+                                                     "-max_new_tokens", "5"],
+                              input="11 12 13\n", capture_output=True, text=True, timeout=120)
+        assert proc.returncode == 0, proc.stderr
+        outs.append([l for l in proc.stdout.splitlines() if l.startswith("> ") and len(l) > 2][0])
+    assert outs[0] == outs[1] and len(outs[0].split()) == 6              # the prompt sign and five ids
+    # (a random model with tied embeddings repeats its last token: that seeds differ shows in logits,
+    # which test_capi.py::test_random_weights_from_c compares)
+    proc = subprocess.run(programs()[program] + ["chat", "-m", str(tmp_path), "-device", "tpu"], input="",
+                          capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 2 and "invalid device name" in proc.stderr
+
+
 def test_command_lines_agree_on_a_text_session(model_b):
     """A session in text (bytes as token ids, since the model folder has no tokenizer): a system
     prompt, quotes, a backslash and characters beyond ASCII in the questions, a second turn that
