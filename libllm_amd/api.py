@@ -92,13 +92,15 @@ class _FileTokenizer:
 class Completion:
     """Iterating yields Chunks until a stop token or the token budget ends the reply."""
 
-    def __init__(self, model: "Model", ids: List[int], params: SamplingParams, max_new_tokens: int):
+    def __init__(self, model: "Model", ids: List[int], params: SamplingParams, max_new_tokens: int,
+                 stop_tokens: Optional[Iterable[int]] = None):
         self._model, self._ids, self._params, self._max = model, ids, params, max_new_tokens
+        self._stop = stop_tokens
 
     def __iter__(self):
         decoder = codecs.getincrementaldecoder("utf-8")(errors="replace")
         gen = self._model._generator
-        for _, token in gen.stream([self._ids], self._params, self._max):
+        for _, token in gen.stream([self._ids], self._params, self._max, self._stop):
             # one chunk per token; its text is empty while a multi-byte character is incomplete
             yield Chunk(decoder.decode(self._model._tokenizer().piece(token)), token)
         tail = decoder.decode(b"", final=True)
@@ -134,6 +136,15 @@ class Model:
     def name(self) -> str:
         return self.engine.model.spec.name
 
+    def is_stop(self, token: int) -> bool:
+        """Whether the model's configuration names ``token`` as a stop token (src/libllm/llama.cc:390-392)."""
+        return int(token) in self.engine.model.spec.stop_tokens
+
+    @property
+    def output_dim(self) -> int:
+        """The width of a row of logits (src/libllm/llama.cc:398-400)."""
+        return self.engine.vocab
+
     def _tokenizer(self):
         if self._tok is None:
             path = os.path.join(self.model_dir, "tokenizer.json")
@@ -162,12 +173,14 @@ class Model:
 
     def complete(self, prompt: Union[str, List[Union[str, int, ControlToken]]], top_k: int = 50,
                  top_p: float = 0.8, temperature: float = 1.0, max_new_tokens: int = 256,
-                 seed: int = 0) -> Completion:
-        """Completes the prompt; defaults as the reference's (python/libllm/__init__.py:76-77)."""
+                 seed: int = 0, stop_ids: Optional[Iterable[int]] = None) -> Completion:
+        """Completes the prompt; defaults as the reference's (python/libllm/__init__.py:76-77).
+        ``stop_ids`` end the reply beside the model's own stop tokens."""
         ids = self._prepare_prompt(prompt)
         if not ids:
             raise RequestError("the prompt is empty")
-        return Completion(self, ids, SamplingParams(temperature, top_k, top_p, seed), max_new_tokens)
+        stop = None if stop_ids is None else set(self.engine.model.spec.stop_tokens) | {int(t) for t in stop_ids}
+        return Completion(self, ids, SamplingParams(temperature, top_k, top_p, seed), max_new_tokens, stop)
 
     def generate(self, prompts: Sequence[Sequence[int]], max_new_tokens: int = 256,
                  temperature: float = 1.0, top_k: int = 50, top_p: float = 0.8, seed: int = 0,

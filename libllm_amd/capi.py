@@ -15,7 +15,7 @@ from .errors import ConfigError, RequestError
 _LOAD_KEYS = {"filename", "device", "dtype", "max_tokens", "max_batch", "random_weights", "seed"}
 _GENERATE_KEYS = {"prompts", "max_new_tokens", "temperature", "top_k", "top_p", "seed", "stop_tokens"}
 _STEP_KEYS = {"step", "entries", "end"}
-_COMPLETE_KEYS = {"messages", "token_ids", "temperature", "top_k", "top_p", "max_new_tokens", "seed"}
+_COMPLETE_KEYS = {"messages", "token_ids", "temperature", "top_k", "top_p", "max_new_tokens", "seed", "stop_ids"}
 
 
 def parse(text: str) -> str:
@@ -52,7 +52,7 @@ def complete(model, kwargs_json: str) -> Iterator:
     """Starts a completion.  ``messages`` is a list of ``{"role", "content"}`` as in the reference
     (src/libllm/llm.cc:98-123); since tokenisation lies outside this library the contents are
     joined as the command line joins them.  Ours: ``token_ids`` in place of ``messages``,
-    ``max_new_tokens``, ``seed``.  Defaults: temperature 1.0, top_k 50, top_p 0.8
+    ``max_new_tokens``, ``seed``, ``stop_ids`` (beside the model's own).  Defaults: temperature 1.0, top_k 50, top_p 0.8
     (src/libllm/llm.cc:125-132)."""
     kw = json.loads(kwargs_json)
     if not isinstance(kw, dict):
@@ -73,7 +73,8 @@ def complete(model, kwargs_json: str) -> Iterator:
         prompt = "".join(parts) + "assistant: "
     completion = model.complete(prompt, top_k=int(kw.get("top_k", 50)), top_p=float(kw.get("top_p", 0.8)),
                                 temperature=float(kw.get("temperature", 1.0)),
-                                max_new_tokens=int(kw.get("max_new_tokens", 256)), seed=int(kw.get("seed", 0)))
+                                max_new_tokens=int(kw.get("max_new_tokens", 256)), seed=int(kw.get("seed", 0)),
+                                stop_ids=kw.get("stop_ids"))
     return iter(completion)
 
 

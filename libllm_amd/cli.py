@@ -65,6 +65,8 @@ def chat_main(argv) -> int:
     _flag(ap, "seed", type=int, default=0, help="seed of the sampler (and of -random_weights)")
     _flag(ap, "max_new_tokens", type=int, default=256)
     _flag(ap, "ids", action="store_true", help="lines are token ids; replies are printed as ids")
+    _flag(ap, "stop_id", type=int, action="append", default=None,
+          help="a token id that ends a reply, beside the model's own (repeatable)")
     args = ap.parse_args(argv)
     model = _load(args, ap)
     print(MSG_INPUT)
@@ -106,7 +108,8 @@ def chat_main(argv) -> int:
         t0 = time.time()
         n, reply_ids, reply_text = 0, [], ""
         for chunk in model.complete(prompt, top_k=args.top_k, top_p=args.top_p, temperature=args.temperature,
-                                    max_new_tokens=args.max_new_tokens, seed=args.seed + turn):
+                                    max_new_tokens=args.max_new_tokens, seed=args.seed + turn,
+                                    stop_ids=args.stop_id):
             if chunk.token_id is not None:
                 n += 1
                 reply_ids.append(chunk.token_id)

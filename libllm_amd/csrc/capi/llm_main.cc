@@ -3,7 +3,7 @@
 //
 //   llm chat -m MODEL [-device cpu|cuda|hip|auto] [-dtype bfloat16|float32] [-max_tokens N]
 //            [-temperature T] [-top_k K] [-top_p P] [-seed S] [-max_new_tokens N] [-ids]
-//            [-random_weights]
+//            [-random_weights] [-stop_id ID]...
 //
 // A prompt loop with `:new` (clear the history), `:sys <prompt>` (set the system prompt and clear),
 // empty lines ignored, end of input leaving; after each reply `(N tokens, time=..s, ..ms per token)`.
@@ -40,7 +40,7 @@ void chat_usage() {
   std::fprintf(stderr,
                "usage: llm chat -m MODEL [-device DEVICE] [-dtype {bfloat16,float32}] [-max_tokens N]\n"
                "                [-temperature T] [-top_k K] [-top_p P] [-seed S] [-max_new_tokens N] [-ids]\n"
-               "                [-random_weights]\n");
+               "                [-random_weights] [-stop_id ID]...\n");
 }
 
 [[noreturn]] void arg_error(const std::string &msg) {
@@ -153,6 +153,7 @@ int chat_main(int argc, char **argv) {
   long max_tokens = 8192, top_k = 50, seed = 0, max_new = 256;
   double temperature = 1.0, top_p = 0.8;
   bool ids = false, random_weights = false;
+  std::vector<long> stop_ids;
   for (int i = 0; i < argc; ++i) {
     std::string flag = argv[i];
     if (flag.size() < 2 || flag[0] != '-') arg_error("unrecognized arguments: " + flag);
@@ -175,6 +176,7 @@ int chat_main(int argc, char **argv) {
     else if (flag == "top_p") top_p = as_double();
     else if (flag == "seed") seed = as_long();
     else if (flag == "max_new_tokens") max_new = as_long();
+    else if (flag == "stop_id") stop_ids.push_back(as_long());
     else arg_error("unrecognized arguments: -" + flag);
   }
   if (device != "cpu" && device != "cuda" && device != "hip" && device != "auto")
@@ -261,7 +263,13 @@ int chat_main(int argc, char **argv) {
     }
     js.precision(17);
     js << ", \"temperature\": " << temperature << ", \"top_k\": " << top_k << ", \"top_p\": " << top_p
-       << ", \"max_new_tokens\": " << max_new << ", \"seed\": " << (seed + turn) << "}";
+       << ", \"max_new_tokens\": " << max_new << ", \"seed\": " << (seed + turn);
+    if (!stop_ids.empty()) {
+      js << ", \"stop_ids\": [";
+      for (size_t i = 0; i < stop_ids.size(); ++i) js << (i ? ", " : "") << stop_ids[i];
+      js << "]";
+    }
+    js << "}";
     CHECK(llm_json_parse(&kwargs, js.str().c_str()));
 
     const auto t0 = std::chrono::steady_clock::now();

@@ -102,6 +102,31 @@ def test_command_line(model_b, program):
 
 
 @pytest.mark.parametrize("program", ["python", "native"])
+def test_command_line_stop_id(model_b, program):
+    """-stop_id names a further stop token: the reply ends before it and it is not printed."""
+    path, cfg, weights = model_b
+    prompt = [11, 12, 13, 14]
+    want = sampling.generate(cfg, weights, prompt, 6)
+    stop = want[2]
+    cut = want[:want.index(stop)]
+    proc = subprocess.run(programs()[program] + ["chat", "-m", path, "-dtype", "float32", "-ids", "-temperature", "0",
+                                                 "-max_new_tokens", "6", "-stop_id", str(stop), "-stop_id", "999999"],
+                          input=" ".join(map(str, prompt)) + "\n", capture_output=True, text=True, timeout=120)
+    assert proc.returncode == 0, proc.stderr
+    reply = [l for l in proc.stdout.splitlines() if l.startswith("> ")][0][2:].split()
+    assert [int(t) for t in reply] == cut
+    assert "(%d tokens," % len(cut) in proc.stdout
+
+
+def test_model_is_stop_and_output_dim(model_b):
+    from libllm_amd import Model
+    path, cfg, _ = model_b
+    model = Model(path, "hip", dtype="fp32", max_tokens=256)
+    assert model.output_dim == cfg.vocab
+    assert all(model.is_stop(t) for t in cfg.stop) and not model.is_stop(max(cfg.stop, default=0) + 1)
+
+
+@pytest.mark.parametrize("program", ["python", "native"])
 def test_command_line_random_weights_and_aliases(model_b, program, tmp_path):
     """-random_weights reads config.json alone; hip names the GPU, fp32 the dtype; two dashes work."""
     import shutil
