@@ -183,6 +183,28 @@ def test_padding_changes_nothing(models):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_batch_order_changes_nothing(models, dtype):
+    """The same requests in the opposite order take other slots and other rows of every step.
+    Prompts short enough for the kernels whose sums do not depend on the row (at most 64 rows a
+    step): the same bits for every request, in 32-bit and in bfloat16.  And a request alone
+    gives what it gives inside the batch."""
+    from libllm_amd.runtime import load_engine
+    path, cfg, weights = models["B"]
+    requests = make_requests(cfg, [9, 30, 17], seed=44)              # 44 rows of prompt, then 4 tokens each
+    swapped = dict(reversed(list(requests.items())))
+    e1 = load_engine(path, dtype=dtype, max_tokens=1024)
+    e2 = load_engine(path, dtype=dtype, max_tokens=1024)
+    a, b = _decode_rows(e1, requests, 4), _decode_rows(e2, swapped, 4)
+    assert np.array_equal(a, b[:, ::-1])
+    e3 = load_engine(path, dtype=dtype, max_tokens=1024)
+    alone = _decode_rows(e3, {"r1": requests["r1"]}, 4)
+    if dtype == "float32":
+        assert np.array_equal(alone[:, 0], a[:, 1])
+    else:
+        assert_logits_close(alone[:, 0], a[:, 1].astype(np.float64), dtype, "alone against in a batch")
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_trace_run_program(models, tmp_path, dtype):
     """bin/trace_run as a user starts it: a child process fed through its standard input, one
     step after each ``done`` line."""
