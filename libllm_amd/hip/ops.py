@@ -173,7 +173,7 @@ class HipOps:
     SKINNY_ROWS = 64        # most rows the streaming matrix product takes at once
     NORM_ROWS = 16          # most rows for which the norm is fused into the product
     NORM_COLS = 4096        # and most rows of the weight
-    DECODE_BLOCKS = 4096    # blocks of the decode attention grid beyond which sequences are not split further
+    DECODE_BLOCKS = 768     # blocks of the decode attention grid beyond which sequences are not split further
     _EPI_NONE, _EPI_SWIGLU, _EPI_ACCUM = 0, 1, 2
 
     def prepare_weight(self, w: torch.Tensor, like=None):
@@ -458,8 +458,12 @@ class HipOps:
                 if window:
                     pages = min(pages, window // 64 + 2)
                 waves = self.lib.llm_attention_decode_waves(hd)
-                # a page for each wave, as long as the grid stays within a few thousand blocks
+                # a page for each wave, as long as the grid stays within two or three blocks a
+                # compute unit; the kernel gives every wave ceil(pages / waves) pages in a row, so
+                # blocks beyond ceil(pages / (that * waves)) would get none: they are not launched
                 n_blocks = max(1, min(-(-pages // waves), max(1, self.DECODE_BLOCKS // (m * n_kv))))
+                per_wave = -(-pages // (n_blocks * waves))
+                n_blocks = -(-pages // (per_wave * waves))
                 part_o = torch.empty((m, n_heads, n_blocks, hd), dtype=torch.float32, device=self.device)
                 part_ml = torch.empty((m, n_heads, n_blocks, 2), dtype=torch.float32, device=self.device)
                 self._check(self.lib.llm_attention_decode_bf16(
