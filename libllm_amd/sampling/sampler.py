@@ -50,20 +50,20 @@ class SamplingParams:
 
 
 class PendingTokens:
-    """Tokens the sampler wrote on the device, on their way to the host on a stream of their own:
-    the device can go on with work queued behind the sampling while the host waits only for the
-    copy.  ``device`` is the int32 tensor; ``tokens()`` waits and returns the list."""
+    """Tokens the sampler wrote on the device, on their way to the host.  The copy is queued on
+    the stream of the sampling itself, at once, so behind it and before whatever the caller queues
+    next: the device goes on with that work while the host waits only for the copy.  (On a stream
+    of its own the copy can end up behind the next step all the same, since streams share few
+    hardware queues, each of which runs its commands in order; the host then sees every token a
+    step late and the device idles while the host queues the step after.)  ``device`` is the
+    int32 tensor; ``tokens()`` waits and returns the list."""
 
-    def __init__(self, device: torch.Tensor, copy_stream):
+    def __init__(self, device: torch.Tensor):
         self.device = device
         self._host = torch.empty(device.shape, dtype=device.dtype, pin_memory=True)
-        ready = torch.cuda.Event()
-        ready.record()
-        with torch.cuda.stream(copy_stream):
-            copy_stream.wait_event(ready)
-            self._host.copy_(device, non_blocking=True)
-            self._done = torch.cuda.Event()
-            self._done.record(copy_stream)
+        self._host.copy_(device, non_blocking=True)
+        self._done = torch.cuda.Event()
+        self._done.record()
         self._list = None
 
     def tokens(self) -> List[int]:
@@ -84,7 +84,6 @@ class Sampler:
     def __init__(self, ops, vocab: int):
         self.ops = ops
         self.vocab = vocab
-        self._copy_stream = None
 
     @property
     def samples_ahead(self) -> bool:
@@ -93,8 +92,8 @@ class Sampler:
 
     def sample_device(self, logits: torch.Tensor, params: SamplingParams, streams: Sequence[int],
                       counters: Sequence[int]) -> PendingTokens:
-        """As ``sample``, but returns at once: the tokens stay on the device and travel to the
-        host on a side stream."""
+        """As ``sample``, but returns at once: the tokens stay on the device, and their copy to
+        the host is queued behind the sampling."""
         p = params.validate(self.vocab)
         if logits.shape[0] != len(streams) or len(streams) != len(counters):
             raise RequestError("one stream and one counter per row of logits are needed")
@@ -103,9 +102,7 @@ class Sampler:
         else:
             out = self.ops.sample(logits, p.temperature, p.top_k, p.top_p, p.seed,
                                   list(streams), list(counters))
-        if self._copy_stream is None:
-            self._copy_stream = torch.cuda.Stream(device=out.device)
-        return PendingTokens(out, self._copy_stream)
+        return PendingTokens(out)
 
     def sample(self, logits: torch.Tensor, params: SamplingParams, streams: Sequence[int],
                counters: Sequence[int]) -> List[int]:
