@@ -21,12 +21,6 @@
 // token's position (src/libllm/llama.cc:151-176 pairs j with j + rot_dim/2; the reordering only
 // moves them side by side), rotated q to the output, rotated k and v to the token's place in the
 // paged cache (keys [page, kv_head, position, dim], values [page, kv_head, dim, position]).
-//
-// Fused RMS norm (up to 16 rows): X is then the float32 residual stream.  Staging multiplies each
-// element by the norm's weight and rounds to bfloat16, and sums the squares of the row on the way
-// (every block stages whole rows); the factor 1/sqrt(mean(x^2) + eps) of a row is applied to its
-// outputs in the epilogue (src/flint/cuda/rms_norm.cu:45-76 computes the same product).  `rows`
-// optionally names the rows of the stream to use.
 #include "mfma.h"
 
 #define SK_WK 8            // waves that split K
@@ -37,13 +31,6 @@
 
 // MT: 16-row tiles of X; RT: 16-row tiles of W per wave; WN: row groups per block; G: granules of
 // 2 steps that a wave takes per chunk (a chunk is 512*G elements of K).
-struct SkinnyNorm {
-  const float* x;          // float32 rows [*, K]
-  const float* weight;     // [K]
-  const int* rows;         // row of x for each of the M rows, or null for 0..M-1
-  float eps;
-};
-
 struct SkinnyRope {
   const float* bias;       // [N] or null
   const float* cos_t;      // [positions, rot_dim / 2]
@@ -57,14 +44,12 @@ struct SkinnyRope {
   int table_stride, n_heads, n_kv, hd, rot_dim, write_kv;
 };
 
-template <int MT, int RT, int WN, int G, int EPI, bool XNORM, typename OutT>
+template <int MT, int RT, int WN, int G, int EPI, typename OutT>
 __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ X,
-                                                                      SkinnyNorm norm,
                                                                       const bf16_t* __restrict__ W,
                                                                       OutT* __restrict__ C, int M,
                                                                       int N, int K, int ldw,
                                                                       int n_out, SkinnyRope rope) {
-  static_assert(!XNORM || (MT == 1 && WN == 1), "the fused norm is built for up to 16 rows");
   constexpr int NT = WN * SK_WK * 64;
   constexpr int CK = 512 * G;                    // elements of K per chunk
   constexpr int ROW_B = CK * 2;                  // bytes of a staged row; 16-byte pieces are swizzled
@@ -75,8 +60,6 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   constexpr int ROWS_PASS = NT / XV;             // rows staged per pass of the block
   constexpr int PASSES = (16 * MT + ROWS_PASS - 1) / ROWS_PASS;
   __shared__ __attribute__((aligned(16))) unsigned char lds[LDS_BYTES];
-  __shared__ float s_ss[XNORM ? SK_WK : 1][PASSES];
-  __shared__ float s_inv[16 * MT];
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int wn = wave / SK_WK, wk = wave % SK_WK;
@@ -117,53 +100,19 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   // staging of X: thread t carries piece (t % XV) of rows (t / XV) + p * ROWS_PASS
   const int x_col = tid % XV, x_row0 = tid / XV;
   uint4 xr[PASSES];
-  float4 xf[XNORM ? PASSES : 1][2], wf[2];
-  float ss[XNORM ? PASSES : 1];
-  const float* xsrc[XNORM ? PASSES : 1];
-  if (XNORM) {
+  auto load_x = [&](int chunk) {
+    const int k = chunk * CK + x_col * 8;
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
       const int row = x_row0 + p * ROWS_PASS;
-      ss[p] = 0.f;
-      const int src = (row < M) ? (norm.rows ? norm.rows[row] : row) : 0;
-      xsrc[p] = norm.x + (size_t)src * K;
-    }
-  }
-  auto load_x = [&](int chunk) {
-    const int k = chunk * CK + x_col * 8;
-    if (XNORM) {
-      const bool in = k < K;
-      wf[0] = in ? *reinterpret_cast<const float4*>(norm.weight + k) : make_float4(0.f, 0.f, 0.f, 0.f);
-      wf[1] = in ? *reinterpret_cast<const float4*>(norm.weight + k + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-#pragma unroll
-      for (int p = 0; p < PASSES; ++p) {
-        const int row = x_row0 + p * ROWS_PASS;
-        const bool ok = in && row < M;
-        xf[p][0] = ok ? *reinterpret_cast<const float4*>(xsrc[p] + k) : make_float4(0.f, 0.f, 0.f, 0.f);
-        xf[p][1] = ok ? *reinterpret_cast<const float4*>(xsrc[p] + k + 4) : make_float4(0.f, 0.f, 0.f, 0.f);
-      }
-    } else {
-#pragma unroll
-      for (int p = 0; p < PASSES; ++p) {
-        const int row = x_row0 + p * ROWS_PASS;
-        xr[p] = (row < M && k < K) ? *reinterpret_cast<const uint4*>(X + (size_t)row * K + k)
-                                   : make_uint4(0u, 0u, 0u, 0u);
-      }
+      xr[p] = (row < M && k < K) ? *reinterpret_cast<const uint4*>(X + (size_t)row * K + k)
+                                 : make_uint4(0u, 0u, 0u, 0u);
     }
   };
   auto store_x = [&]() {
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
       const int row = x_row0 + p * ROWS_PASS;
-      if (XNORM) {
-        const float4 a0 = xf[p][0], a1 = xf[p][1];
-        ss[p] += a0.x * a0.x + a0.y * a0.y + a0.z * a0.z + a0.w * a0.w + a1.x * a1.x + a1.y * a1.y +
-                 a1.z * a1.z + a1.w * a1.w;
-        xr[p].x = (uint32_t)f32_to_bf16(a0.x * wf[0].x) | ((uint32_t)f32_to_bf16(a0.y * wf[0].y) << 16);
-        xr[p].y = (uint32_t)f32_to_bf16(a0.z * wf[0].z) | ((uint32_t)f32_to_bf16(a0.w * wf[0].w) << 16);
-        xr[p].z = (uint32_t)f32_to_bf16(a1.x * wf[1].x) | ((uint32_t)f32_to_bf16(a1.y * wf[1].y) << 16);
-        xr[p].w = (uint32_t)f32_to_bf16(a1.z * wf[1].z) | ((uint32_t)f32_to_bf16(a1.w * wf[1].w) << 16);
-      }
       if (row < 16 * MT) *reinterpret_cast<uint4*>(lds + row * ROW_B + ((x_col ^ (row & 7)) * 16)) = xr[p];
     }
   };
@@ -215,24 +164,6 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   }
 #undef SK_STEP
 
-  if (XNORM) {
-    // a wave stages one row per pass: rows (wave / (XV/64)) + p * ROWS_PASS; XV/64 waves share a row
-    constexpr int WPR = XV / 64;
-#pragma unroll
-    for (int p = 0; p < PASSES; ++p) {
-      const float t = wave_sum(ss[p]);
-      if (lane == 0) s_ss[wave][p] = t;
-    }
-    __syncthreads();
-    if (tid < 16 * MT) {
-      const int p = tid / ROWS_PASS, w0 = (tid % ROWS_PASS) * WPR;
-      float t = 0.f;
-#pragma unroll
-      for (int w = 0; w < WPR; ++w) t += s_ss[w0 + w][p];
-      s_inv[tid] = 1.0f / sqrtf(t / (float)K + norm.eps);
-    }
-  }
-
   // ---- add the partial sums of the 8 waves in order, apply the epilogue, store: one output tile
   // of every row group a round (a gate and its up tile together), so that the buffer stays small
   float* red = reinterpret_cast<float*>(lds);
@@ -268,10 +199,9 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
         gsum[0] += pg.x; gsum[1] += pg.y; gsum[2] += pg.z; gsum[3] += pg.w;
         usum[0] += pu.x; usum[1] += pu.y; usum[2] += pu.z; usum[3] += pu.w;
       }
-      const float scale = XNORM ? s_inv[mt * 16 + (ln & 15)] : 1.0f;
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float gt = bf16_to_f32(f32_to_bf16(gsum[e] * scale)), up = bf16_to_f32(f32_to_bf16(usum[e] * scale));
+        const float gt = bf16_to_f32(f32_to_bf16(gsum[e])), up = bf16_to_f32(f32_to_bf16(usum[e]));
         v[e] = up * gt / (1.0f + expf(-gt));
       }
       n = ((blockIdx.x * WN + w_n) * OUT_RT + ort) * 16 + 4 * (ln >> 4);
@@ -283,9 +213,8 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
             red + (((w * WN + w_n) * MT + mt) * 64 + ln) * 4);
         sum[0] += p.x; sum[1] += p.y; sum[2] += p.z; sum[3] += p.w;
       }
-      const float scale = XNORM ? s_inv[mt * 16 + (ln & 15)] : 1.0f;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] = sum[e] * scale;
+      for (int e = 0; e < 4; ++e) v[e] = sum[e];
       n = ((blockIdx.x * WN + w_n) * RT + ort) * 16 + 4 * (ln >> 4);
     }
     const int m = mt * 16 + (ln & 15);
@@ -361,7 +290,6 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
 
 struct SkinnyArgs {
   const bf16_t* X;
-  SkinnyNorm norm;
   const bf16_t* W;
   void* C;
   int M, N, K, ldw, n_out;     // ldw: elements between rows of W (a multiple of 8, at least K)
@@ -369,26 +297,26 @@ struct SkinnyArgs {
   SkinnyRope rope;
 };
 
-template <int MT, int RT, int WN, int G, int EPI, bool XNORM, typename OutT>
+template <int MT, int RT, int WN, int G, int EPI, typename OutT>
 static int launch_skinny(const SkinnyArgs& a) {
   const int rows = (EPI == SK_EPI_SWIGLU) ? a.n_out : a.N;
   const int tiles = (rows + 15) / 16;
   constexpr int OUT_RT = (EPI == SK_EPI_SWIGLU) ? RT / 2 : RT;
   const int blocks = (tiles + OUT_RT * WN - 1) / (OUT_RT * WN);
-  gemm_skinny_kernel<MT, RT, WN, G, EPI, XNORM, OutT><<<blocks, WN * SK_WK * 64, 0, a.stream>>>(
-      a.X, a.norm, a.W, (OutT*)a.C, a.M, a.N, a.K, a.ldw, a.n_out, a.rope);
+  gemm_skinny_kernel<MT, RT, WN, G, EPI, OutT><<<blocks, WN * SK_WK * 64, 0, a.stream>>>(
+      a.X, a.W, (OutT*)a.C, a.M, a.N, a.K, a.ldw, a.n_out, a.rope);
   return llm_launch_status();
 }
 
 template <int MT, int EPI, typename OutT>
 static int pick_rows(const SkinnyArgs& a) {
   if constexpr (EPI == SK_EPI_SWIGLU) {
-    if (a.n_out >= 8192) return launch_skinny<MT, 4, 1, 1, EPI, false, OutT>(a);
-    return launch_skinny<MT, 2, 1, 1, EPI, false, OutT>(a);
+    if (a.n_out >= 8192) return launch_skinny<MT, 4, 1, 1, EPI, OutT>(a);
+    return launch_skinny<MT, 2, 1, 1, EPI, OutT>(a);
   } else {
-    if (a.N >= 8192) return launch_skinny<MT, 2, 2, 1, EPI, false, OutT>(a);
-    if (a.N >= 6144) return launch_skinny<MT, 2, 1, 1, EPI, false, OutT>(a);
-    return launch_skinny<MT, 1, 1, 1, EPI, false, OutT>(a);
+    if (a.N >= 8192) return launch_skinny<MT, 2, 2, 1, EPI, OutT>(a);
+    if (a.N >= 6144) return launch_skinny<MT, 2, 1, 1, EPI, OutT>(a);
+    return launch_skinny<MT, 1, 1, 1, EPI, OutT>(a);
   }
 }
 
@@ -396,18 +324,13 @@ template <int EPI, typename OutT>
 static int pick_shape(const SkinnyArgs& a) {
   constexpr int RT = (EPI == SK_EPI_SWIGLU) ? 2 : 1;
   const int mt = (a.M + 15) / 16;
-  if (a.norm.x != nullptr) {
-    if (mt != 1) return LLM_ERR_ARG;
-    if constexpr (EPI != SK_EPI_ACCUM) return launch_skinny<1, RT, 1, 2, EPI, true, OutT>(a);
-    return LLM_ERR_ARG;
-  }
   switch (mt) {
     case 1:
       // a long K with few rows of W: more of each row in flight per wave
       if constexpr (RT == 1) {
-        if (a.K >= 4096 && a.N <= 4096) return launch_skinny<1, RT, 1, 4, EPI, false, OutT>(a);
+        if (a.K >= 4096 && a.N <= 4096) return launch_skinny<1, RT, 1, 4, EPI, OutT>(a);
       }
-      return launch_skinny<1, RT, 1, 2, EPI, false, OutT>(a);
+      return launch_skinny<1, RT, 1, 2, EPI, OutT>(a);
     // More rows of W per block where W has rows enough to fill the GPU with such blocks: the rows
     // of X are then staged once for 64 rows of W instead of 16.
     case 2: return pick_rows<2, EPI, OutT>(a);
@@ -420,26 +343,16 @@ static int pick_shape(const SkinnyArgs& a) {
 // Rows of W lie ldw elements apart (ldw >= K, a multiple of 8); ldw == 0 says that W is the
 // tiled copy that llm_pack_weight makes.
 // C[M, N] (epilogue 0: stored as out_dtype; 2: added into the float32 C) or C[M, N/2] (epilogue 1,
-// SwiGLU over W = [Wg; Wu], N/2 a multiple of 16) from X[M, K] and W[N, K].  X is bfloat16, or,
-// with norm_x given (M <= 16), the rows `norm_rows` of the float32 matrix norm_x, RMS-normalised
-// with norm_weight and norm_eps on the way.
-extern "C" int llm_gemm_skinny_bf16(const void* X, const float* norm_x, const float* norm_weight,
-                                    float norm_eps, const int* norm_rows, const void* W, void* C,
+// SwiGLU over W = [Wg; Wu], N/2 a multiple of 16) from X[M, K] and W[N, K].  X is bfloat16.
+extern "C" int llm_gemm_skinny_bf16(const void* X, const void* W, void* C,
                                     int epilogue, int out_dtype, int M, int N, int K, int ldw,
                                     hipStream_t stream) {
   if (M <= 0 || N <= 0) return LLM_OK;
   if (M > 64 || K <= 0 || (K & 7) || (ldw != 0 && (ldw < K || (ldw & 7)))) return LLM_ERR_ARG;
-  const void* x = norm_x ? (const void*)norm_x : X;
-  if (x == nullptr || W == nullptr || C == nullptr) return LLM_ERR_ARG;
-  if ((((uintptr_t)x) | ((uintptr_t)W) | ((uintptr_t)C)) & 15) return LLM_ERR_ARG;
-  if (norm_x && (norm_weight == nullptr || (((uintptr_t)norm_weight) & 15) || M > 16 || !(norm_eps >= 0.f)))
-    return LLM_ERR_ARG;
+  if (X == nullptr || W == nullptr || C == nullptr) return LLM_ERR_ARG;
+  if ((((uintptr_t)X) | ((uintptr_t)W) | ((uintptr_t)C)) & 15) return LLM_ERR_ARG;
   SkinnyArgs a;
   a.X = (const bf16_t*)X;
-  a.norm.x = norm_x;
-  a.norm.weight = norm_weight;
-  a.norm.rows = norm_rows;
-  a.norm.eps = norm_eps;
   a.W = (const bf16_t*)W;
   a.C = C;
   a.M = M;
@@ -466,8 +379,7 @@ extern "C" int llm_gemm_skinny_bf16(const void* X, const float* norm_x, const fl
 // The stacked q|k|v projection with the rotary epilogue (see the head of this file): rotated q as
 // bfloat16 [M, n_heads * hd] to `q_out`, k and v to the cache if write_kv.  N is
 // (n_heads + 2 n_kv) * hd with write_kv, else n_heads * hd; hd a multiple of 16, rot_dim even.
-extern "C" int llm_gemm_skinny_rope_bf16(const void* X, const float* norm_x, const float* norm_weight,
-                                         float norm_eps, const int* norm_rows, const void* W,
+extern "C" int llm_gemm_skinny_rope_bf16(const void* X, const void* W,
                                          const float* bias, void* q_out, int M, int K, int ldw, int n_heads,
                                          int n_kv, int hd, const float* cos_t, const float* sin_t,
                                          int rot_dim, const int* tok_pos, const int* tok_seq,
@@ -478,20 +390,14 @@ extern "C" int llm_gemm_skinny_rope_bf16(const void* X, const float* norm_x, con
   if (M > 64 || K <= 0 || (K & 7) || (ldw != 0 && (ldw < K || (ldw & 7))) || n_heads <= 0 || n_kv < 0 || hd <= 0 || (hd & 15) || rot_dim < 0 ||
       rot_dim > hd || (rot_dim & 1) || page_size != 64)
     return LLM_ERR_ARG;
-  const void* x = norm_x ? (const void*)norm_x : X;
-  if (x == nullptr || W == nullptr || q_out == nullptr || tok_pos == nullptr) return LLM_ERR_ARG;
-  if ((((uintptr_t)x) | ((uintptr_t)W) | ((uintptr_t)q_out)) & 15) return LLM_ERR_ARG;
-  if (norm_x && (norm_weight == nullptr || (((uintptr_t)norm_weight) & 15) || M > 16)) return LLM_ERR_ARG;
+  if (X == nullptr || W == nullptr || q_out == nullptr || tok_pos == nullptr) return LLM_ERR_ARG;
+  if ((((uintptr_t)X) | ((uintptr_t)W) | ((uintptr_t)q_out)) & 15) return LLM_ERR_ARG;
   if (rot_dim > 0 && (cos_t == nullptr || sin_t == nullptr)) return LLM_ERR_ARG;
   if (write_kv && (!k_pages || !v_pages || !table || !seq_slot || !tok_seq || n_kv <= 0 ||
                    ((((uintptr_t)k_pages) | ((uintptr_t)v_pages)) & 7)))
     return LLM_ERR_ARG;
   SkinnyArgs a;
   a.X = (const bf16_t*)X;
-  a.norm.x = norm_x;
-  a.norm.weight = norm_weight;
-  a.norm.rows = norm_rows;
-  a.norm.eps = norm_eps;
   a.W = (const bf16_t*)W;
   a.C = q_out;
   a.M = M;

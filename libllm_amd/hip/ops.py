@@ -35,13 +35,13 @@ _SIGNATURES = {
     "llm_add_bias": [_vp, _i, _vp, _i, _i, _vp],
     "llm_rope_kv_write": [_vp, _i, _i, _vp, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp,
                           _vp, _i, _i, _i, _i, _vp],
-    "llm_gemm_skinny_rope_bf16": [_vp, _vp, _vp, _f, _vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _i,
+    "llm_gemm_skinny_rope_bf16": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _i,
                                   _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _vp],
     "llm_pack_weight": [_vp, _vp, _i, _i, _i, _vp],
     "llm_gemm_f32": [_vp, _vp, _vp, _i, _i, _i, _vp],
     "llm_attention_ref": [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
                           _f, _i, _vp],
-    "llm_gemm_skinny_bf16": [_vp, _vp, _vp, _f, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "llm_gemm_skinny_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "llm_attention_mfma_supported": [_i],
     "llm_attention_prefill_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i,
                                    _i, _i, _f, _i, _vp],
@@ -171,8 +171,6 @@ class HipOps:
         return out
 
     SKINNY_ROWS = 64        # most rows the streaming matrix product takes at once
-    NORM_ROWS = 16          # most rows for which the norm is fused into the product
-    NORM_COLS = 4096        # and most rows of the weight
     DECODE_BLOCKS = 768     # blocks of the decode attention grid beyond which sequences are not split further
     _EPI_NONE, _EPI_SWIGLU, _EPI_ACCUM = 0, 1, 2
 
@@ -209,8 +207,9 @@ class HipOps:
 
     def normed(self, res, weight, eps, rows=None):
         """Rows of the float32 stream ``res`` that are to be RMS-normalised: a record that
-        ``linear`` and ``linear_swiglu`` take in place of a matrix, fusing the norm into the
-        product where they can and running the norm kernel first where they cannot."""
+        ``linear``, ``linear_swiglu`` and ``qkv_rope`` take in place of a matrix: they run the
+        norm kernel on just these rows, in the dtype they need.  (The norm fused into the product
+        itself was measured and lost: every block then normalises the rows again.)"""
         return NormedRows(res, weight, float(eps), rows)
 
     def _materialise(self, x, dtype):
@@ -224,24 +223,17 @@ class HipOps:
                 and w.stride(0) % 8 == 0):
             return False
         if isinstance(x, NormedRows):
-            # every block normalises the rows itself: worth it only while the blocks are few
-            return (m <= self.NORM_ROWS and w.shape[0] <= self.NORM_COLS
-                    and x.res.data_ptr() % 16 == 0 and x.weight.data_ptr() % 16 == 0)
+            return False                     # the norm kernel runs first; the product takes its rows
         return x.dtype == torch.bfloat16 and x.data_ptr() % 16 == 0
 
     def _skinny(self, x, w, out, epilogue, m0=0, mm=None):
-        """Launches the skinny kernel on rows m0 .. m0+mm of x (a matrix or NormedRows)."""
+        """Launches the skinny kernel on rows m0 .. m0+mm of the bfloat16 matrix x."""
         n, k = w.shape
-        if isinstance(x, NormedRows):
-            xp, nx, nw, eps = None, x.res.data_ptr(), x.weight.data_ptr(), x.eps
-            rows = None if x.rows is None else x.rows.data_ptr()
-            mm = x.n_rows
-        else:
-            xp, nx, nw, eps, rows = x.data_ptr() + m0 * k * 2, None, None, 0.0, None
+        xp = x.data_ptr() + m0 * k * 2
         width = n // 2 if epilogue == self._EPI_SWIGLU else n
         wptr, ldw = self._streamed(w)
         self._check(self.lib.llm_gemm_skinny_bf16(
-            xp, nx, nw, eps, rows, wptr, out.data_ptr() + m0 * width * out.element_size(),
+            xp, wptr, out.data_ptr() + m0 * width * out.element_size(),
             epilogue, _code(out.dtype), mm, n, k, ldw, self._stream()), "gemm_skinny_bf16")
 
     def linear(self, x, w, bias, out_dtype, residual=None):
@@ -348,7 +340,7 @@ class HipOps:
         fused = (dtype == torch.bfloat16 and (adjacent or rot_dim == 0) and hd % 16 == 0
                  and m <= self.SKINNY_ROWS and m == ctx.n_tokens
                  and (not write or (kv is not None and kv.k_pages.dtype == torch.bfloat16)))
-        if fused and lazy and not (m <= self.NORM_ROWS and n <= self.NORM_COLS):
+        if fused and lazy:
             x, lazy = self._materialise(x, dtype), False
         if fused and self._skinny_ok(x, w, m, k):
             self._weight(self._plain(w), "qkv weight")
@@ -371,17 +363,11 @@ class HipOps:
                 self._check_kv(kv, n_kv, hd, torch.bfloat16)
                 kptr, vptr, tptr = kv.k_pages.data_ptr(), kv.v_pages.data_ptr(), kv.block_table.data_ptr()
                 stride = kv.block_table.shape[1]
-            if lazy:
-                self._dev(x.res, "residual stream", torch.float32)
-                self._dev(x.weight, "norm weight", torch.float32, (k,))
-                xp, nx, nw, eps = None, x.res.data_ptr(), x.weight.data_ptr(), x.eps
-                rows = None if x.rows is None else x.rows.data_ptr()
-            else:
-                xp, nx, nw, eps, rows = self._dev(x, "qkv input", torch.bfloat16), None, None, 0.0, None
+            xp = self._dev(x, "qkv input", torch.bfloat16)
             q = torch.empty((m, n_heads * hd), dtype=torch.bfloat16, device=self.device)
             wptr, ldw = self._streamed(w)
             self._check(self.lib.llm_gemm_skinny_rope_bf16(
-                xp, nx, nw, eps, rows, wptr, bptr, q.data_ptr(), m, k, ldw, n_heads, n_kv, hd,
+                xp, wptr, bptr, q.data_ptr(), m, k, ldw, n_heads, n_kv, hd,
                 cptr, sptr, rot_dim, ctx.tok_pos.data_ptr(), ctx.tok_seq.data_ptr(),
                 ctx.seq_slot.data_ptr(), tptr, stride, kptr, vptr, 64, 1 if write else 0,
                 self._stream()), "gemm_skinny_rope_bf16")

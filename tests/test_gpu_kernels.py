@@ -167,8 +167,7 @@ def test_gemm_skinny_refuses(ops):
     out = ops.linear(x, w, None, torch.bfloat16)
     assert close(out, x.double() @ w.double().t(), torch.bfloat16)
     c = torch.empty((2, 16), dtype=torch.bfloat16, device="cuda")
-    st = ops.lib.llm_gemm_skinny_bf16(x.data_ptr(), None, None, 0.0, None, w.data_ptr(), c.data_ptr(),
-                                      0, 1, 2, 16, 12, 12, 0)
+    st = ops.lib.llm_gemm_skinny_bf16(x.data_ptr(), w.data_ptr(), c.data_ptr(), 0, 1, 2, 16, 12, 12, 0)
     assert st == 1                                        # refused, not wrong
 
 
@@ -245,9 +244,9 @@ def test_gemm_skinny_adds_into_the_stream(ops, m, nk):
 @pytest.mark.parametrize("m", [1, 3, 8, 16, 20])
 @pytest.mark.parametrize("nk", [(16, 8), (300, 520), (3072, 2048), (72, 1032)])
 @pytest.mark.parametrize("gather", [False, True])
-def test_gemm_skinny_with_fused_norm(ops, m, nk, gather):
-    """A product over rows that are RMS-normalised on the way; beyond 16 rows the norm kernel
-    runs first.  Against the plain formulas, and against the unfused kernels."""
+def test_products_of_rows_still_to_be_normalised(ops, m, nk, gather):
+    """A product over a ``normed`` record: the norm kernel runs on just those rows, then the
+    product.  Against the plain formulas, and against the two steps called one by one."""
     n, k = nk
     stream = rnd((m + 3, k), torch.float32, 33, 7.0).cuda()
     stream[0] *= 1e-3                                      # rows of very different size
@@ -368,7 +367,7 @@ def pair_order(n_heads, n_kv, hd, rot):
 @pytest.mark.parametrize("seqs", [[(2, 0, 5), (0, 61, 9), (1, 130, 1)], [(1, 63, 1), (0, 0, 1), (2, 200, 1)]])
 def test_projection_with_rotation_and_cache_write(ops, dtype, shape, bias, seqs):
     """The q|k|v projection, rotation and cache write in one call (one kernel for few rows in
-    bfloat16, with and without a fused norm) against the plain formulas on the rows in their
+    bfloat16, from a matrix and from rows still to be normalised) against the plain formulas on the rows in their
     natural order; the two pairings hold the same numbers in different places."""
     n_heads, n_kv, hd, rot = shape
     k_in = 72
