@@ -136,8 +136,9 @@ class Mixer(Part):
 
     Two optional abilities, off unless the class sets them (they apply to feed-forwards too):
     ``takes_normed = True``: ``x`` may be the record that ``ops.normed`` returns instead of a
-    matrix; the part hands it to ``ops.linear`` / ``ops.linear_swiglu`` only, which fuse the norm
-    into the product.  ``adds_to_stream = True``: ``forward`` takes a keyword ``residual`` (the
+    matrix; the part hands it to ``ops.linear`` / ``ops.linear_swiglu`` / ``ops.qkv_rope`` only,
+    which decide how the norm is run (on which rows, in which dtype, in which kernel).
+    ``adds_to_stream = True``: ``forward`` takes a keyword ``residual`` (the
     float32 stream) and may add its result into it, returning None.
     """
     takes_normed = False
@@ -166,8 +167,8 @@ class Norm(Part):
     """``add_norm(ctx, stream, rows)``: adds ``stream.delta`` (if any) into ``stream.res`` in
     32-bit, then returns the normalised rows in the activation dtype.  With ``rows`` (int32
     indices) only those rows are normalised and returned, in that order.  With ``lazy`` a norm
-    that can be fused into a matrix product may return ``ctx.ops.normed(...)`` instead, when
-    nothing is left to add."""
+    whose consumer ``takes_normed`` may return ``ctx.ops.normed(...)`` instead, when nothing is
+    left to add: the record names the rows, and the product that takes it runs the norm."""
 
     def add_norm(self, ctx: StepContext, stream: Stream, rows=None, lazy=False) -> torch.Tensor:
         raise NotImplementedError
