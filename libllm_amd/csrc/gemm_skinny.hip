@@ -326,9 +326,11 @@ static int pick_shape(const SkinnyArgs& a) {
   const int mt = (a.M + 15) / 16;
   switch (mt) {
     case 1:
-      // a long K with few rows of W: more of each row in flight per wave
+      // few rows of W (so few blocks): more of each row in flight per wave.  Whole engines compared
+      // in one process: 1 to 1.5 % of a decode step at the 1B shape, nothing lost at 3B and 8B;
+      // for the 6,144 rows of the 8B shape's q|k|v product it costs 2.5 %.
       if constexpr (RT == 1) {
-        if (a.K >= 4096 && a.N <= 4096) return launch_skinny<1, RT, 1, 4, EPI, OutT>(a);
+        if (a.N <= 4096) return launch_skinny<1, RT, 1, 4, EPI, OutT>(a);
       }
       return launch_skinny<1, RT, 1, 2, EPI, OutT>(a);
     // More rows of W per block where W has rows enough to fill the GPU with such blocks: the rows

@@ -112,7 +112,7 @@ def test_linear_bias_and_mixed_dtypes(ops):
 
 
 @pytest.mark.parametrize("m", [1, 3, 16, 17, 33, 64])
-@pytest.mark.parametrize("nk", [(16, 8), (24, 136), (1000, 2048), (2050, 264), (40, 4104)])
+@pytest.mark.parametrize("nk", [(16, 8), (24, 136), (1000, 2048), (2050, 264), (40, 4104), (4112, 72)])
 @pytest.mark.parametrize("out_dtype", DTYPES)
 def test_gemm_skinny(ops, m, nk, out_dtype):
     n, k = nk
@@ -171,7 +171,7 @@ def test_gemm_skinny_refuses(ops):
     assert st == 1                                        # refused, not wrong
 
 
-@pytest.mark.parametrize("nk", [(16, 8), (300, 520), (2050, 264), (3072, 2048), (40, 4104)])
+@pytest.mark.parametrize("nk", [(16, 8), (300, 520), (2050, 264), (3072, 2048), (40, 4104), (4128, 136)])
 def test_prepared_weight_gives_the_same_bits(ops, nk):
     """The copy tiled for the matrix cores holds the same numbers: every product for few rows
     returns the same bits from it as from the matrix, and the product for many rows reads the matrix."""
