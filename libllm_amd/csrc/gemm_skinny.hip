@@ -311,7 +311,9 @@ static int launch_skinny(const SkinnyArgs& a) {
 template <int MT, int EPI, typename OutT>
 static int pick_rows(const SkinnyArgs& a) {
   if constexpr (EPI == SK_EPI_SWIGLU) {
-    if (a.n_out >= 8192) return launch_skinny<MT, 4, 1, 1, EPI, OutT>(a);
+    // four tiles a block pay from 33 rows of X on; at 17 to 32 rows two are 2 % of a decode step
+    // faster (whole engines compared in one process, 1B and 8B shapes)
+    if (a.n_out >= 8192 && MT >= 3) return launch_skinny<MT, 4, 1, 1, EPI, OutT>(a);
     return launch_skinny<MT, 2, 1, 1, EPI, OutT>(a);
   } else {
     if (a.N >= 8192) return launch_skinny<MT, 2, 2, 1, EPI, OutT>(a);

@@ -163,23 +163,23 @@ def _decode_rows(engine, requests, n_last):
 
 
 def test_padding_changes_nothing(models):
-    """Three sequences decode through the graph captured for four rows, the fourth row being
+    """Five sequences decode through the graph captured for six rows, the sixth row being
     padding.  In 32-bit the same bits come out without graphs (no padding row at all); in
-    bfloat16 the same bits come out when the fourth row is a real sequence."""
+    bfloat16 the same bits come out when the sixth row is a real sequence."""
     from libllm_amd.runtime import load_engine
     path, cfg, weights = models["A"]
-    three = make_requests(cfg, [9, 70, 31], seed=12)
-    four = dict(three, extra=make_requests(cfg, [50], seed=13)["r0"])
+    five = make_requests(cfg, [9, 70, 31, 12, 44], seed=12)
+    six = dict(five, extra=make_requests(cfg, [50], seed=13)["r0"])
     padded = load_engine(path, dtype="float32", max_tokens=1024, use_graphs=True)
     plain_path = load_engine(path, dtype="float32", max_tokens=1024, use_graphs=False)
-    a, b = _decode_rows(padded, three, 4), _decode_rows(plain_path, three, 4)
-    assert len(padded._graphs) == 1 and not plain_path._graphs
+    a, b = _decode_rows(padded, five, 4), _decode_rows(plain_path, five, 4)
+    assert [k[0] for k in padded._graphs] == [6] and not plain_path._graphs
     assert np.array_equal(a, b)
-    e3 = load_engine(path, dtype="bfloat16", max_tokens=1024, use_graphs=True)
-    e4 = load_engine(path, dtype="bfloat16", max_tokens=1024, use_graphs=True)
-    a, b = _decode_rows(e3, three, 4), _decode_rows(e4, four, 4)
-    assert [k[0] for k in e3._graphs] == [4] and [k[0] for k in e4._graphs] == [4]
-    assert np.array_equal(a, b[:, :3])
+    e5 = load_engine(path, dtype="bfloat16", max_tokens=1024, use_graphs=True)
+    e6 = load_engine(path, dtype="bfloat16", max_tokens=1024, use_graphs=True)
+    a, b = _decode_rows(e5, five, 4), _decode_rows(e6, six, 4)
+    assert [k[0] for k in e5._graphs] == [6] and [k[0] for k in e6._graphs] == [6]
+    assert np.array_equal(a, b[:, :5])
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
