@@ -171,6 +171,7 @@ class HipOps:
         return out
 
     SKINNY_ROWS = 64        # most rows the streaming matrix product takes at once
+    ACCUM_ROWS = 32         # most rows for which a product adds into the stream itself; beyond, the library's
     DECODE_BLOCKS = 768     # blocks of the decode attention grid beyond which sequences are not split further
     _EPI_NONE, _EPI_SWIGLU, _EPI_ACCUM = 0, 1, 2
 
@@ -252,7 +253,7 @@ class HipOps:
             self._dev(x.weight, "norm weight", torch.float32, (k,))
         else:
             self._dev(x, "linear input")
-        if self._skinny_ok(x, w, m, k) and bias is None:
+        if self._skinny_ok(x, w, m, k) and bias is None and not (residual is not None and m > self.ACCUM_ROWS):
             if residual is not None and m <= self.SKINNY_ROWS:
                 self._dev(residual, "residual stream", torch.float32, (m, n))
                 self._skinny(x, w, residual, self._EPI_ACCUM, 0, m)

@@ -226,19 +226,29 @@ def test_weight_rows_may_lie_apart(ops):
     assert torch.equal(ops.linear_swiglu(x, wide2[:, :1024]), ops.linear_swiglu(x, w2))
 
 
-@pytest.mark.parametrize("m", [1, 5, 16, 40])
+@pytest.mark.parametrize("m", [1, 5, 16, 32, 40])
 @pytest.mark.parametrize("nk", [(16, 8), (300, 520), (2048, 2048), (72, 4104)])
-def test_gemm_skinny_adds_into_the_stream(ops, m, nk):
+def test_gemm_skinny_adds_into_the_stream(ops, monkeypatch, m, nk):
+    """Up to ``ACCUM_ROWS`` rows the product adds into the stream itself and returns None; beyond,
+    the product is returned for the caller to add and the stream is left alone.  Forced to 64
+    the kernel adds for 40 rows too."""
     n, k = nk
     x = rnd((m, k), torch.bfloat16, 30).cuda()
     w = rnd((n, k), torch.bfloat16, 31).cuda()
-    res = rnd((m, n), torch.float32, 32, 5.0).cuda()
-    ref = res.double() + x.double() @ w.double().t()
-    assert ops.linear(x, w, None, torch.bfloat16, residual=res) is None
-    assert max_err(res, ref) < 2e-6
-    plain = ops.linear(x, w, None, torch.float32)          # the same sums as the plain product
-    again = rnd((m, n), torch.float32, 32, 5.0).cuda()
-    assert torch.equal(res, again + plain)
+    ref = x.double() @ w.double().t()
+    for limit in (ops.ACCUM_ROWS, 64):
+        monkeypatch.setattr(ops, "ACCUM_ROWS", limit)
+        res = rnd((m, n), torch.float32, 32, 5.0).cuda()
+        before = res.clone()
+        out = ops.linear(x, w, None, torch.bfloat16, residual=res)
+        if m > limit:
+            assert out is not None and torch.equal(res, before)
+            assert close(out, ref, torch.bfloat16)
+            continue
+        assert out is None
+        assert max_err(res, before.double() + ref.cuda()) < 2e-6
+        plain = ops.linear(x, w, None, torch.float32)          # the same sums as the plain product
+        assert torch.equal(res, before + plain)
 
 
 @pytest.mark.parametrize("m", [1, 3, 8, 16, 20])

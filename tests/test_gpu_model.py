@@ -204,6 +204,41 @@ def test_batch_order_changes_nothing(models, dtype):
         assert_logits_close(alone[:, 0], a[:, 1].astype(np.float64), dtype, "alone against in a batch")
 
 
+@pytest.mark.parametrize("widths", [(2048, 32, 64, 8192), (4096, 32, 128, 14336)])
+def test_library_products_inside_decode_graphs(widths):
+    """From 33 rows on the products that add into the stream are the library's, also inside the
+    captured decode graphs.  Layers of real width (where the library picks the kernels it uses for
+    large products): a graph of 48 rows replayed twelve times, an engine without graphs stepping
+    beside it, other work and a synchronisation between the replays; every replay gives the bits
+    of the eager step."""
+    import torch
+    from libllm_amd.config import config_from_dict
+    from libllm_amd.engine import StepEntry
+    from libllm_amd.runtime import random_engine
+    hidden, heads, head_dim, inter = widths
+    cfg = config_from_dict({
+        "model_type": "llama", "num_hidden_layers": 2, "hidden_size": hidden, "num_attention_heads": heads,
+        "num_key_value_heads": 8, "head_dim": head_dim, "intermediate_size": inter, "vocab_size": 4096,
+        "rope_theta": 500000.0, "rms_norm_eps": 1e-5, "tie_word_embeddings": True,
+        "max_position_embeddings": 4096, "hidden_act": "silu", "bos_token_id": 1, "eos_token_id": 2})
+    rng = np.random.default_rng(3)
+    prompts = {i: rng.integers(3, 4096, size=int(n)).tolist() for i, n in enumerate(rng.integers(3, 40, size=40))}
+    engines = [random_engine(cfg, seed=5, dtype="bfloat16", max_tokens=8192, use_graphs=g) for g in (True, False)]
+    assert engines[0].ops.ACCUM_ROWS < 40 <= engines[0].ops.SKINNY_ROWS
+    for e in engines:
+        e.step([StepEntry(r, t, []) for r, t in prompts.items()])
+    scratch = torch.randn((512, 512), device="cuda")
+    for k in range(12):
+        toks = {r: int((7 * r + 13 * k) % 4096) for r in prompts}
+        outs = []
+        for e in engines:
+            outs.append(e.step([StepEntry(r, [toks[r]], [0]) for r in prompts]).clone())
+            scratch = (scratch @ scratch).clamp_(-1, 1)         # the program's own eager work
+            torch.cuda.synchronize()
+        assert torch.equal(outs[0], outs[1]), "replay %d differs from the eager step" % k
+    assert [key[0] for key in engines[0]._graphs] == [48] and not engines[1]._graphs
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_trace_run_program(models, tmp_path, dtype):
     """bin/trace_run as a user starts it: a child process fed through its standard input, one
