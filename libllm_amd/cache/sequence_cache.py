@@ -31,6 +31,15 @@ def pages_for(n_tokens: int, page: int = PAGE) -> int:
     return (n_tokens + page - 1) // page
 
 
+
+def _send(t: torch.Tensor, device) -> torch.Tensor:
+    """``t`` on ``device``.  To a GPU it goes through pinned memory and without waiting: a copy
+    from pageable memory holds the host until the stream gets to it, and rows of the table change
+    whenever a sequence enters a new page, which with unequal lengths is on most steps."""
+    if torch.device(device).type == "cuda":
+        return t.pin_memory().to(device, non_blocking=True)
+    return t.to(device)
+
 class CacheGroup:
     def __init__(self, need: CacheNeed, entries: List[int], n_pages: int, n_slots: int,
                  pages_per_seq: int, dtype, device):
@@ -108,8 +117,8 @@ class CacheGroup:
         if not self.dirty:
             return
         rows = sorted(self.dirty)
-        idx = torch.tensor(rows, dtype=torch.long, device=self.table.device)
-        data = torch.from_numpy(self.table_host[rows]).to(self.table.device)
+        idx = _send(torch.tensor(rows, dtype=torch.long), self.table.device)
+        data = _send(torch.from_numpy(self.table_host[rows]), self.table.device)
         self.table.index_copy_(0, idx, data)
         self.dirty.clear()
 

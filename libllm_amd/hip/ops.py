@@ -127,7 +127,9 @@ class HipOps:
         return t.data_ptr()
 
     def upload_int32(self, arr: np.ndarray) -> torch.Tensor:
-        return torch.from_numpy(np.ascontiguousarray(arr, dtype=np.int32)).to(self.device)
+        """The array on the device, sent through pinned memory without waiting for the stream."""
+        host = torch.from_numpy(np.ascontiguousarray(arr, dtype=np.int32)).pin_memory()
+        return host.to(self.device, non_blocking=True)
 
     def capture(self, body):
         """Runs ``body`` once to warm up, then captures it into a HIP graph."""
@@ -489,7 +491,9 @@ class HipOps:
         self._dev(logits, "logits", torch.float32)
         if len(streams) != r or len(counters) != r:
             raise KernelError("sample: one stream and counter per row are needed")
-        keys = torch.tensor([streams, counters], dtype=torch.int64).to(self.device)
+        # through pinned memory and without waiting: a copy from pageable memory holds the host
+        # until the stream gets to it, and the step after this one could not be queued meanwhile
+        keys = torch.tensor([streams, counters], dtype=torch.int64).pin_memory().to(self.device, non_blocking=True)
         out = torch.empty((r,), dtype=torch.int32, device=self.device)
         parts = self.lib.llm_sample_parts(v)
         k_part = self.lib.llm_sample_k_part(v, int(top_k))

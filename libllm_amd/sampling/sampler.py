@@ -76,7 +76,7 @@ class PendingTokens:
         """The device tokens of the given rows, in that order."""
         if list(index) == list(range(self.device.shape[0])):
             return self.device
-        idx = torch.tensor(list(index), dtype=torch.long).to(self.device.device, non_blocking=True)
+        idx = torch.tensor(list(index), dtype=torch.long).pin_memory().to(self.device.device, non_blocking=True)
         return self.device.index_select(0, idx)
 
 
