@@ -33,6 +33,13 @@ class Engine:
     # (2.73 ms a step at the 1B shape against 2.43 in a graph of 48).
     GRAPH_BATCHES = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64)
     GRAPH_MIN_CTX = 1024
+    # Steps that bring whole prompts are captured too, padded to one of these numbers of rows and
+    # of sequences (one sequence is always spare: it takes the padding rows, in the sink slot).  A
+    # shape is captured when it comes the second time, so that a lone prompt does not pay for it.
+    # Queued from the host a prompt of up to some hundred tokens waits for the host, not the device.
+    PROMPT_ROWS = (16, 32, 64, 128, 192, 256, 384, 512, 768, 1024, 1536, 2048)
+    PROMPT_SEQS = (2, 3, 5, 9, 17)
+    PROMPT_SEEN = 2
 
     def __init__(self, model: DecoderModel, ops, dtype: torch.dtype, max_tokens: int,
                  max_slots: Optional[int] = None, use_graphs: bool = True):
@@ -45,6 +52,8 @@ class Engine:
                                    model.spec.max_position, dtype, self.device, max_slots)
         self.use_graphs = bool(use_graphs) and ops.supports_graphs and model.graph_safe()
         self._graphs: Dict[tuple, "_DecodeGraph"] = {}     # (batch bucket, context bucket) -> graph
+        self._prompt_graphs: Dict[tuple, "_PromptGraph"] = {}   # (rows, sequences) -> graph
+        self._prompt_seen: Dict[tuple, int] = {}
         self.steps_run = 0
 
     # ---- requests
@@ -119,8 +128,12 @@ class Engine:
         lens = [len(e.tokens) for e in entries]
         pos0 = [cache.length(s) for s in slots]
         want_all_single = all(n == 1 for n in lens) and all(list(e.want) == [0] for e in entries)
+        graph = None
         if self.use_graphs and want_all_single and len(entries) <= self.GRAPH_BATCHES[-1]:
             logits = self._graph_step(entries, slots, pos0, tokens_device)
+        elif self.use_graphs and tokens_device is None and not all(n == 1 for n in lens) \
+                and (graph := self._prompt_graph(entries, lens)) is not None:
+            logits = graph.run(entries, slots, lens, pos0)
         else:
             ctx, want_rows = self._context(entries, slots, lens, pos0)
             if tokens_device is not None:
@@ -171,6 +184,30 @@ class Engine:
                 ctx._kv[entry] = view
             if entry in self.cache.state:
                 ctx._state[entry] = self.cache.state[entry]
+
+    # ---- whole prompts through a captured graph
+    def _prompt_graph(self, entries, lens):
+        """The captured graph that holds this step, or None if the step runs from the host."""
+        m, b = sum(lens), len(entries)
+        wanted = sum(len(e.want) for e in entries)
+        if m > self.PROMPT_ROWS[-1] or b + 1 > self.PROMPT_SEQS[-1]:
+            return None
+        rows = next(r for r in self.PROMPT_ROWS if r >= m)
+        seqs = next(q for q in self.PROMPT_SEQS if q >= b + 1)
+        # the spare sequence may take all rows but one: its positions must lie within a table row;
+        # the wanted rows must fit the places the graph has for them
+        if rows > self.cache.pages_per_seq * PAGE or wanted > seqs:
+            return None
+        key = (rows, seqs)
+        graph = self._prompt_graphs.get(key)
+        if graph is None:
+            seen = self._prompt_seen.get(key, 0) + 1
+            self._prompt_seen[key] = seen
+            if seen < self.PROMPT_SEEN:
+                return None
+            graph = _PromptGraph(self, rows, seqs)
+            self._prompt_graphs[key] = graph
+        return graph
 
     # ---- decoding one token per sequence through a captured graph
     def _graph_step(self, entries, slots, pos0, tokens_device=None):
@@ -259,3 +296,85 @@ class _DecodeGraph:
             self.static[:len(tokens)].copy_(tokens_device, non_blocking=True)
         self.graph.replay()
         return self.logits[:len(tokens)]
+
+
+class _PromptGraph:
+    """One captured step of exactly ``rows`` tokens in ``seqs`` sequences, any of which may hold
+    past tokens.  The live sequences come first; the next one takes the rows that are left over,
+    at positions 0.. of the sink slot, whose every page is the sink page; the others are empty.
+    ``seqs`` places hold the wanted rows; spare ones ask for row 0.  Kernels read offsets, slots
+    and lengths from device memory; their grids are sized for one sequence of all the rows."""
+
+    RING = 4
+
+    def __init__(self, engine: Engine, rows: int, seqs: int):
+        self.engine, self.rows, self.seqs = engine, rows, seqs
+        ops = engine.ops
+        t, b = rows, seqs
+        self.size = 3 * t + (b + 1) + 3 * b
+        self.ring = [torch.zeros(self.size, dtype=torch.int32, pin_memory=True) for _ in range(self.RING)]
+        self.ring_done = [None] * self.RING
+        self.turn = 0
+        self.static = self.ring[0].to(ops.device)
+        ctx = StepContext(ops, engine.dtype, t, b)
+        o = 0
+        ctx.tokens = self.static[o:o + t]; o += t
+        ctx.tok_pos = self.static[o:o + t]; o += t
+        ctx.tok_seq = self.static[o:o + t]; o += t
+        ctx.seq_start = self.static[o:o + b + 1]; o += b + 1
+        ctx.seq_slot = self.static[o:o + b]; o += b
+        ctx.seq_pos0 = self.static[o:o + b]; o += b
+        self.want_rows = self.static[o:o + b]
+        ctx.max_new = t
+        ctx.max_ctx = engine.cache.pages_per_seq * PAGE
+        ctx.decode = False
+        ctx.captured = True
+        engine._attach_cache(ctx)
+        self.ctx = ctx
+        self._fill([], [], [], [], [])
+        self.logits = None
+        self.graph = ops.capture(self._body)
+
+    def _body(self):
+        self.logits = self.engine.model.forward(self.ctx, self.want_rows)
+
+    def _fill(self, tokens, slots, lens, pos0, want):
+        t, b = self.rows, self.seqs
+        n, m = len(lens), len(tokens)
+        sink = self.engine.cache.sink_slot
+        self.turn = (self.turn + 1) % self.RING
+        if self.ring_done[self.turn] is not None:
+            self.ring_done[self.turn].synchronize()        # its last upload has been read
+        h = self.ring[self.turn].numpy()
+        starts = np.zeros(n + 1, dtype=np.int64)
+        starts[1:] = np.cumsum(lens)
+        tok_seq = np.repeat(np.arange(n, dtype=np.int64), lens)
+        o = 0
+        h[o:o + t] = 0
+        h[o:o + m] = tokens; o += t
+        h[o + m:o + t] = np.arange(t - m)                   # the spare sequence counts from 0
+        if m:
+            h[o:o + m] = np.arange(m) - starts[tok_seq] + np.asarray(pos0, dtype=np.int64)[tok_seq]
+        o += t
+        h[o:o + m] = tok_seq
+        h[o + m:o + t] = n; o += t
+        h[o:o + n + 1] = starts
+        h[o + n + 1:o + b + 1] = t; o += b + 1               # the spare one ends at the last row, the rest are empty
+        h[o:o + b] = sink
+        h[o:o + n] = slots; o += b
+        h[o:o + b] = 0
+        h[o:o + n] = pos0; o += b
+        h[o:o + b] = 0
+        h[o:o + len(want)] = want
+        self.static.copy_(self.ring[self.turn], non_blocking=True)
+        done = torch.cuda.Event()
+        done.record()
+        self.ring_done[self.turn] = done
+
+    def run(self, entries, slots, lens, pos0):
+        starts = np.concatenate([[0], np.cumsum(lens)])
+        want = [int(starts[i]) + int(w) for i, e in enumerate(entries) for w in e.want]
+        tokens = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
+        self._fill(tokens, slots, lens, pos0, want)
+        self.graph.replay()
+        return self.logits[:len(want)] if want else None

@@ -204,6 +204,82 @@ def test_batch_order_changes_nothing(models, dtype):
         assert_logits_close(alone[:, 0], a[:, 1].astype(np.float64), dtype, "alone against in a batch")
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_prompt_steps_through_graphs(models, name, dtype):
+    """Steps that bring whole prompts replay captured graphs, padded to fixed numbers of rows and
+    sequences (here from the first time a shape comes).  Unequal batches, prompts continued over
+    several steps, one wanted row or none, then single tokens that read what the prompts cached:
+    against the plain implementation, and in 32-bit the bits of an engine without graphs."""
+    from libllm_amd.engine import StepEntry
+    from libllm_amd.runtime import load_engine
+    path, cfg, weights = models[name]
+    limit = min(cfg.max_pos, 120)
+    rng = np.random.default_rng(17)
+    eng = load_engine(path, dtype=dtype, max_tokens=4096)
+    eng.PROMPT_SEEN = 1
+    ref = load_engine(path, dtype=dtype, max_tokens=4096, use_graphs=False)
+    for rnd in range(3):                                   # the same shapes again: replays, and slots used again
+        lengths = [int(x) for x in rng.integers(2, limit - 8, size=int(rng.integers(1, 5)))]
+        toks = {i: rng.integers(3, cfg.vocab, size=n + 6).tolist() for i, n in enumerate(lengths)}
+        cut = {i: int(rng.integers(1, n)) for i, n in enumerate(lengths)}
+        steps = [[StepEntry(i, toks[i][:cut[i]], []) for i in toks],                        # nothing wanted
+                 [StepEntry(i, toks[i][cut[i]:lengths[i]], [lengths[i] - cut[i] - 1]) for i in toks]]
+        steps += [[StepEntry(i, [toks[i][lengths[i] + k]], [0]) for i in toks] for k in range(6)]
+        for k, entries in enumerate(steps):
+            a, b = eng.step(entries), ref.step(entries)
+            if k == 0:
+                assert a is None and b is None
+                continue
+            if dtype == "float32":
+                assert torch_equal(a, b), "round %d step %d" % (rnd, k)
+            for j, e in enumerate(entries):
+                upto = (lengths[e.request] if k == 1 else lengths[e.request] + k - 1)
+                want = oracle(name, cfg, weights, toks[e.request][:upto])[-1]
+                assert_logits_close(a[j].cpu().numpy()[None], want[None], dtype, "round %d step %d" % (rnd, k))
+        eng.end(list(toks)); ref.end(list(toks))
+    assert eng._prompt_graphs and not ref._prompt_graphs
+    eng.cache.check()
+
+
+def torch_equal(a, b):
+    import torch
+    return torch.equal(a, b)
+
+
+@pytest.mark.parametrize("rows", [512, 2048])
+def test_library_products_inside_prompt_graphs(rows):
+    """A prompt of real width fills its graph exactly, so that the graph and an engine without
+    graphs run the same kernels, the library's for large products among them: six replays with
+    other prompts, eager work and a synchronisation between them, each the bits of the eager step;
+    then a token for each, which reads the keys and values the graphs wrote."""
+    import torch
+    from libllm_amd.config import config_from_dict
+    from libllm_amd.engine import StepEntry
+    from libllm_amd.runtime import random_engine
+    cfg = config_from_dict({
+        "model_type": "llama", "num_hidden_layers": 2, "hidden_size": 2048, "num_attention_heads": 32,
+        "num_key_value_heads": 8, "head_dim": 64, "intermediate_size": 8192, "vocab_size": 4096,
+        "rope_theta": 500000.0, "rms_norm_eps": 1e-5, "tie_word_embeddings": True,
+        "max_position_embeddings": 4096, "hidden_act": "silu", "bos_token_id": 1, "eos_token_id": 2})
+    engines = [random_engine(cfg, seed=5, dtype="bfloat16", max_tokens=8192, use_graphs=g) for g in (True, False)]
+    engines[0].PROMPT_SEEN = 1
+    rng = np.random.default_rng(8)
+    scratch = torch.randn((512, 512), device="cuda")
+    for k in range(6):
+        prompt = rng.integers(3, 4096, size=rows).tolist()
+        outs, nxt = [], []
+        for e in engines:
+            outs.append(e.step([StepEntry("p", prompt, [rows - 1])]).clone())
+            scratch = (scratch @ scratch).clamp_(-1, 1)
+            torch.cuda.synchronize()
+            nxt.append(e.step([StepEntry("p", [7 + k], [0])]).clone())
+            e.end(["p"])
+        assert torch.equal(outs[0], outs[1]), "replay %d differs from the eager step" % k
+        assert torch.equal(nxt[0], nxt[1]), "the token after replay %d differs" % k
+    assert list(engines[0]._prompt_graphs) == [(rows, 2)] and not engines[1]._prompt_graphs
+
+
 @pytest.mark.parametrize("widths", [(2048, 32, 64, 8192), (4096, 32, 128, 14336)])
 def test_library_products_inside_decode_graphs(widths):
     """From 33 rows on the products that add into the stream are the library's, also inside the
