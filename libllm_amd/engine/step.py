@@ -234,7 +234,10 @@ class _DecodeGraph:
     RING = 4
 
     def __init__(self, engine: Engine, bucket: int, max_ctx: int):
-        self.engine = engine
+        # no reference back to the engine: an engine that is dropped then goes at once, with its
+        # graphs, and not whenever the collector of cycles next runs
+        self.model = engine.model
+        self.sink_slot = engine.cache.sink_slot
         self.bucket = bucket
         ops = engine.ops
         b = bucket
@@ -264,12 +267,12 @@ class _DecodeGraph:
         self.graph = ops.capture(self._body)
 
     def _body(self):
-        self.logits = self.engine.model.forward(self.ctx, self.want_rows)
+        self.logits = self.model.forward(self.ctx, self.want_rows)
 
     def _fill(self, tokens, slots, pos0):
         b = self.bucket
         n = len(tokens)
-        sink = self.engine.cache.sink_slot
+        sink = self.sink_slot
         self.turn = (self.turn + 1) % self.RING
         if self.ring_done[self.turn] is not None:
             self.ring_done[self.turn].synchronize()        # its last upload has been read
@@ -308,7 +311,8 @@ class _PromptGraph:
     RING = 4
 
     def __init__(self, engine: Engine, rows: int, seqs: int):
-        self.engine, self.rows, self.seqs = engine, rows, seqs
+        self.model, self.sink_slot = engine.model, engine.cache.sink_slot     # and no reference back
+        self.rows, self.seqs = rows, seqs
         ops = engine.ops
         t, b = rows, seqs
         self.size = 3 * t + (b + 1) + 3 * b
@@ -336,12 +340,12 @@ class _PromptGraph:
         self.graph = ops.capture(self._body)
 
     def _body(self):
-        self.logits = self.engine.model.forward(self.ctx, self.want_rows)
+        self.logits = self.model.forward(self.ctx, self.want_rows)
 
     def _fill(self, tokens, slots, lens, pos0, want):
         t, b = self.rows, self.seqs
         n, m = len(lens), len(tokens)
-        sink = self.engine.cache.sink_slot
+        sink = self.sink_slot
         self.turn = (self.turn + 1) % self.RING
         if self.ring_done[self.turn] is not None:
             self.ring_done[self.turn].synchronize()        # its last upload has been read

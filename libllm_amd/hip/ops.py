@@ -7,6 +7,7 @@ for them as well, src/flint/cuda/gemm_cublas.cc:160-197); every other operation 
 ``csrc``.
 """
 import ctypes
+import gc
 from typing import List, Optional
 
 import numpy as np
@@ -132,16 +133,28 @@ class HipOps:
         return host.to(self.device, non_blocking=True)
 
     def capture(self, body):
-        """Runs ``body`` once to warm up, then captures it into a HIP graph."""
+        """Runs ``body`` once to warm up, then captures it into a HIP graph.
+
+        The capture is in global mode: runtime calls that free or query device resources are
+        errors anywhere in the process while it lasts, and a finaliser that makes one (of a graph,
+        a pinned buffer, an event) ends the process.  So whatever is dead and waits for the
+        collector goes before the capture begins, and the collector does not run during it."""
         side = torch.cuda.Stream(self.device)
         side.wait_stream(torch.cuda.current_stream(self.device))
         with torch.cuda.stream(side):
             body()
         torch.cuda.current_stream(self.device).wait_stream(side)
         torch.cuda.synchronize(self.device)
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
-            body()
+        gc.collect()
+        collecting = gc.isenabled()
+        gc.disable()
+        try:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                body()
+        finally:
+            if collecting:
+                gc.enable()
         return graph
 
     # ---- operations

@@ -168,3 +168,23 @@ def test_toy_mixer_with_state_of_its_own():
     for rid, toks in (("a", reqs["a"]), ("b", reqs["b"]), ("c", reqs["b"])):   # c reuses a slot: clean state
         ref = toy.toy_oracle(cfg, w, w["model.layers.1.toy.mix.weight"], toks)
         assert err(np.stack(got[rid]), ref) < 1e-4
+
+
+def test_a_dropped_engine_goes_at_once(models):
+    """Nothing an engine owns refers back to it, so dropping it frees it there and then, without
+    the collector of cycles (which may run at any later time, for instance while a graph is being
+    captured, when freeing device resources ends the process)."""
+    import gc
+    import weakref
+    path, cfg, _ = models["A"]
+    gc.collect()
+    gc.disable()
+    try:
+        model = Model(path, dtype="float32", max_tokens=512, ops=CpuOps(), max_batch=3)
+        model.generate([[5, 6, 7], [8, 9]], max_new_tokens=3, temperature=0.0)
+        engine = weakref.ref(model.engine)
+        cache = weakref.ref(model.engine.cache)
+        del model
+        assert engine() is None and cache() is None
+    finally:
+        gc.enable()

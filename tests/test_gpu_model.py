@@ -247,6 +247,40 @@ def torch_equal(a, b):
     return torch.equal(a, b)
 
 
+def test_a_dropped_engine_goes_at_once_with_its_graphs(models):
+    """An engine that has captured graphs of both kinds is freed the moment it is dropped, with
+    the collector of cycles switched off: its graphs hold no reference back to it.  Otherwise it
+    would wait for the collector, which may run while another graph is being captured; the capture
+    is in global mode, and a graph, a pinned buffer or an event freed then ends the process.
+    ``HipOps.capture`` also collects before a capture and keeps the collector off during it."""
+    import gc
+    import weakref
+    import torch
+    from libllm_amd.engine import StepEntry
+    from libllm_amd.runtime import load_engine
+    path, cfg, _ = models["B"]
+    gc.collect()
+    torch.cuda.synchronize()
+    before = torch.cuda.memory_allocated()
+    gc.disable()
+    try:
+        engine = load_engine(path, dtype="bfloat16", max_tokens=1024)
+        engine.PROMPT_SEEN = 1
+        engine.step([StepEntry(i, [5 + i, 6, 7, 8][:2 + i], [1 + i]) for i in range(3)])
+        for k in range(3):
+            engine.step([StepEntry(i, [9 + k], [0]) for i in range(3)])
+        assert engine._graphs and engine._prompt_graphs
+        assert gc.isenabled() is False                      # captures leave the collector as they found it
+        ref = weakref.ref(engine)
+        graphs = [weakref.ref(g) for g in list(engine._graphs.values()) + list(engine._prompt_graphs.values())]
+        del engine
+        assert ref() is None and all(g() is None for g in graphs)
+        torch.cuda.synchronize()
+        assert torch.cuda.memory_allocated() <= before + (1 << 20)
+    finally:
+        gc.enable()
+
+
 @pytest.mark.parametrize("rows", [512, 2048])
 def test_library_products_inside_prompt_graphs(rows):
     """A prompt of real width fills its graph exactly, so that the graph and an engine without
