@@ -149,6 +149,56 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   load_x(0);
   load_w(0, a[0]);
   if (1 < n_chunks) load_w(1, a[1]);
+
+  // What the epilogue needs from memory beside the sums is asked for now, behind the first loads:
+  // a thread finishes at most one group of four outputs per round (ITEMS <= NT), and which one is
+  // known from the start, so its position, cache page and rotation, or the values it adds to,
+  // are in registers by the time the sums are (1 % of a decode step at up to 16 rows).
+  constexpr int RPR = (EPI == SK_EPI_SWIGLU) ? 2 : 1;    // W tiles of a row group per round
+  constexpr int OUT_RT = RT / RPR;
+  constexpr int ITEMS = WN * MT * 64;
+  static_assert(ITEMS <= NT, "one item a thread");
+  const int ldc = (EPI == SK_EPI_SWIGLU) ? n_out : N;
+  const int e_ln = tid & 63, e_mt = (tid >> 6) % MT, e_wn = tid / (64 * MT);
+  const int e_m = e_mt * 16 + (e_ln & 15);
+  const int e_n0 = (blockIdx.x * WN + e_wn) * OUT_RT * 16 + 4 * (e_ln >> 4);   // round ort adds 16 * ort
+  const bool e_on = tid < ITEMS && e_m < M;
+  int e_pos = 0, e_page = 0;
+  float2 e_cos[EPI == SK_EPI_ROPE ? OUT_RT : 1], e_sin[EPI == SK_EPI_ROPE ? OUT_RT : 1];
+  float e_prev[EPI == SK_EPI_ACCUM ? OUT_RT : 1][4];
+  if (EPI == SK_EPI_ROPE && e_on) {
+    e_pos = rope.tok_pos[e_m];
+    const int q_dim = rope.n_heads * rope.hd, kv_dim = rope.n_kv * rope.hd;
+#pragma unroll
+    for (int ort = 0; ort < OUT_RT; ++ort) {
+      const int n = e_n0 + ort * 16, d = n % rope.hd;
+      e_cos[ort] = make_float2(1.f, 1.f);
+      e_sin[ort] = make_float2(0.f, 0.f);
+      if (n < q_dim + kv_dim && d < rope.rot_dim) {       // rot_dim is even; d is a multiple of 4
+        const float* cr = rope.cos_t + (size_t)e_pos * (rope.rot_dim / 2) + (d >> 1);
+        const float* sr = rope.sin_t + (size_t)e_pos * (rope.rot_dim / 2) + (d >> 1);
+        e_cos[ort].x = cr[0];
+        e_sin[ort].x = sr[0];
+        if (d + 2 < rope.rot_dim) {
+          e_cos[ort].y = cr[1];
+          e_sin[ort].y = sr[1];
+        }
+      }
+    }
+    if (rope.write_kv && e_n0 + (OUT_RT - 1) * 16 >= q_dim) {
+      const int slot = rope.seq_slot[rope.tok_seq[e_m]];
+      e_page = rope.table[(size_t)slot * rope.table_stride + e_pos / 64];
+    }
+  }
+  if (EPI == SK_EPI_ACCUM && e_on) {
+#pragma unroll
+    for (int ort = 0; ort < OUT_RT; ++ort) {
+      const int n = e_n0 + ort * 16;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        e_prev[ort][e] = (n + e < ldc) ? Conv<OutT>::load(C + (size_t)e_m * ldc + n + e) : 0.f;
+    }
+  }
 #define SK_STEP(C, CUR, NXT)                    \
   store_x();                                    \
   __syncthreads();                              \
@@ -167,10 +217,6 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   // ---- add the partial sums of the 8 waves in order, apply the epilogue, store: one output tile
   // of every row group a round (a gate and its up tile together), so that the buffer stays small
   float* red = reinterpret_cast<float*>(lds);
-  constexpr int RPR = (EPI == SK_EPI_SWIGLU) ? 2 : 1;    // W tiles of a row group per round
-  constexpr int OUT_RT = RT / RPR;
-  constexpr int ITEMS = WN * MT * 64;
-  const int ldc = (EPI == SK_EPI_SWIGLU) ? n_out : N;
 #pragma unroll
   for (int ort = 0; ort < OUT_RT; ++ort) {
   if (ort > 0) __syncthreads();                          // the round before has been read
@@ -182,12 +228,10 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
           make_float4(acc[ort * RPR + j][mt][0], acc[ort * RPR + j][mt][1], acc[ort * RPR + j][mt][2],
                       acc[ort * RPR + j][mt][3]);
   __syncthreads();
-  for (int it = tid; it < ITEMS; it += NT) {
-    const int ln = it & 63;
-    const int mt = (it >> 6) % MT;
-    const int w_n = it / (64 * MT);
+  if (tid < ITEMS) {
+    const int ln = e_ln, mt = e_mt, w_n = e_wn;
     float v[4];
-    int n;
+    const int n = e_n0 + ort * 16;
     if (EPI == SK_EPI_SWIGLU) {
       float gsum[4] = {0.f, 0.f, 0.f, 0.f}, usum[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -204,7 +248,6 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
         const float gt = bf16_to_f32(f32_to_bf16(gsum[e])), up = bf16_to_f32(f32_to_bf16(usum[e]));
         v[e] = up * gt / (1.0f + expf(-gt));
       }
-      n = ((blockIdx.x * WN + w_n) * OUT_RT + ort) * 16 + 4 * (ln >> 4);
     } else {
       float sum[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
@@ -215,9 +258,8 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
       }
 #pragma unroll
       for (int e = 0; e < 4; ++e) v[e] = sum[e];
-      n = ((blockIdx.x * WN + w_n) * RT + ort) * 16 + 4 * (ln >> 4);
     }
-    const int m = mt * 16 + (ln & 15);
+    const int m = e_m;
     if (EPI == SK_EPI_ROPE) {
       if (m >= M || n >= N) continue;                 // N, hd are multiples of 16: four outputs, one head
       if (rope.bias) {
@@ -225,20 +267,15 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
         for (int e = 0; e < 4; ++e) v[e] += rope.bias[n + e];
       }
       const int q_dim = rope.n_heads * rope.hd, kv_dim = rope.n_kv * rope.hd;
-      const int pos = rope.tok_pos[m];
+      const int pos = e_pos;
       const int d = n % rope.hd;
-      if (n < q_dim + kv_dim) {                       // q and k rotate
-        const float* cr = rope.cos_t + (size_t)pos * (rope.rot_dim / 2);
-        const float* sr = rope.sin_t + (size_t)pos * (rope.rot_dim / 2);
-#pragma unroll
-        for (int e = 0; e < 4; e += 2) {
-          if (d + e < rope.rot_dim) {
-            const float c = cr[(d + e) >> 1], sn = sr[(d + e) >> 1];
-            const float x1 = v[e], x2 = v[e + 1];
-            v[e] = x1 * c - x2 * sn;
-            v[e + 1] = x2 * c + x1 * sn;
-          }
-        }
+      {                                               // q and k rotate; elsewhere the angle is zero
+        const float c0 = e_cos[ort].x, s0 = e_sin[ort].x, c1 = e_cos[ort].y, s1 = e_sin[ort].y;
+        const float a0 = v[0], a1 = v[1], a2 = v[2], a3 = v[3];
+        v[0] = a0 * c0 - a1 * s0;
+        v[1] = a1 * c0 + a0 * s0;
+        v[2] = a2 * c1 - a3 * s1;
+        v[3] = a3 * c1 + a2 * s1;
       }
       uint2 pk;
       pk.x = pack2_bf16(v[0], v[1]);
@@ -246,8 +283,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
       if (n < q_dim) {
         *reinterpret_cast<uint2*>(C + (size_t)m * q_dim + n) = pk;
       } else if (rope.write_kv) {
-        const int slot = rope.seq_slot[rope.tok_seq[m]];
-        const int page = rope.table[(size_t)slot * rope.table_stride + pos / 64];
+        const int page = e_page;
         const int kn = n - q_dim;
         if (kn < kv_dim) {
           const int kvh = kn / rope.hd;
@@ -267,8 +303,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
     OutT* dst = C + (size_t)m * ldc + n;
     if (EPI == SK_EPI_ACCUM) {
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        if (n + e < ldc) v[e] += Conv<OutT>::load(dst + e);
+      for (int e = 0; e < 4; ++e) v[e] += e_prev[ort][e];
     }
     if (n + 3 < ldc && (ldc & 3) == 0) {
       if (sizeof(OutT) == 2) {
