@@ -281,6 +281,39 @@ def test_a_dropped_engine_goes_at_once_with_its_graphs(models):
         gc.enable()
 
 
+def test_captures_with_an_eager_collector(models):
+    """The collector of cycles set to run at almost every allocation, engines built and dropped one
+    after another, each capturing graphs of both kinds, some cyclic garbage that owns device
+    memory lying about: captures collect first and keep the collector off while they last, so the
+    steps give what an engine without graphs gives."""
+    import gc
+    import torch
+    from libllm_amd.engine import StepEntry
+    from libllm_amd.runtime import load_engine
+    path, cfg, _ = models["A"]
+    ref = load_engine(path, dtype="float32", max_tokens=1024, use_graphs=False)
+    steps = [[StepEntry(i, [5 + i, 6, 7, 8, 9][:3 + i], [2 + i]) for i in range(3)]]
+    steps += [[StepEntry(i, [11 + k], [0]) for i in range(3)] for k in range(4)]
+    want = [ref.step(e).clone() for e in steps]
+    ref.end([0, 1, 2])
+    old = gc.get_threshold()
+    gc.set_threshold(1, 1, 1)
+    try:
+        for rnd in range(3):
+            junk = [torch.empty(1024, device="cuda")]
+            junk.append(junk)                                  # a cycle that owns device memory
+            del junk
+            engine = load_engine(path, dtype="float32", max_tokens=1024)
+            engine.PROMPT_SEEN = 1
+            for e, w in zip(steps, want):
+                assert torch.equal(engine.step(e), w)
+            assert engine._graphs and engine._prompt_graphs
+            assert gc.isenabled()
+            del engine
+    finally:
+        gc.set_threshold(*old)
+
+
 @pytest.mark.parametrize("rows", [512, 2048])
 def test_library_products_inside_prompt_graphs(rows):
     """A prompt of real width fills its graph exactly, so that the graph and an engine without
