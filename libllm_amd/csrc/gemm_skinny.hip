@@ -369,6 +369,10 @@ static int pick_shape(const SkinnyArgs& a) {
       if constexpr (RT == 1) {
         if (a.N <= 4096) return launch_skinny<1, RT, 1, 4, EPI, OutT>(a);
       }
+      // gate/up has more blocks than the chip has compute units: with the narrow chunk a block
+      // needs few enough registers for two of them to share a unit, and the tail of one overlaps
+      // the head of the next (3 % of a decode step at the 1B and 8B shapes, whole engines compared)
+      if constexpr (EPI == SK_EPI_SWIGLU) return launch_skinny<1, RT, 1, 1, EPI, OutT>(a);
       return launch_skinny<1, RT, 1, 2, EPI, OutT>(a);
     // More rows of W per block where W has rows enough to fill the GPU with such blocks: the rows
     // of X are then staged once for 64 rows of W instead of 16.
