@@ -76,7 +76,16 @@ class PreparedWeight:
 
 
 class HipOps:
+    """The operations of the model on the GPU: the only implementation there is.  Every method
+    checks its operands on the host before a kernel is launched."""
+
     supports_graphs = True
+
+    # Launch decisions, each measured with variants side by side in one process:
+    SKINNY_ROWS = 64        # most rows the streaming matrix product takes at once; beyond, the library's
+    ACCUM_ROWS = 32         # most rows for which a product adds into the stream itself; beyond, the library's
+    DECODE_BLOCKS = 768     # blocks of the decode attention grid beyond which sequences are not split further
+    _EPI_NONE, _EPI_SWIGLU, _EPI_ACCUM = 0, 1, 2
 
     def __init__(self, device: Optional[str] = None):
         if not torch.cuda.is_available():
@@ -93,9 +102,10 @@ class HipOps:
             fn.argtypes = argtypes
             fn.restype = _i
         torch.backends.cuda.matmul.allow_tf32 = False
-        self.fast_attention = True
-        self.pack_weights = True
-        self.fast_gemm = True
+        # switches for tests and measurements; the product runs with all three on
+        self.fast_attention = True      # bfloat16 attention on the matrix cores (else the plain kernel, as for float32)
+        self.pack_weights = True        # keep a tiled copy of every weight for the skinny product
+        self.fast_gemm = True           # the skinny product for few rows (else the library's for every product)
 
     # ---- helpers
     def _stream(self):
@@ -184,11 +194,6 @@ class HipOps:
                                              float(eps), out.data_ptr(), _code(out_dtype), rptr,
                                              n_out, h, self._stream()), "add_rmsnorm")
         return out
-
-    SKINNY_ROWS = 64        # most rows the streaming matrix product takes at once
-    ACCUM_ROWS = 32         # most rows for which a product adds into the stream itself; beyond, the library's
-    DECODE_BLOCKS = 768     # blocks of the decode attention grid beyond which sequences are not split further
-    _EPI_NONE, _EPI_SWIGLU, _EPI_ACCUM = 0, 1, 2
 
     def prepare_weight(self, w: torch.Tensor, like=None):
         """Called once for a weight matrix that products will stream many times.  Returns what
