@@ -40,6 +40,7 @@ class Engine:
     PROMPT_ROWS = (16, 32, 64, 128, 192, 256, 384, 512, 768, 1024, 1536, 2048)
     PROMPT_SEQS = (2, 3, 5, 9, 17)
     PROMPT_SEEN = 2
+    PROMPT_GRAPHS = 24      # prompt graphs kept; the one unused for longest goes first (each holds its activations)
 
     def __init__(self, model: DecoderModel, ops, dtype: torch.dtype, max_tokens: int,
                  max_slots: Optional[int] = None, use_graphs: bool = True):
@@ -199,14 +200,16 @@ class Engine:
         if rows > self.cache.pages_per_seq * PAGE or wanted > seqs:
             return None
         key = (rows, seqs)
-        graph = self._prompt_graphs.get(key)
+        graph = self._prompt_graphs.pop(key, None)
         if graph is None:
             seen = self._prompt_seen.get(key, 0) + 1
             self._prompt_seen[key] = seen
             if seen < self.PROMPT_SEEN:
                 return None
+            while len(self._prompt_graphs) >= max(1, self.PROMPT_GRAPHS):
+                del self._prompt_graphs[next(iter(self._prompt_graphs))]     # dicts keep the order of insertion
             graph = _PromptGraph(self, rows, seqs)
-            self._prompt_graphs[key] = graph
+        self._prompt_graphs[key] = graph                                      # the last used lies last
         return graph
 
     # ---- decoding one token per sequence through a captured graph

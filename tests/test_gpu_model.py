@@ -281,6 +281,27 @@ def test_a_dropped_engine_goes_at_once_with_its_graphs(models):
         gc.enable()
 
 
+def test_prompt_graphs_are_bounded(models):
+    """At most ``PROMPT_GRAPHS`` prompt graphs are kept, the one unused for longest goes first, and a
+    shape that comes again after its graph went is captured again and gives the same logits."""
+    import torch
+    from libllm_amd.engine import StepEntry
+    from libllm_amd.runtime import load_engine
+    path, cfg, _ = models["A"]
+    engine = load_engine(path, dtype="float32", max_tokens=2048)
+    engine.PROMPT_SEEN, engine.PROMPT_GRAPHS = 1, 2
+    ref = load_engine(path, dtype="float32", max_tokens=2048, use_graphs=False)
+    rng = np.random.default_rng(6)
+    seen = []
+    for n in (5, 20, 40, 5, 70, 20):                    # rows 16, 32, 64, 16, 128, 32
+        prompt = rng.integers(3, cfg.vocab, size=n).tolist()
+        a, b = engine.step([StepEntry("p", prompt, [n - 1])]), ref.step([StepEntry("p", prompt, [n - 1])])
+        assert torch.equal(a, b)
+        engine.end(["p"]); ref.end(["p"])
+        seen.append([k[0] for k in engine._prompt_graphs])
+    assert seen == [[16], [16, 32], [32, 64], [64, 16], [16, 128], [128, 32]]
+
+
 def test_captures_with_an_eager_collector(models):
     """The collector of cycles set to run at almost every allocation, engines built and dropped one
     after another, each capturing graphs of both kinds, some cyclic garbage that owns device
