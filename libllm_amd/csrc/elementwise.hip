@@ -34,9 +34,9 @@ extern "C" int llm_embed(const void* table, int table_dtype, const int* ids, flo
 //   x = res[r] + delta[r] (stored back into res when delta is given)
 //   out[b] = x * w * 1/sqrt(mean(x^2) + eps)         (src/flint/cuda/rms_norm.cu:45-76)
 template <typename TD, typename TO, int NT>
-__global__ void add_rmsnorm_kernel(float* __restrict__ res, const TD* __restrict__ delta,
-                                   const float* __restrict__ w, float eps, TO* __restrict__ out,
-                                   const int* __restrict__ rows, int H) {
+__global__ void add_rmsnorm_kernel(float* __restrict__ res, const TD* __restrict__ delta, int n_delta,
+                                   size_t delta_stride, const float* __restrict__ w, float eps,
+                                   TO* __restrict__ out, const int* __restrict__ rows, int H) {
   __shared__ float scratch[NT / 64];
   const int b = blockIdx.x;
   const int r = rows ? rows[b] : b;
@@ -46,7 +46,7 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ res, const TD* __restrict
   for (int i = threadIdx.x; i < H; i += NT) {
     float v = x[i];
     if (d) {
-      v += Conv<TD>::load(d + i);
+      for (int j = 0; j < n_delta; ++j) v += Conv<TD>::load(d + j * delta_stride + i);   // in this order
       x[i] = v;
     }
     ss += v * v;
@@ -62,7 +62,8 @@ __global__ void add_rmsnorm_kernel(float* __restrict__ res, const TD* __restrict
 // in flight together.
 template <typename TD, typename TO, int NT, int NV>
 __global__ __launch_bounds__(NT) void add_rmsnorm_reg_kernel(float* __restrict__ res,
-                                                              const TD* __restrict__ delta,
+                                                              const TD* __restrict__ delta, int n_delta,
+                                                              size_t delta_stride,
                                                               const float* __restrict__ w, float eps,
                                                               TO* __restrict__ out,
                                                               const int* __restrict__ rows, int H) {
@@ -79,10 +80,13 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_reg_kernel(float* __restrict__
     v[j] = in ? *reinterpret_cast<const float4*>(x + i) : make_float4(0.f, 0.f, 0.f, 0.f);
     wv[j] = in ? *reinterpret_cast<const float4*>(w + i) : make_float4(0.f, 0.f, 0.f, 0.f);
     if (d && in) {
-      v[j].x += Conv<TD>::load(d + i);
-      v[j].y += Conv<TD>::load(d + i + 1);
-      v[j].z += Conv<TD>::load(d + i + 2);
-      v[j].w += Conv<TD>::load(d + i + 3);
+      for (int q = 0; q < n_delta; ++q) {                  // several deltas are added in this order
+        const TD* dq = d + q * delta_stride + i;
+        v[j].x += Conv<TD>::load(dq);
+        v[j].y += Conv<TD>::load(dq + 1);
+        v[j].z += Conv<TD>::load(dq + 2);
+        v[j].w += Conv<TD>::load(dq + 3);
+      }
       *reinterpret_cast<float4*>(x + i) = v[j];
     }
   }
@@ -104,23 +108,24 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_reg_kernel(float* __restrict__
   }
 }
 
-extern "C" int llm_add_rmsnorm(float* res, const void* delta, int delta_dtype, const float* w,
-                               float eps, void* out, int out_dtype, const int* rows, int n_out,
-                               int H, hipStream_t stream) {
+// delta: nothing, a matrix like res, or n_delta of them delta_stride elements apart, added in order.
+extern "C" int llm_add_rmsnorm(float* res, const void* delta, int delta_dtype, int n_delta,
+                               size_t delta_stride, const float* w, float eps, void* out, int out_dtype,
+                               const int* rows, int n_out, int H, hipStream_t stream) {
   if (n_out <= 0) return LLM_OK;
-  if (H <= 0) return LLM_ERR_ARG;
+  if (H <= 0 || (delta != nullptr && n_delta < 1)) return LLM_ERR_ARG;
   constexpr int NT = 256;
   const bool reg = (H % 4 == 0) && H <= NT * 4 * 4 && ((((uintptr_t)res) | ((uintptr_t)w)) & 15) == 0;
   const bool reg2 = reg && H <= NT * 4 * 2;
 #define LAUNCH(TD, TO) do {                                                                         \
   if (reg2)                                                                                         \
-    add_rmsnorm_reg_kernel<TD, TO, NT, 2><<<n_out, NT, 0, stream>>>(res, (const TD*)delta, w, eps,  \
+    add_rmsnorm_reg_kernel<TD, TO, NT, 2><<<n_out, NT, 0, stream>>>(res, (const TD*)delta, n_delta, delta_stride, w, eps,  \
                                                                     (TO*)out, rows, H);             \
   else if (reg)                                                                                     \
-    add_rmsnorm_reg_kernel<TD, TO, NT, 4><<<n_out, NT, 0, stream>>>(res, (const TD*)delta, w, eps,  \
+    add_rmsnorm_reg_kernel<TD, TO, NT, 4><<<n_out, NT, 0, stream>>>(res, (const TD*)delta, n_delta, delta_stride, w, eps,  \
                                                                     (TO*)out, rows, H);             \
   else                                                                                              \
-    add_rmsnorm_kernel<TD, TO, NT><<<n_out, NT, 0, stream>>>(res, (const TD*)delta, w, eps, (TO*)out, rows, H); \
+    add_rmsnorm_kernel<TD, TO, NT><<<n_out, NT, 0, stream>>>(res, (const TD*)delta, n_delta, delta_stride, w, eps, (TO*)out, rows, H); \
   } while (0)
   if (delta == nullptr) delta_dtype = out_dtype;
   if (delta_dtype == LLM_DTYPE_F32 && out_dtype == LLM_DTYPE_F32) LAUNCH(float, float);

@@ -49,7 +49,8 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
                                                                       const bf16_t* __restrict__ W,
                                                                       OutT* __restrict__ C, int M,
                                                                       int N, int K, int ldw,
-                                                                      int n_out, SkinnyRope rope) {
+                                                                      int n_out, int ldx, int w_steps,
+                                                                      SkinnyRope rope) {
   constexpr int NT = WN * SK_WK * 64;
   constexpr int CK = 512 * G;                    // elements of K per chunk
   constexpr int ROW_B = CK * 2;                  // bytes of a staged row; 16-byte pieces are swizzled
@@ -65,6 +66,12 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   const int wn = wave / SK_WK, wk = wave % SK_WK;
   const int r = lane & 15, g = lane >> 4;
   const int group = blockIdx.x * WN + wn;                       // row group of this wave
+  // K may be a slice of the rows of X and W: blockIdx.y counts the slices (K elements each, a
+  // multiple of 32 then), rows of X lie ldx apart, a full row of W has w_steps steps of 32, and
+  // each slice stores its sums to a matrix of its own (plain epilogue only).  Whoever adds the
+  // matrices does it in a fixed order; one launch with a grid of height 1 is the whole product.
+  const int k0 = blockIdx.y * K;
+  X += k0;
   const int n_steps = (K + 31) / 32;
   const int n_chunks = (K + CK - 1) / CK;
 
@@ -83,11 +90,11 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
     if (ldw == 0) {                             // tiled for the matrix cores: see llm_pack_weight
       int t = tile_row[rt] / 16;
       if (t > (N - 1) / 16) t = (N - 1) / 16;
-      wp[rt] = W + ((size_t)t * n_steps * 64 + lane) * 8;
+      wp[rt] = W + ((size_t)t * w_steps * 64 + lane) * 8 + (size_t)(k0 / 32) * 512;
     } else {
       int n = tile_row[rt] + r;
       if (n > N - 1) n = N - 1;                 // rows past the end read the last row; not stored
-      wp[rt] = W + (size_t)n * ldw + g * 8;
+      wp[rt] = W + (size_t)n * ldw + g * 8 + k0;
     }
   }
 
@@ -105,7 +112,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
 #pragma unroll
     for (int p = 0; p < PASSES; ++p) {
       const int row = x_row0 + p * ROWS_PASS;
-      xr[p] = (row < M && k < K) ? *reinterpret_cast<const uint4*>(X + (size_t)row * K + k)
+      xr[p] = (row < M && k < K) ? *reinterpret_cast<const uint4*>(X + (size_t)row * ldx + k)
                                  : make_uint4(0u, 0u, 0u, 0u);
     }
   };
@@ -300,7 +307,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
       continue;
     }
     if (m >= M || n >= ldc) continue;
-    OutT* dst = C + (size_t)m * ldc + n;
+    OutT* dst = C + ((size_t)blockIdx.y * M + m) * ldc + n;
     if (EPI == SK_EPI_ACCUM) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) v[e] += e_prev[ort][e];
@@ -328,6 +335,7 @@ struct SkinnyArgs {
   const bf16_t* W;
   void* C;
   int M, N, K, ldw, n_out;     // ldw: elements between rows of W (a multiple of 8, at least K)
+  int k_split;                 // slices of K, each to a result matrix of its own (1: the whole product)
   hipStream_t stream;
   SkinnyRope rope;
 };
@@ -338,8 +346,9 @@ static int launch_skinny(const SkinnyArgs& a) {
   const int tiles = (rows + 15) / 16;
   constexpr int OUT_RT = (EPI == SK_EPI_SWIGLU) ? RT / 2 : RT;
   const int blocks = (tiles + OUT_RT * WN - 1) / (OUT_RT * WN);
-  gemm_skinny_kernel<MT, RT, WN, G, EPI, OutT><<<blocks, WN * SK_WK * 64, 0, a.stream>>>(
-      a.X, a.W, (OutT*)a.C, a.M, a.N, a.K, a.ldw, a.n_out, a.rope);
+  const dim3 grid(blocks, a.k_split);
+  gemm_skinny_kernel<MT, RT, WN, G, EPI, OutT><<<grid, WN * SK_WK * 64, 0, a.stream>>>(
+      a.X, a.W, (OutT*)a.C, a.M, a.N, a.K / a.k_split, a.ldw, a.n_out, a.K, (a.K + 31) / 32, a.rope);
   return llm_launch_status();
 }
 
@@ -351,6 +360,8 @@ static int pick_rows(const SkinnyArgs& a) {
     if (a.n_out >= 8192 && MT >= 3) return launch_skinny<MT, 4, 1, 1, EPI, OutT>(a);
     return launch_skinny<MT, 2, 1, 1, EPI, OutT>(a);
   } else {
+    // slices of K: 64 rows of W a block, so that a slice of X is staged for as many as possible
+    if (a.k_split > 1) return launch_skinny<MT, 2, 2, 1, EPI, OutT>(a);
     if (a.N >= 8192) return launch_skinny<MT, 2, 2, 1, EPI, OutT>(a);
     if (a.N >= 6144) return launch_skinny<MT, 2, 1, 1, EPI, OutT>(a);
     return launch_skinny<MT, 1, 1, 1, EPI, OutT>(a);
@@ -385,12 +396,18 @@ static int pick_shape(const SkinnyArgs& a) {
 
 // Rows of W lie ldw elements apart (ldw >= K, a multiple of 8); ldw == 0 says that W is the
 // tiled copy that llm_pack_weight makes.
+// With k_split > 1 (more than 16 rows, epilogue 0, float32) C is [k_split, M, N]: the products over
+// the k_split slices of K, for the caller to add in order.
 // C[M, N] (epilogue 0: stored as out_dtype; 2: added into the float32 C) or C[M, N/2] (epilogue 1,
 // SwiGLU over W = [Wg; Wu], N/2 a multiple of 16) from X[M, K] and W[N, K].  X is bfloat16.
 extern "C" int llm_gemm_skinny_bf16(const void* X, const void* W, void* C,
                                     int epilogue, int out_dtype, int M, int N, int K, int ldw,
-                                    hipStream_t stream) {
+                                    int k_split, hipStream_t stream) {
   if (M <= 0 || N <= 0) return LLM_OK;
+  // slices of K: more than 16 rows, plain epilogue, float32 results [k_split, M, N]
+  if (k_split < 1 || (k_split > 1 && (M <= 16 || epilogue != SK_EPI_NONE || out_dtype != LLM_DTYPE_F32 ||
+                                      K % (k_split * 32) != 0)))
+    return LLM_ERR_ARG;
   if (M > 64 || K <= 0 || (K & 7) || (ldw != 0 && (ldw < K || (ldw & 7)))) return LLM_ERR_ARG;
   if (X == nullptr || W == nullptr || C == nullptr) return LLM_ERR_ARG;
   if ((((uintptr_t)X) | ((uintptr_t)W) | ((uintptr_t)C)) & 15) return LLM_ERR_ARG;
@@ -403,6 +420,7 @@ extern "C" int llm_gemm_skinny_bf16(const void* X, const void* W, void* C,
   a.K = K;
   a.ldw = ldw;
   a.n_out = N;
+  a.k_split = k_split;
   a.stream = stream;
   a.rope = SkinnyRope{};
   if (epilogue == SK_EPI_NONE) {
@@ -448,6 +466,7 @@ extern "C" int llm_gemm_skinny_rope_bf16(const void* X, const void* W,
   a.K = K;
   a.ldw = ldw;
   a.n_out = a.N;
+  a.k_split = 1;
   a.stream = stream;
   a.rope.bias = bias;
   a.rope.cos_t = cos_t;

@@ -31,7 +31,7 @@ def _code(dtype: torch.dtype) -> int:
 
 _SIGNATURES = {
     "llm_embed": [_vp, _i, _vp, _vp, _i, _i, _i, _f, _vp],
-    "llm_add_rmsnorm": [_vp, _vp, _i, _vp, _f, _vp, _i, _vp, _i, _i, _vp],
+    "llm_add_rmsnorm": [_vp, _vp, _i, _i, ctypes.c_size_t, _vp, _f, _vp, _i, _vp, _i, _i, _vp],
     "llm_silu_mul": [_vp, _vp, _i, _i, _i, _vp],
     "llm_add_bias": [_vp, _i, _vp, _i, _i, _vp],
     "llm_rope_kv_write": [_vp, _i, _i, _vp, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp,
@@ -42,7 +42,7 @@ _SIGNATURES = {
     "llm_gemm_f32": [_vp, _vp, _vp, _i, _i, _i, _vp],
     "llm_attention_ref": [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
                           _f, _i, _vp],
-    "llm_gemm_skinny_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "llm_gemm_skinny_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "llm_attention_mfma_supported": [_i],
     "llm_attention_prefill_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i,
                                    _i, _i, _f, _i, _vp],
@@ -83,7 +83,8 @@ class HipOps:
 
     # Launch decisions, each measured with variants side by side in one process:
     SKINNY_ROWS = 64        # most rows the streaming matrix product takes at once; beyond, the library's
-    ACCUM_ROWS = 32         # most rows for which a product adds into the stream itself; beyond, the library's
+    ACCUM_ROWS = 16         # most rows for which a product adds into the stream itself
+    SPLIT_ROWS = 64         # beyond those and up to here it goes in slices of K that the next norm adds; then the library's
     DECODE_BLOCKS = 768     # blocks of the decode attention grid beyond which sequences are not split further
     _EPI_NONE, _EPI_SWIGLU, _EPI_ACCUM = 0, 1, 2
 
@@ -181,16 +182,21 @@ class HipOps:
         m, h = res.shape
         self._dev(res, "residual stream", torch.float32)
         self._dev(weight, "norm weight", torch.float32, (h,))
-        dptr, dcode = None, _code(out_dtype)
+        dptr, dcode, n_delta = None, _code(out_dtype), 1
         if delta is not None:
-            dptr, dcode = self._dev(delta, "delta", shape=(m, h)), _code(delta.dtype)
+            if delta.dim() == 3:                     # several float32 matrices, added in their order
+                n_delta = delta.shape[0]
+                dptr = self._dev(delta, "delta", torch.float32, (n_delta, m, h))
+            else:
+                dptr = self._dev(delta, "delta", shape=(m, h))
+            dcode = _code(delta.dtype)
         n_out = m
         rptr = None
         if rows is not None:
             rptr = self._dev(rows, "row indices", torch.int32)
             n_out = rows.shape[0]
         out = torch.empty((n_out, h), dtype=out_dtype, device=self.device)
-        self._check(self.lib.llm_add_rmsnorm(res.data_ptr(), dptr, dcode, weight.data_ptr(),
+        self._check(self.lib.llm_add_rmsnorm(res.data_ptr(), dptr, dcode, n_delta, m * h, weight.data_ptr(),
                                              float(eps), out.data_ptr(), _code(out_dtype), rptr,
                                              n_out, h, self._stream()), "add_rmsnorm")
         return out
@@ -247,15 +253,25 @@ class HipOps:
             return False                     # the norm kernel runs first; the product takes its rows
         return x.dtype == torch.bfloat16 and x.data_ptr() % 16 == 0
 
-    def _skinny(self, x, w, out, epilogue, m0=0, mm=None):
-        """Launches the skinny kernel on rows m0 .. m0+mm of the bfloat16 matrix x."""
+    @staticmethod
+    def _k_split(n, k):
+        """Slices of K for a product of 17 to 64 rows with a weight of ``n`` rows: enough for about
+        a block a compute unit at 64 weight rows a block, each at least 512 long and a multiple of 32."""
+        ks = max(1, min(8, 256 // max(1, -(-n // 64))))
+        while ks > 1 and (k % (ks * 32) or k // ks < 512):
+            ks -= 1
+        return ks
+
+    def _skinny(self, x, w, out, epilogue, m0=0, mm=None, k_split=1):
+        """Launches the skinny kernel on rows m0 .. m0+mm of the bfloat16 matrix x; with ``k_split``
+        the products over that many slices of K go to ``out[k_split, mm, n]``."""
         n, k = w.shape
         xp = x.data_ptr() + m0 * k * 2
         width = n // 2 if epilogue == self._EPI_SWIGLU else n
         wptr, ldw = self._streamed(w)
         self._check(self.lib.llm_gemm_skinny_bf16(
             xp, wptr, out.data_ptr() + m0 * width * out.element_size(),
-            epilogue, _code(out.dtype), mm, n, k, ldw, self._stream()), "gemm_skinny_bf16")
+            epilogue, _code(out.dtype), mm, n, k, ldw, k_split, self._stream()), "gemm_skinny_bf16")
 
     def linear(self, x, w, bias, out_dtype, residual=None):
         """x W^T (+ bias) as ``out_dtype``.  ``x`` is a matrix or a ``normed`` record.  With
@@ -273,6 +289,13 @@ class HipOps:
             self._dev(x.weight, "norm weight", torch.float32, (k,))
         else:
             self._dev(x, "linear input")
+        if (self._skinny_ok(x, w, m, k) and bias is None and residual is not None
+                and self.ACCUM_ROWS < m <= self.SPLIT_ROWS and (ks := self._k_split(n, k)) > 1):
+            # K in slices, one block for 64 rows of the weight and a slice: each slice of X is staged
+            # for four times the rows; the norm kernel that follows adds the slices, in order
+            parts = torch.empty((ks, m, n), dtype=torch.float32, device=self.device)
+            self._skinny(x, w, parts, self._EPI_NONE, 0, m, k_split=ks)
+            return parts
         if self._skinny_ok(x, w, m, k) and bias is None and not (residual is not None and m > self.ACCUM_ROWS):
             if residual is not None and m <= self.SKINNY_ROWS:
                 self._dev(residual, "residual stream", torch.float32, (m, n))

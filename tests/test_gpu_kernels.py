@@ -167,7 +167,7 @@ def test_gemm_skinny_refuses(ops):
     out = ops.linear(x, w, None, torch.bfloat16)
     assert close(out, x.double() @ w.double().t(), torch.bfloat16)
     c = torch.empty((2, 16), dtype=torch.bfloat16, device="cuda")
-    st = ops.lib.llm_gemm_skinny_bf16(x.data_ptr(), w.data_ptr(), c.data_ptr(), 0, 1, 2, 16, 12, 12, 0)
+    st = ops.lib.llm_gemm_skinny_bf16(x.data_ptr(), w.data_ptr(), c.data_ptr(), 0, 1, 2, 16, 12, 12, 1, 0)
     assert st == 1                                        # refused, not wrong
 
 
@@ -230,7 +230,7 @@ def test_weight_rows_may_lie_apart(ops):
 @pytest.mark.parametrize("nk", [(16, 8), (300, 520), (2048, 2048), (72, 4104)])
 def test_gemm_skinny_adds_into_the_stream(ops, monkeypatch, m, nk):
     """Up to ``ACCUM_ROWS`` rows the product adds into the stream itself and returns None; beyond,
-    the product is returned for the caller to add and the stream is left alone.  Forced to 64
+    the product is returned (a matrix, or slices over K) for the norm to add and the stream is left alone.  Forced to 64
     the kernel adds for 40 rows too."""
     n, k = nk
     x = rnd((m, k), torch.bfloat16, 30).cuda()
@@ -241,9 +241,9 @@ def test_gemm_skinny_adds_into_the_stream(ops, monkeypatch, m, nk):
         res = rnd((m, n), torch.float32, 32, 5.0).cuda()
         before = res.clone()
         out = ops.linear(x, w, None, torch.bfloat16, residual=res)
-        if m > limit:
+        if m > limit:                       # the product comes back, whole or in slices of K, for the norm to add
             assert out is not None and torch.equal(res, before)
-            assert close(out, ref, torch.bfloat16)
+            assert close(out.sum(0) if out.dim() == 3 else out, ref, torch.bfloat16)
             continue
         assert out is None
         assert max_err(res, before.double() + ref.cuda()) < 2e-6
@@ -279,6 +279,49 @@ def test_products_of_rows_still_to_be_normalised(ops, m, nk, gather):
         g, u = ref[:, :n // 2], ref[:, n // 2:]
         sw = ops.linear_swiglu(lazy, w, torch.bfloat16)
         assert max_err(sw, g / (1 + torch.exp(-g)) * u) < 4 * BF16_2ULP
+
+
+@pytest.mark.parametrize("m", [17, 33, 40, 64])
+@pytest.mark.parametrize("nk", [(128, 2048), (2048, 2048), (2048, 8192), (3072, 3072), (200, 1536)])
+def test_products_in_slices_of_k(ops, monkeypatch, m, nk):
+    """From 33 to 64 rows a product that adds into the stream is computed over slices of K, each
+    slice to a float32 matrix of its own, and the norm kernel that follows adds them in order:
+    against the plain formulas, from the weight as it lies and from its tiled copy (the same
+    bits), and the same bits when other rows share the step."""
+    n, k = nk
+    monkeypatch.setattr(ops, "ACCUM_ROWS", 16)               # so that 17 rows take this path too
+    ks = ops._k_split(n, k)
+    assert ks > 1 and k % (ks * 32) == 0
+    x = rnd((m, k), torch.bfloat16, 80).cuda()
+    w = rnd((n, k), torch.bfloat16, 81).cuda()
+    pw = ops.prepare_weight(w)
+    res = rnd((m, n), torch.float32, 82, 3.0).cuda()
+    parts = ops.linear(x, pw, None, torch.bfloat16, residual=res)
+    assert tuple(parts.shape) == (ks, m, n) and parts.dtype == torch.float32
+    ref = x.double() @ w.double().t()
+    assert max_err(parts.double().sum(0), ref.cuda()) < 2e-6
+    for j in range(ks):                                      # every slice is the product over its part of K
+        sl = slice(j * (k // ks), (j + 1) * (k // ks))
+        assert max_err(parts[j], (x[:, sl].double() @ w[:, sl].double().t()).cuda()) < 2e-6
+    plain = torch.empty_like(parts)
+    ops._skinny(x, w, plain, ops._EPI_NONE, 0, m, k_split=ks)
+    assert torch.equal(plain, parts)
+    fewer = ops.linear(x[:17].contiguous(), pw, None, torch.bfloat16, residual=res[:17].contiguous())
+    assert torch.equal(fewer, parts[:, :17])                 # a row's sums do not depend on the other rows
+    # the norm adds the slices into the stream in their order and normalises
+    wn = (1.0 + 0.2 * rnd((n,), torch.float32, 83)).cuda()
+    stream = res.clone()
+    out = ops.add_rmsnorm(stream, parts, wn, 1e-5, torch.bfloat16)
+    want = res.clone()
+    for j in range(ks):
+        want += parts[j]
+    assert torch.equal(stream, want)
+    sd = want.double()
+    assert close(out, sd * wn.double() / torch.sqrt((sd * sd).mean(-1, keepdim=True) + 1e-5), torch.bfloat16)
+    # a buffer for the slices that is too small, or slices that do not divide K, are refused
+    from libllm_amd.errors import KernelError
+    with pytest.raises(KernelError):
+        ops._skinny(x, w, plain, ops._EPI_NONE, 0, m, k_split=7)
 
 
 def test_large_bf16_product(ops):

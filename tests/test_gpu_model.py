@@ -369,12 +369,11 @@ def test_library_products_inside_prompt_graphs(rows):
 
 
 @pytest.mark.parametrize("widths", [(2048, 32, 64, 8192), (4096, 32, 128, 14336)])
-def test_library_products_inside_decode_graphs(widths):
-    """From 33 rows on the products that add into the stream are the library's, also inside the
-    captured decode graphs.  Layers of real width (where the library picks the kernels it uses for
-    large products): a graph of 48 rows replayed twelve times, an engine without graphs stepping
-    beside it, other work and a synchronisation between the replays; every replay gives the bits
-    of the eager step."""
+def test_decode_graphs_of_many_rows(widths):
+    """From 17 rows on the products that add into the stream are computed over slices of K, which
+    the next norm kernel adds.  Layers of real width: a graph of 48 rows replayed twelve times, an
+    engine without graphs stepping beside it, other work and a synchronisation between the
+    replays; every replay gives the bits of the eager step."""
     import torch
     from libllm_amd.config import config_from_dict
     from libllm_amd.engine import StepEntry
@@ -388,7 +387,7 @@ def test_library_products_inside_decode_graphs(widths):
     rng = np.random.default_rng(3)
     prompts = {i: rng.integers(3, 4096, size=int(n)).tolist() for i, n in enumerate(rng.integers(3, 40, size=40))}
     engines = [random_engine(cfg, seed=5, dtype="bfloat16", max_tokens=8192, use_graphs=g) for g in (True, False)]
-    assert engines[0].ops.ACCUM_ROWS < 40 <= engines[0].ops.SKINNY_ROWS
+    assert engines[0].ops.ACCUM_ROWS < 40 <= engines[0].ops.SPLIT_ROWS
     for e in engines:
         e.step([StepEntry(r, t, []) for r, t in prompts.items()])
     scratch = torch.randn((512, 512), device="cuda")
