@@ -17,6 +17,15 @@
 
 #define PAGE 64
 
+// The largest of three in one instruction.  fmaxf first quiets a signalling NaN in every operand
+// the compiler cannot prove clean (one more instruction each for sums that come off the matrix
+// cores); the instruction alone gives the same result for everything but the NaN's payload.
+__device__ __forceinline__ float max3(float a, float b, float c) {
+  float r;
+  asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+  return r;
+}
+
 template <int HD>
 struct AttnState {
   f32x4 o[HD / 16];   // O^T[d = 16*dt + 4*(lane/16) + e][query = lane % 16]
@@ -107,14 +116,15 @@ __device__ __forceinline__ void load_query(const bf16_t* qrow, bool valid, Frag 
 }
 
 // ---------------------------------------------------------------------------------- prompts
-// A block of 4 waves owns 64 consecutive new tokens of one sequence and up to QT query heads that
-// share one kv head; wave w owns rows 16w .. 16w+15 for all those heads (QT tiles of 16 query
-// columns).  The block walks the pages its rows may see; a page's keys and values travel global
-// memory -> registers (issued one page ahead) -> shared memory, where all four waves read their
-// fragments, so a page is fetched once for 64 * QT queries.  16-byte pieces are swizzled in
-// shared memory so that the 16 rows a fragment load touches fall on different banks.
-// Blocks are numbered kv head first, so that the blocks of a kv head run on the same chiplet
-// and share its cache, and long rows first, since later rows see more keys.
+// A block of 4 waves owns 64 * QT consecutive new tokens of one sequence and one query head; wave
+// w owns QT tiles of 16 rows (query columns), tile t being rows 64t + 16w .. 64t + 16w + 15.  The
+// block walks the pages its rows may see; a page's keys and values travel global memory ->
+// registers (issued one page ahead) -> shared memory, where all four waves read their fragments,
+// and a fragment read from shared memory serves all the wave's tiles.  16-byte pieces are
+// swizzled in shared memory so that the 16 rows a fragment load touches fall on different banks.
+// Blocks are numbered kv head first (consecutive blocks go to consecutive chiplets, so with 8 kv
+// heads each chiplet's cache holds one head's keys and values), and long rows first, since later
+// rows see more keys.
 template <int HD>
 struct KeyRow {            // bytes between staged key rows: a power of two of at least 128
   static constexpr int BYTES = (HD * 2 <= 128) ? 128 : ((HD * 2 <= 256) ? 256 : 512);
@@ -166,47 +176,49 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     const bf16_t* __restrict__ v_pages, const int* __restrict__ table, int table_stride,
     const int* __restrict__ seq_start, const int* __restrict__ seq_slot,
     const int* __restrict__ seq_pos0, bf16_t* __restrict__ out, int n_heads, int n_kv,
-    float scale_log2, int window, int n_qblocks, int n_chunks) {
+    float scale_log2, int window, int n_qblocks) {
   constexpr int KS = (HD + 31) / 32, DT = HD / 16, KRB = KeyRow<HD>::BYTES;
   constexpr int LOADS = (8 * HD + 255) / 256;    // 16-byte pieces of a page per thread
+  constexpr int ROWS = 64 * QT;                  // rows of a block
   __shared__ __attribute__((aligned(16))) unsigned char k_lds[64 * KRB];
   __shared__ __attribute__((aligned(16))) unsigned char v_lds[HD * 128];
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
-  const int n_kvc = n_kv * n_chunks;
-  const int kvc = blockIdx.x % n_kvc, rest = blockIdx.x / n_kvc;
+  const int hi = blockIdx.x % n_heads, rest = blockIdx.x / n_heads;
   const int qb = n_qblocks - 1 - rest % n_qblocks, b = rest / n_qblocks;
-  const int kvh = kvc / n_chunks, chunk = kvc % n_chunks;
-  const int group = n_heads / n_kv;
-  const int per_chunk = (group + n_chunks - 1) / n_chunks;
-  const int h0 = kvh * group + chunk * per_chunk;
-  const int n_h = min(per_chunk, group - chunk * per_chunk);     // heads of this block (<= QT)
+  const int kvh = hi % n_kv, h = kvh * (n_heads / n_kv) + hi / n_kv;
   const int start = seq_start[b];
   const int n = seq_start[b + 1] - start;
-  const int q0b = qb * 64;
-  if (q0b >= n || n_h <= 0) return;                              // the whole block leaves
+  const int q0b = qb * ROWS;
+  if (q0b >= n) return;                                          // the whole block leaves
   const int pos0 = seq_pos0[b], slot = seq_slot[b];
-  const int q0w = q0b + wave * 16;
-  const int row = q0w + r;
-  const bool valid = row < n;
-  const int qpos = pos0 + row;                                   // rows past the end compute and are dropped
-  const int kmax = qpos;
-  const int kmin = (window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
-
+  // tile qt of wave w: rows q0b + 64 * qt + 16 * w .. + 15, so that every page staged for the
+  // block's first 64 rows is used by all four waves
+  int q0w[QT], row[QT], kmax[QT], kmin[QT];
+  bool valid[QT];
   Frag qf[QT][KS];
 #pragma unroll
-  for (int qt = 0; qt < QT; ++qt)
-    load_query<HD>(q + (size_t)(start + (valid ? row : n - 1)) * q_stride + (size_t)(h0 + (qt < n_h ? qt : 0)) * HD,
-                   valid && qt < n_h, qf[qt]);
+  for (int qt = 0; qt < QT; ++qt) {
+    q0w[qt] = q0b + 64 * qt + wave * 16;
+    row[qt] = q0w[qt] + r;
+    valid[qt] = row[qt] < n;
+    const int qpos = pos0 + row[qt];                             // rows past the end compute and are dropped
+    kmax[qt] = qpos;
+    kmin[qt] = (window > 0 && qpos - window + 1 > 0) ? qpos - window + 1 : 0;
+    load_query<HD>(q + (size_t)(start + (valid[qt] ? row[qt] : n - 1)) * q_stride + (size_t)h * HD, valid[qt], qf[qt]);
+  }
 
-  // pages of the block, and of this wave
-  const int last_row_b = (q0b + 63 < n) ? q0b + 63 : n - 1;
+  // pages of the block, and of this wave's tiles
+  const int last_row_b = (q0b + ROWS - 1 < n) ? q0b + ROWS - 1 : n - 1;
   const int pg_first = (window > 0 && pos0 + q0b - window + 1 > 0) ? (pos0 + q0b - window + 1) / PAGE : 0;
   const int pg_last = (pos0 + last_row_b) / PAGE;
-  const bool wave_live = q0w < n;
-  const int last_row_w = (q0w + 15 < n) ? q0w + 15 : n - 1;
-  const int wpg_first = (window > 0 && pos0 + q0w - window + 1 > 0) ? (pos0 + q0w - window + 1) / PAGE : 0;
-  const int wpg_last = wave_live ? (pos0 + last_row_w) / PAGE : -1;
+  int wpg_first[QT], wpg_last[QT];
+#pragma unroll
+  for (int qt = 0; qt < QT; ++qt) {
+    const int last_row_w = (q0w[qt] + 15 < n) ? q0w[qt] + 15 : n - 1;
+    wpg_first[qt] = (window > 0 && pos0 + q0w[qt] - window + 1 > 0) ? (pos0 + q0w[qt] - window + 1) / PAGE : 0;
+    wpg_last[qt] = (q0w[qt] < n) ? (pos0 + last_row_w) / PAGE : -1;
+  }
 
   f32x4 o[QT][DT], l_acc[QT];           // every row of l_acc holds the running sum of its column
   float m_run[QT];
@@ -226,7 +238,13 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     stage_page<HD>(k_lds, v_lds, kreg, vreg);
     __syncthreads();
     if (pg < pg_last) fetch_page<HD>(k_pages, v_pages, trow[pg + 1], n_kv, kvh, kreg, vreg);
-    if (pg < wpg_first || pg > wpg_last) continue;
+    // the last tile's rows are the latest and, with a window, a page of the first tile's is
+    // one of the last's too unless the window is shorter than the block; a page outside a tile's
+    // view is masked as a whole for it
+    bool live = false;
+#pragma unroll
+    for (int qt = 0; qt < QT; ++qt) live = live || (pg >= wpg_first[qt] && pg <= wpg_last[qt]);
+    if (!live) continue;
     const int key0 = pg * PAGE;
 
     // ---- scores S^T[key][query] for 64 keys and QT * 16 queries
@@ -250,8 +268,6 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
         for (int qt = 0; qt < QT; ++qt) sc[qt][t4] = mfma_bf16(a, qf[qt][ks], sc[qt][t4]);
       }
     }
-    // a page wholly inside every row's view needs no mask
-    const bool mask = (key0 + 63 > pos0 + q0w) || (window > 0 && key0 < pos0 + q0w + 15 - window + 1);
 
     // ---- running softmax per query column, probabilities as B fragments.  Maxima are taken of
     // the raw scores (the scale is positive) and the scale goes into the exponent's multiply-add.
@@ -259,19 +275,25 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     float corr[QT];
 #pragma unroll
     for (int qt = 0; qt < QT; ++qt) {
+      // a page wholly inside every row's view needs no mask
+      const bool mask = (key0 + 63 > pos0 + q0w[qt]) || (window > 0 && key0 < pos0 + q0w[qt] + 15 - window + 1);
       if (mask) {
 #pragma unroll
         for (int t4 = 0; t4 < 4; ++t4)
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const int key = key0 + (t4 >> 1) * 32 + 8 * g + 4 * (t4 & 1) + e;
-            if (key < kmin || key > kmax) sc[qt][t4][e] = -INFINITY;
+            if (key < kmin[qt] || key > kmax[qt]) sc[qt][t4][e] = -INFINITY;
           }
       }
-      float mx = fmaxf(fmaxf(sc[qt][0][0], sc[qt][0][1]), fmaxf(sc[qt][0][2], sc[qt][0][3]));
-#pragma unroll
-      for (int t4 = 1; t4 < 4; ++t4)
-        mx = fmaxf(mx, fmaxf(fmaxf(sc[qt][t4][0], sc[qt][t4][1]), fmaxf(sc[qt][t4][2], sc[qt][t4][3])));
+      float mx = max3(sc[qt][0][0], sc[qt][0][1], sc[qt][0][2]);
+      mx = max3(mx, sc[qt][0][3], sc[qt][1][0]);
+      mx = max3(mx, sc[qt][1][1], sc[qt][1][2]);
+      mx = max3(mx, sc[qt][1][3], sc[qt][2][0]);
+      mx = max3(mx, sc[qt][2][1], sc[qt][2][2]);
+      mx = max3(mx, sc[qt][2][3], sc[qt][3][0]);
+      mx = max3(mx, sc[qt][3][1], sc[qt][3][2]);
+      mx = max3(mx, sc[qt][3][3], sc[qt][3][3]);
       mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
       mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
       const float m_new = fmaxf(m_run[qt], mx * scale_log2);
@@ -321,19 +343,17 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
     }
   }
 
-  if (valid) {
 #pragma unroll
-    for (int qt = 0; qt < QT; ++qt) {
-      if (qt >= n_h) break;
-      const float inv = 1.0f / l_acc[qt][0];
-      bf16_t* orow = out + (size_t)(start + row) * n_heads * HD + (size_t)(h0 + qt) * HD;
+  for (int qt = 0; qt < QT; ++qt) {
+    if (!valid[qt]) continue;
+    const float inv = 1.0f / l_acc[qt][0];
+    bf16_t* orow = out + (size_t)(start + row[qt]) * n_heads * HD + (size_t)h * HD;
 #pragma unroll
-      for (int dt = 0; dt < DT; ++dt) {
-        uint2 pk;
-        pk.x = (uint32_t)f32_to_bf16(o[qt][dt][0] * inv) | ((uint32_t)f32_to_bf16(o[qt][dt][1] * inv) << 16);
-        pk.y = (uint32_t)f32_to_bf16(o[qt][dt][2] * inv) | ((uint32_t)f32_to_bf16(o[qt][dt][3] * inv) << 16);
-        *reinterpret_cast<uint2*>(orow + dt * 16 + 4 * g) = pk;
-      }
+    for (int dt = 0; dt < DT; ++dt) {
+      uint2 pk;
+      pk.x = (uint32_t)f32_to_bf16(o[qt][dt][0] * inv) | ((uint32_t)f32_to_bf16(o[qt][dt][1] * inv) << 16);
+      pk.y = (uint32_t)f32_to_bf16(o[qt][dt][2] * inv) | ((uint32_t)f32_to_bf16(o[qt][dt][3] * inv) << 16);
+      *reinterpret_cast<uint2*>(orow + dt * 16 + 4 * g) = pk;
     }
   }
 }
@@ -615,27 +635,30 @@ extern "C" int llm_attention_prefill_bf16(const void* q, int q_stride, const voi
                                           int page_size, const int* seq_start, const int* seq_slot,
                                           const int* seq_pos0, void* out, int n_seqs, int max_new,
                                           int n_heads, int n_kv, int hd, float scale, int window,
-                                          hipStream_t stream) {
+                                          int tiles, hipStream_t stream) {
   if (n_seqs <= 0 || max_new <= 0) return LLM_OK;
-  if (page_size != PAGE || !attn_args_ok(q, q_stride, k_pages, v_pages, n_heads, n_kv, hd, window) ||
+  if ((tiles != 1 && tiles != 2) || page_size != PAGE || !attn_args_ok(q, q_stride, k_pages, v_pages, n_heads, n_kv, hd, window) ||
       n_heads > 65535 || n_seqs > 65535)
     return LLM_ERR_ARG;
   const float scale_log2 = scale * 1.4426950408889634f;
-  const int group = n_heads / n_kv;
-  // One query head per block measured fastest (more blocks in flight, better balance between
-  // short and long rows) although a page is then staged once per query head of its group.
-  const int n_chunks = group;
-  const int n_qblocks = (max_new + 63) / 64;
-  const long long blocks = (long long)n_qblocks * n_kv * n_chunks * n_seqs;
+  // tiles: tiles of 16 rows a wave takes, so a block covers 64 or 128 rows.  Two halve the reads
+  // from shared memory and the staging per row; the caller chooses (one balances short and long
+  // rows better while the blocks are few).
+  const int qt = tiles;
+  const int n_qblocks = (max_new + 64 * qt - 1) / (64 * qt);
+  const long long blocks = (long long)n_qblocks * n_heads * n_seqs;
   if (blocks > 0x7fffffffLL) return LLM_ERR_ARG;
 #define LAUNCH(D, Q)                                                                              \
   attn_prefill_kernel<D, Q><<<(unsigned)blocks, 256, 0, stream>>>(                                \
       (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, table,          \
       table_stride, seq_start, seq_slot, seq_pos0, (bf16_t*)out, n_heads, n_kv, scale_log2,       \
-      window, n_qblocks, n_chunks)
+      window, n_qblocks)
 #define CASE(D)                                                                                   \
   if (hd == D) {                                                                                  \
-    LAUNCH(D, 1);                                                                                 \
+    if (qt == 2)                                                                                  \
+      LAUNCH(D, 2);                                                                               \
+    else                                                                                          \
+      LAUNCH(D, 1);                                                                               \
     return llm_launch_status();                                                                   \
   }
   FOR_HEAD_DIMS(CASE)

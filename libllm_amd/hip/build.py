@@ -22,9 +22,14 @@ ARCH = "gfx950"
 _HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(os.path.dirname(_HERE), "csrc")
 LIB_NAME = "libllm_amd_hip.so"
-# packed FP32 instructions stay switched off for every kernel of this library
+# Packed FP32 instructions stay switched off for every kernel of this library.  The sums of the
+# matrix cores stay in ordinary vector registers (gfx950 has one register file for both kinds):
+# left to itself the compiler keeps them in accumulation registers and moves them out and back
+# for every other instruction that touches them, two moves a value and page in the attention
+# kernels, where instruction issue is what bounds the time.
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17",
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-mllvm", "-amdgpu-mfma-vgpr-form=1"]
 
 _lib: Optional[ctypes.CDLL] = None
 

@@ -45,7 +45,7 @@ _SIGNATURES = {
     "llm_gemm_skinny_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "llm_attention_mfma_supported": [_i],
     "llm_attention_prefill_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i,
-                                   _i, _i, _f, _i, _vp],
+                                   _i, _i, _f, _i, _i, _vp],
     "llm_attention_decode_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i,
                                   _i, _i, _i, _f, _i, _i, _vp],
     "llm_attention_decode_waves": [_i],
@@ -86,6 +86,7 @@ class HipOps:
     ACCUM_ROWS = 16         # most rows for which a product adds into the stream itself
     SPLIT_ROWS = 64         # beyond those and up to here it goes in slices of K that the next norm adds; then the library's
     DECODE_BLOCKS = 768     # blocks of the decode attention grid beyond which sequences are not split further
+    PROMPT_TILE_BLOCKS = (1024, 768)   # blocks of 128 rows from which a wave of prompt attention takes two tiles of rows: heads up to 64 wide, wider ones
     _EPI_NONE, _EPI_SWIGLU, _EPI_ACCUM = 0, 1, 2
 
     def __init__(self, device: Optional[str] = None):
@@ -107,6 +108,7 @@ class HipOps:
         self.fast_attention = True      # bfloat16 attention on the matrix cores (else the plain kernel, as for float32)
         self.pack_weights = True        # keep a tiled copy of every weight for the skinny product
         self.fast_gemm = True           # the skinny product for few rows (else the library's for every product)
+        self.prompt_tiles = 0           # tiles of rows a wave of prompt attention takes (1 or 2; 0: by the number of blocks)
 
     # ---- helpers
     def _stream(self):
@@ -502,11 +504,15 @@ class HipOps:
                     ctx.seq_pos0.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), m, n_heads, n_kv, hd, float(scale),
                     int(window), n_blocks, self._stream()), "attention_decode_bf16")
             else:
+                tiles = self.prompt_tiles
+                if not tiles:
+                    blocks = -(-ctx.max_new // 128) * n_heads * ctx.n_seqs
+                    tiles = 2 if blocks >= self.PROMPT_TILE_BLOCKS[0 if hd <= 64 else 1] else 1
                 self._check(self.lib.llm_attention_prefill_bf16(
                     qkv.data_ptr(), width, kv.k_pages.data_ptr(), kv.v_pages.data_ptr(),
                     table.data_ptr(), table.shape[1], 64, ctx.seq_start.data_ptr(),
                     ctx.seq_slot.data_ptr(), ctx.seq_pos0.data_ptr(), out.data_ptr(), ctx.n_seqs,
-                    ctx.max_new, n_heads, n_kv, hd, float(scale), int(window), self._stream()),
+                    ctx.max_new, n_heads, n_kv, hd, float(scale), int(window), tiles, self._stream()),
                     "attention_prefill_bf16")
             return out
         self._check(self.lib.llm_attention_ref(

@@ -559,7 +559,7 @@ def test_rope_pairing_and_sign(ops):
 
 
 # ------------------------------------------------------------------------------- attention
-def run_attention(ops, dtype, n_heads, n_kv, hd, seqs, window=0, seed=0, boost=None, fast=True):
+def run_attention(ops, dtype, n_heads, n_kv, hd, seqs, window=0, seed=0, boost=None, fast=True, tiles=0):
     """seqs: (slot, past, new).  Returns (out, oracle) over all new tokens."""
     ctx = make_ctx(ops, dtype, seqs)
     pages = max((p + n + PAGE - 1) // PAGE for _, p, n in seqs)
@@ -578,11 +578,11 @@ def run_attention(ops, dtype, n_heads, n_kv, hd, seqs, window=0, seed=0, boost=N
             qt = q[o + t, :n_heads * hd].double().reshape(n_heads, hd)
             ref.append(attention_oracle(qt, keys.double(), vals.double(), past + t, scale, window).reshape(-1))
         o += new
-    ops.fast_attention = fast
+    ops.fast_attention, ops.prompt_tiles = fast, tiles
     try:
         out = ops.attention(q.cuda(), n_heads, n_kv, hd, ctx, kv, scale, window)
     finally:
-        ops.fast_attention = True
+        ops.fast_attention, ops.prompt_tiles = True, 0
     return out.double().cpu(), torch.stack(ref)
 
 
@@ -634,6 +634,42 @@ def test_attention_far_key_stands_out(ops, dtype, far):
     for seqs in ([(0, 900, 1)], [(0, 0, 901)]):
         out, ref = run_attention(ops, dtype, 4, 2, 64, seqs, seed=9, boost=(far, 12.0))
         assert max_err(out, ref) < (1e-5 if dtype == torch.float32 else BF16_2ULP)
+
+
+@pytest.mark.parametrize("tiles", [1, 2])
+@pytest.mark.parametrize("hd,window", [(16, 0), (64, 0), (64, 70), (80, 5), (128, 0), (128, 130), (256, 64)])
+def test_prompt_attention_tiles_of_rows(ops, hd, window, tiles):
+    """A wave of the prompt kernel takes one or two tiles of 16 rows (blocks of 64 or 128 rows),
+    by the number of blocks; here both are forced on small cases: prompts that end inside the first
+    and inside the second half of a block, a continued one that crosses pages, a single token, and
+    windows shorter and longer than a block."""
+    seqs = [(1, 0, 70), (0, 100, 137), (2, 300, 1), (3, 0, 200), (4, 40, 128)]
+    out, ref = run_attention(ops, torch.bfloat16, 6, 3, hd, seqs, window=window, seed=hd + window, tiles=tiles)
+    assert max_err(out, ref) < BF16_2ULP
+    out, ref = run_attention(ops, torch.bfloat16, 4, 2, hd, [(0, 0, 901)], window=window, seed=9,
+                             boost=(63 if window else 700, 12.0), tiles=tiles)
+    assert max_err(out, ref) < BF16_2ULP
+
+
+def test_prompt_attention_takes_two_tiles_when_blocks_are_many(ops):
+    """Left to itself the launcher takes two tiles a wave from 1,024 blocks of 128 rows on; a row's
+    bits do not depend on it."""
+    n_heads, n_kv, hd, rows = 32, 8, 64, 2048
+    seqs = [(0, 0, rows), (1, 64, rows - 100)]
+    assert -(-rows // 128) * n_heads * len(seqs) >= ops.PROMPT_TILE_BLOCKS[0]
+    ctx = make_ctx(ops, torch.bfloat16, seqs)
+    kv = make_kv("cuda", torch.bfloat16, 2, (rows + 64) // PAGE + 1, n_kv, hd, seed=2)
+    kv.k_pages.normal_(); kv.v_pages.normal_()
+    q = rnd((ctx.n_tokens, n_heads * hd), torch.bfloat16, 5).cuda()
+    outs = []
+    for tiles in (0, 1, 2):
+        ops.prompt_tiles = tiles
+        try:
+            outs.append(ops.attention(q, n_heads, n_kv, hd, ctx, kv, hd ** -0.5, 0))
+        finally:
+            ops.prompt_tiles = 0
+    assert torch.equal(outs[0], outs[1]) and torch.equal(outs[0], outs[2])
+    assert outs[0].float().abs().max() < 10 and torch.isfinite(outs[0].float()).all()
 
 
 @pytest.mark.parametrize("ctx_len,far", [(2100, 5), (9000, 4321), (9000, 8999)])
