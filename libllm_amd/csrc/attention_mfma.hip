@@ -25,6 +25,21 @@ __device__ __forceinline__ float max3(float a, float b, float c) {
   asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
   return r;
 }
+__device__ __forceinline__ float max2(float a, float b) {
+  float r;
+  asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+  return r;
+}
+
+// The largest of x over the four lanes that share lane % 16, in all four: the halves of the wave
+// swapped, then the rows of 16 lanes, in registers (a shuffle goes through shared memory).
+__device__ __forceinline__ float max_over_lane_groups(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const auto h = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+  const uint32_t v = __float_as_uint(max2(__uint_as_float(h[0]), __uint_as_float(h[1])));
+  const auto q = __builtin_amdgcn_permlane16_swap(v, v, false, false);
+  return max2(__uint_as_float(q[0]), __uint_as_float(q[1]));
+}
 
 template <int HD>
 struct AttnState {
@@ -293,10 +308,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
       mx = max3(mx, sc[qt][2][1], sc[qt][2][2]);
       mx = max3(mx, sc[qt][2][3], sc[qt][3][0]);
       mx = max3(mx, sc[qt][3][1], sc[qt][3][2]);
-      mx = max3(mx, sc[qt][3][3], sc[qt][3][3]);
-      mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-      mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-      const float m_new = fmaxf(m_run[qt], mx * scale_log2);
+      mx = max_over_lane_groups(max2(mx, sc[qt][3][3]));
+      const float m_new = max2(m_run[qt], mx * scale_log2);
       const float m_safe = (m_new > -INFINITY) ? m_new : 0.f;    // nothing seen yet: every p is 2^-inf = 0
       corr[qt] = fast_exp2(m_run[qt] - m_safe);
       m_run[qt] = m_new;

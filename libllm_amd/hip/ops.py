@@ -86,7 +86,7 @@ class HipOps:
     ACCUM_ROWS = 16         # most rows for which a product adds into the stream itself
     SPLIT_ROWS = 64         # beyond those and up to here it goes in slices of K that the next norm adds; then the library's
     DECODE_BLOCKS = 768     # blocks of the decode attention grid beyond which sequences are not split further
-    PROMPT_TILE_BLOCKS = (1024, 768)   # blocks of 128 rows from which a wave of prompt attention takes two tiles of rows: heads up to 64 wide, wider ones
+    PROMPT_TILE_BLOCKS = (1024, 768)   # blocks of 128 rows from which a wave of prompt attention takes two tiles of rows: heads up to 64 wide, up to 128 (wider ones never: one wave a unit would be left)
     _EPI_NONE, _EPI_SWIGLU, _EPI_ACCUM = 0, 1, 2
 
     def __init__(self, device: Optional[str] = None):
@@ -507,7 +507,7 @@ class HipOps:
                 tiles = self.prompt_tiles
                 if not tiles:
                     blocks = -(-ctx.max_new // 128) * n_heads * ctx.n_seqs
-                    tiles = 2 if blocks >= self.PROMPT_TILE_BLOCKS[0 if hd <= 64 else 1] else 1
+                    tiles = 2 if hd <= 128 and blocks >= self.PROMPT_TILE_BLOCKS[0 if hd <= 64 else 1] else 1
                 self._check(self.lib.llm_attention_prefill_bf16(
                     qkv.data_ptr(), width, kv.k_pages.data_ptr(), kv.v_pages.data_ptr(),
                     table.data_ptr(), table.shape[1], 64, ctx.seq_start.data_ptr(),
