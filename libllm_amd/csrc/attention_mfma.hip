@@ -40,6 +40,24 @@ __device__ __forceinline__ float max_over_lane_groups(float x) {
   const auto q = __builtin_amdgcn_permlane16_swap(v, v, false, false);
   return max2(__uint_as_float(q[0]), __uint_as_float(q[1]));
 }
+// The sum likewise: neighbouring rows of 16 lanes first, then the halves of the wave.
+__device__ __forceinline__ float sum_over_lane_groups(float x) {
+  const uint32_t u = __float_as_uint(x);
+  const auto q = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+  const uint32_t v = __float_as_uint(__uint_as_float(q[0]) + __uint_as_float(q[1]));
+  const auto h = __builtin_amdgcn_permlane32_swap(v, v, false, false);
+  return __uint_as_float(h[0]) + __uint_as_float(h[1]);
+}
+__device__ __forceinline__ float max_of_16(const f32x4 (&s)[4]) {
+  float mx = max3(s[0][0], s[0][1], s[0][2]);
+  mx = max3(mx, s[0][3], s[1][0]);
+  mx = max3(mx, s[1][1], s[1][2]);
+  mx = max3(mx, s[1][3], s[2][0]);
+  mx = max3(mx, s[2][1], s[2][2]);
+  mx = max3(mx, s[2][3], s[3][0]);
+  mx = max3(mx, s[3][1], s[3][2]);
+  return max2(mx, s[3][3]);
+}
 
 template <int HD>
 struct AttnState {
@@ -301,14 +319,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
             if (key < kmin[qt] || key > kmax[qt]) sc[qt][t4][e] = -INFINITY;
           }
       }
-      float mx = max3(sc[qt][0][0], sc[qt][0][1], sc[qt][0][2]);
-      mx = max3(mx, sc[qt][0][3], sc[qt][1][0]);
-      mx = max3(mx, sc[qt][1][1], sc[qt][1][2]);
-      mx = max3(mx, sc[qt][1][3], sc[qt][2][0]);
-      mx = max3(mx, sc[qt][2][1], sc[qt][2][2]);
-      mx = max3(mx, sc[qt][2][3], sc[qt][3][0]);
-      mx = max3(mx, sc[qt][3][1], sc[qt][3][2]);
-      mx = max_over_lane_groups(max2(mx, sc[qt][3][3]));
+      const float mx = max_over_lane_groups(max_of_16(sc[qt]));
       const float m_new = max2(m_run[qt], mx * scale_log2);
       const float m_safe = (m_new > -INFINITY) ? m_new : 0.f;    // nothing seen yet: every p is 2^-inf = 0
       corr[qt] = fast_exp2(m_run[qt] - m_safe);
@@ -430,13 +441,8 @@ __device__ __forceinline__ void compute_page(const PageFrags<HD>& f, const Frag 
     }
     s[t4] = acc;
   }
-  float mx = -INFINITY;
-#pragma unroll
-  for (int t4 = 0; t4 < 4; ++t4)
-    mx = fmaxf(mx, fmaxf(fmaxf(s[t4][0], s[t4][1]), fmaxf(s[t4][2], s[t4][3])));
-  mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
-  mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
-  const float m_new = fmaxf(st.m, mx * scale_log2);
+  const float mx = max_over_lane_groups(max_of_16(s));
+  const float m_new = max2(st.m, mx * scale_log2);
   const float m_safe = (m_new > -INFINITY) ? m_new : 0.f;      // nothing seen yet: every p is 0
   const float corr = fast_exp2(st.m - m_safe);
   float sum = 0.f;
@@ -453,9 +459,7 @@ __device__ __forceinline__ void compute_page(const PageFrags<HD>& f, const Frag 
       sum += __uint_as_float(pk << 16) + __uint_as_float(pk & 0xffff0000u);   // the rounded values
     }
   }
-  sum += __shfl_xor(sum, 16, 64);
-  sum += __shfl_xor(sum, 32, 64);
-  st.l = st.l * corr + sum;
+  st.l = st.l * corr + sum_over_lane_groups(sum);
   st.m = m_new;
 #pragma unroll
   for (int dt = 0; dt < HD / 16; ++dt) {
