@@ -21,6 +21,15 @@
 // token's position (src/libllm/llama.cc:151-176 pairs j with j + rot_dim/2; the reordering only
 // moves them side by side), rotated q to the output, rotated k and v to the token's place in the
 // paged cache (keys [page, kv_head, position, dim], values [page, kv_head, dim, position]).
+//
+// An RMS norm between two such products needs no kernel of its own (up to 16 rows): y = x w s with
+// s = rsqrt(mean(x^2) + eps) a factor of the whole row, so (x w s) W^T = s ((x w) W^T).  The
+// product that adds into the stream also stores the new stream times the next norm's weight,
+// rounded to bfloat16, and the sums of squares of the new stream over its tiles of 16 columns; the
+// product that follows takes those rows as its X, adds the sums of squares of a row in a fixed
+// order, and multiplies its sums by s before its own epilogue.  The statistics are those of the
+// 32-bit stream, as in the norm kernel (src/flint/cuda/rms_norm.cu:45-76); a row is rounded once,
+// before instead of after its scale.
 #include "mfma.h"
 
 #define SK_WK 8            // waves that split K
@@ -44,13 +53,22 @@ struct SkinnyRope {
   int table_stride, n_heads, n_kv, hd, rot_dim, write_kv;
 };
 
+struct SkinnyNorm {
+  const float* next_w;     // accumulating epilogue: weight [N] of the norm that reads the stream next, or null
+  bf16_t* raw;             //   out [M, N]: the new stream times next_w
+  float* ssq_out;          //   out [M, N / 16]: sums of squares of the new stream over tiles of 16 columns
+  const float* ssq_in;     // [M, parts_in]: such sums for the rows of X, which still lack their scale; or null
+  int parts_in;
+  float eps;
+};
+
 template <int MT, int RT, int WN, int G, int EPI, typename OutT>
 __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_t* __restrict__ X,
                                                                       const bf16_t* __restrict__ W,
                                                                       OutT* __restrict__ C, int M,
                                                                       int N, int K, int ldw,
                                                                       int n_out, int ldx, int w_steps,
-                                                                      SkinnyRope rope) {
+                                                                      SkinnyRope rope, SkinnyNorm norm) {
   constexpr int NT = WN * SK_WK * 64;
   constexpr int CK = 512 * G;                    // elements of K per chunk
   constexpr int ROW_B = CK * 2;                  // bytes of a staged row; 16-byte pieces are swizzled
@@ -61,6 +79,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   constexpr int ROWS_PASS = NT / XV;             // rows staged per pass of the block
   constexpr int PASSES = (16 * MT + ROWS_PASS - 1) / ROWS_PASS;
   __shared__ __attribute__((aligned(16))) unsigned char lds[LDS_BYTES];
+  __shared__ float s_scale[16 * MT];             // a row's rsqrt(mean(x^2) + eps) where X lacks it
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int wn = wave / SK_WK, wk = wave % SK_WK;
@@ -172,7 +191,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   const bool e_on = tid < ITEMS && e_m < M;
   int e_pos = 0, e_page = 0;
   float2 e_cos[EPI == SK_EPI_ROPE ? OUT_RT : 1], e_sin[EPI == SK_EPI_ROPE ? OUT_RT : 1];
-  float e_prev[EPI == SK_EPI_ACCUM ? OUT_RT : 1][4];
+  float e_prev[EPI == SK_EPI_ACCUM ? OUT_RT : 1][4], e_nw[EPI == SK_EPI_ACCUM ? OUT_RT : 1][4];
   if (EPI == SK_EPI_ROPE && e_on) {
     e_pos = rope.tok_pos[e_m];
     const int q_dim = rope.n_heads * rope.hd, kv_dim = rope.n_kv * rope.hd;
@@ -202,8 +221,24 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
     for (int ort = 0; ort < OUT_RT; ++ort) {
       const int n = e_n0 + ort * 16;
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
+      for (int e = 0; e < 4; ++e) {
         e_prev[ort][e] = (n + e < ldc) ? Conv<OutT>::load(C + (size_t)e_m * ldc + n + e) : 0.f;
+        e_nw[ort][e] = (norm.next_w != nullptr && n + e < ldc) ? norm.next_w[n + e] : 0.f;
+      }
+    }
+  }
+  if constexpr (MT == 1) {                       // (the host asks for it with up to 16 rows only)
+    if (norm.ssq_in != nullptr) {
+      // TPR threads a row add its sums of squares: each every TPR-th one, then across the threads
+      constexpr int TPR = NT / 16;
+      static_assert(TPR <= 64 && (TPR & (TPR - 1)) == 0, "the threads of a row lie in one wave");
+      const int row = tid / TPR, part = tid % TPR;
+      float ss = 0.f;
+      if (row < M)
+        for (int p = part; p < norm.parts_in; p += TPR) ss += norm.ssq_in[(size_t)row * norm.parts_in + p];
+#pragma unroll
+      for (int off = TPR / 2; off >= 1; off >>= 1) ss += __shfl_xor(ss, off, 64);
+      if (part == 0) s_scale[row] = rsqrtf(ss / (float)K + norm.eps);   // read after the loop's barriers
     }
   }
 #define SK_STEP(C, CUR, NXT)                    \
@@ -250,6 +285,14 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
         gsum[0] += pg.x; gsum[1] += pg.y; gsum[2] += pg.z; gsum[3] += pg.w;
         usum[0] += pu.x; usum[1] += pu.y; usum[2] += pu.z; usum[3] += pu.w;
       }
+      if (norm.ssq_in != nullptr) {
+        const float sc = s_scale[e_m];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          gsum[e] *= sc;
+          usum[e] *= sc;
+        }
+      }
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const float gt = bf16_to_f32(f32_to_bf16(gsum[e])), up = bf16_to_f32(f32_to_bf16(usum[e]));
@@ -263,8 +306,9 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
             red + (((w * WN + w_n) * MT + mt) * 64 + ln) * 4);
         sum[0] += p.x; sum[1] += p.y; sum[2] += p.z; sum[3] += p.w;
       }
+      const float sc = (norm.ssq_in != nullptr) ? s_scale[e_m] : 1.0f;
 #pragma unroll
-      for (int e = 0; e < 4; ++e) v[e] = sum[e];
+      for (int e = 0; e < 4; ++e) v[e] = (norm.ssq_in != nullptr) ? sum[e] * sc : sum[e];
     }
     const int m = e_m;
     if (EPI == SK_EPI_ROPE) {
@@ -306,6 +350,27 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
       }
       continue;
     }
+    if (EPI == SK_EPI_ACCUM && norm.next_w != nullptr) {
+      // (N is a multiple of 16 here: a tile is whole or absent; every lane of the wave comes along)
+      const bool on = m < M && n < ldc;
+      float ss = 0.f;
+      if (on) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          v[e] += e_prev[ort][e];
+          ss += v[e] * v[e];
+        }
+        *reinterpret_cast<float4*>(C + (size_t)m * ldc + n) = make_float4(v[0], v[1], v[2], v[3]);
+        uint2 pk;
+        pk.x = pack2_bf16(v[0] * e_nw[ort][0], v[1] * e_nw[ort][1]);
+        pk.y = pack2_bf16(v[2] * e_nw[ort][2], v[3] * e_nw[ort][3]);
+        *reinterpret_cast<uint2*>(norm.raw + (size_t)m * ldc + n) = pk;
+      }
+      ss += __shfl_xor(ss, 16, 64);                  // the four lanes that hold a row's 16 columns
+      ss += __shfl_xor(ss, 32, 64);
+      if (on && (ln >> 4) == 0) norm.ssq_out[(size_t)m * (ldc / 16) + n / 16] = ss;
+      continue;
+    }
     if (m >= M || n >= ldc) continue;
     OutT* dst = C + ((size_t)blockIdx.y * M + m) * ldc + n;
     if (EPI == SK_EPI_ACCUM) {
@@ -338,6 +403,7 @@ struct SkinnyArgs {
   int k_split;                 // slices of K, each to a result matrix of its own (1: the whole product)
   hipStream_t stream;
   SkinnyRope rope;
+  SkinnyNorm norm;
 };
 
 template <int MT, int RT, int WN, int G, int EPI, typename OutT>
@@ -348,7 +414,8 @@ static int launch_skinny(const SkinnyArgs& a) {
   const int blocks = (tiles + OUT_RT * WN - 1) / (OUT_RT * WN);
   const dim3 grid(blocks, a.k_split);
   gemm_skinny_kernel<MT, RT, WN, G, EPI, OutT><<<grid, WN * SK_WK * 64, 0, a.stream>>>(
-      a.X, a.W, (OutT*)a.C, a.M, a.N, a.K / a.k_split, a.ldw, a.n_out, a.K, (a.K + 31) / 32, a.rope);
+      a.X, a.W, (OutT*)a.C, a.M, a.N, a.K / a.k_split, a.ldw, a.n_out, a.K, (a.K + 31) / 32, a.rope,
+      a.norm);
   return llm_launch_status();
 }
 
@@ -400,9 +467,9 @@ static int pick_shape(const SkinnyArgs& a) {
 // the k_split slices of K, for the caller to add in order.
 // C[M, N] (epilogue 0: stored as out_dtype; 2: added into the float32 C) or C[M, N/2] (epilogue 1,
 // SwiGLU over W = [Wg; Wu], N/2 a multiple of 16) from X[M, K] and W[N, K].  X is bfloat16.
-extern "C" int llm_gemm_skinny_bf16(const void* X, const void* W, void* C,
-                                    int epilogue, int out_dtype, int M, int N, int K, int ldw,
-                                    int k_split, hipStream_t stream) {
+static int skinny_product(const void* X, const void* W, void* C, int epilogue, int out_dtype, int M,
+                          int N, int K, int ldw, int k_split, const SkinnyNorm& norm,
+                          hipStream_t stream) {
   if (M <= 0 || N <= 0) return LLM_OK;
   // slices of K: more than 16 rows, plain epilogue, float32 results [k_split, M, N]
   if (k_split < 1 || (k_split > 1 && (M <= 16 || epilogue != SK_EPI_NONE || out_dtype != LLM_DTYPE_F32 ||
@@ -423,6 +490,7 @@ extern "C" int llm_gemm_skinny_bf16(const void* X, const void* W, void* C,
   a.k_split = k_split;
   a.stream = stream;
   a.rope = SkinnyRope{};
+  a.norm = norm;
   if (epilogue == SK_EPI_NONE) {
     if (out_dtype == LLM_DTYPE_BF16) return pick_shape<SK_EPI_NONE, bf16_t>(a);
     if (out_dtype == LLM_DTYPE_F32) return pick_shape<SK_EPI_NONE, float>(a);
@@ -437,6 +505,41 @@ extern "C" int llm_gemm_skinny_bf16(const void* X, const void* W, void* C,
   return LLM_ERR_ARG;
 }
 
+extern "C" int llm_gemm_skinny_bf16(const void* X, const void* W, void* C,
+                                    int epilogue, int out_dtype, int M, int N, int K, int ldw,
+                                    int k_split, hipStream_t stream) {
+  return skinny_product(X, W, C, epilogue, out_dtype, M, N, K, ldw, k_split, SkinnyNorm{}, stream);
+}
+
+// The same around an RMS norm that gets no kernel of its own (see the head of this file), for up
+// to 16 rows.  Epilogue 2 with next_w: beside adding into the float32 stream C[M, N] (N a multiple
+// of 16), raw[M, N] = bfloat16(C * next_w) and ssq_out[M, N / 16], the sums of squares of C over
+// tiles of 16 columns, are written for the product after the norm whose weight next_w is.
+// With ssq_in[M, parts_in]: X holds such rows, and the sums are multiplied by
+// rsqrt(sum(ssq_in[m]) / K + eps) before the epilogue (0 or 1).
+extern "C" int llm_gemm_skinny_norm_bf16(const void* X, const void* W, void* C, int epilogue,
+                                         int out_dtype, int M, int N, int K, int ldw,
+                                         const float* next_w, void* raw, float* ssq_out,
+                                         const float* ssq_in, int parts_in, float eps,
+                                         hipStream_t stream) {
+  if (M > 16) return LLM_ERR_ARG;
+  SkinnyNorm norm{};
+  if (next_w != nullptr) {
+    if (epilogue != SK_EPI_ACCUM || (N & 15) || raw == nullptr || ssq_out == nullptr || (((uintptr_t)raw) & 15))
+      return LLM_ERR_ARG;
+    norm.next_w = next_w;
+    norm.raw = (bf16_t*)raw;
+    norm.ssq_out = ssq_out;
+  }
+  if (ssq_in != nullptr) {
+    if (epilogue == SK_EPI_ACCUM || parts_in <= 0 || !(eps >= 0.f)) return LLM_ERR_ARG;
+    norm.ssq_in = ssq_in;
+    norm.parts_in = parts_in;
+    norm.eps = eps;
+  }
+  return skinny_product(X, W, C, epilogue, out_dtype, M, N, K, ldw, 1, norm, stream);
+}
+
 // The stacked q|k|v projection with the rotary epilogue (see the head of this file): rotated q as
 // bfloat16 [M, n_heads * hd] to `q_out`, k and v to the cache if write_kv.  N is
 // (n_heads + 2 n_kv) * hd with write_kv, else n_heads * hd; hd a multiple of 16, rot_dim even.
@@ -446,8 +549,11 @@ extern "C" int llm_gemm_skinny_rope_bf16(const void* X, const void* W,
                                          int rot_dim, const int* tok_pos, const int* tok_seq,
                                          const int* seq_slot, const int* table, int table_stride,
                                          void* k_pages, void* v_pages, int page_size, int write_kv,
+                                         const float* ssq_in, int parts_in, float eps,
                                          hipStream_t stream) {
   if (M <= 0) return LLM_OK;
+  // ssq_in: the rows of X still lack their norm's scale (see llm_gemm_skinny_norm_bf16), or null
+  if (ssq_in != nullptr && (M > 16 || parts_in <= 0 || !(eps >= 0.f))) return LLM_ERR_ARG;
   if (M > 64 || K <= 0 || (K & 7) || (ldw != 0 && (ldw < K || (ldw & 7))) || n_heads <= 0 || n_kv < 0 || hd <= 0 || (hd & 15) || rot_dim < 0 ||
       rot_dim > hd || (rot_dim & 1) || page_size != 64)
     return LLM_ERR_ARG;
@@ -483,6 +589,10 @@ extern "C" int llm_gemm_skinny_rope_bf16(const void* X, const void* W,
   a.rope.hd = hd;
   a.rope.rot_dim = rot_dim;
   a.rope.write_kv = write_kv;
+  a.norm = SkinnyNorm{};
+  a.norm.ssq_in = ssq_in;
+  a.norm.parts_in = parts_in;
+  a.norm.eps = eps;
   return pick_shape<SK_EPI_ROPE, bf16_t>(a);
 }
 

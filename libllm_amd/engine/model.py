@@ -119,8 +119,13 @@ class DecoderModel:
         s = self.spec
         res = ctx.ops.embed(self.embed_table, ctx.tokens, s.embedding.scale)
         stream = Stream(res)
-        for entry in s.schedule:
+        for i, entry in enumerate(s.schedule):
+            # the block is told which norm reads the stream after it, so that its last product
+            # may prepare that norm (the final norm gathers rows and is left alone)
+            nxt = s.schedule[i + 1] if i + 1 < len(s.schedule) else None
+            ctx.norm_after_block = self.blocks[nxt.layer].entry_norm() if nxt is not None else None
             self.blocks[entry.layer].forward(ctx, stream, entry)
+        ctx.norm_after_block = None
         if want_rows is None or want_rows.numel() == 0:
             return None
         h = self.final_norm.add_norm(ctx, stream, rows=want_rows, lazy=True)

@@ -37,12 +37,13 @@ _SIGNATURES = {
     "llm_rope_kv_write": [_vp, _i, _i, _vp, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp,
                           _vp, _i, _i, _i, _i, _vp],
     "llm_gemm_skinny_rope_bf16": [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _i,
-                                  _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _vp],
+                                  _vp, _vp, _vp, _vp, _i, _vp, _vp, _i, _i, _vp, _i, _f, _vp],
     "llm_pack_weight": [_vp, _vp, _i, _i, _i, _vp],
     "llm_gemm_f32": [_vp, _vp, _vp, _i, _i, _i, _vp],
     "llm_attention_ref": [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
                           _f, _i, _vp],
     "llm_gemm_skinny_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "llm_gemm_skinny_norm_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _f, _vp],
     "llm_attention_mfma_supported": [_i],
     "llm_attention_prefill_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i,
                                    _i, _i, _f, _i, _i, _vp],
@@ -57,12 +58,23 @@ _SIGNATURES = {
 }
 
 
+class Prenormed:
+    """What a product that added into the stream leaves for the norm with ``weight`` and ``eps``
+    that reads the stream next: ``raw`` = bfloat16(stream * weight) and ``ssq[M, width / 16]``, the
+    sums of squares of the stream's rows over tiles of 16 columns.  The product after that norm
+    takes ``raw`` as its rows and multiplies its sums by rsqrt(sum(ssq[m]) / width + eps)."""
+
+    def __init__(self, raw, ssq, weight, eps):
+        self.raw, self.ssq, self.weight, self.eps = raw, ssq, weight, eps
+
+
 class NormedRows:
     """Rows ``rows`` (all, if None) of the float32 matrix ``res``, to be RMS-normalised with
-    ``weight`` and ``eps``: what ``HipOps.normed`` returns."""
+    ``weight`` and ``eps``: what ``HipOps.normed`` returns.  ``pre``: what the product before
+    left for this norm, if it did."""
 
-    def __init__(self, res, weight, eps, rows=None):
-        self.res, self.weight, self.eps, self.rows = res, weight, eps, rows
+    def __init__(self, res, weight, eps, rows=None, pre=None):
+        self.res, self.weight, self.eps, self.rows, self.pre = res, weight, eps, rows, pre
         self.n_rows = res.shape[0] if rows is None else rows.shape[0]
 
 
@@ -80,6 +92,7 @@ class HipOps:
     checks its operands on the host before a kernel is launched."""
 
     supports_graphs = True
+    folds_norms = True      # ``linear`` takes ``then_norm`` and may return a ``Prenormed``
 
     # Launch decisions, each measured with variants side by side in one process:
     SKINNY_ROWS = 64        # most rows the streaming matrix product takes at once; beyond, the library's
@@ -108,6 +121,7 @@ class HipOps:
         self.fast_attention = True      # bfloat16 attention on the matrix cores (else the plain kernel, as for float32)
         self.pack_weights = True        # keep a tiled copy of every weight for the skinny product
         self.fast_gemm = True           # the skinny product for few rows (else the library's for every product)
+        self.fold_norms = True          # up to ACCUM_ROWS rows, a norm between two products gets no kernel of its own
         self.prompt_tiles = 0           # tiles of rows a wave of prompt attention takes (1 or 2; 0: by the number of blocks)
 
     # ---- helpers
@@ -234,12 +248,17 @@ class HipOps:
             return w.tiled.data_ptr(), 0
         return w.data_ptr(), w.stride(0)
 
-    def normed(self, res, weight, eps, rows=None):
+    def normed(self, res, weight, eps, rows=None, pre=None):
         """Rows of the float32 stream ``res`` that are to be RMS-normalised: a record that
         ``linear``, ``linear_swiglu`` and ``qkv_rope`` take in place of a matrix: they run the
-        norm kernel on just these rows, in the dtype they need.  (The norm fused into the product
-        itself was measured and lost: every block then normalises the rows again.)"""
-        return NormedRows(res, weight, float(eps), rows)
+        norm kernel on just these rows, in the dtype they need, or, with ``pre`` (what
+        ``linear(..., then_norm=)`` returned when it added into ``res``, nothing having touched
+        ``res`` since), take the rows the product before has left.  (The norm computed inside the
+        product itself was measured and lost: every block then normalises the rows again.)"""
+        if pre is not None and (rows is not None or pre.weight is not weight or pre.eps != float(eps)
+                                or pre.raw.shape != res.shape):
+            pre = None
+        return NormedRows(res, weight, float(eps), rows, pre)
 
     def _materialise(self, x, dtype):
         if isinstance(x, NormedRows):
@@ -252,7 +271,8 @@ class HipOps:
                 and w.stride(0) % 8 == 0):
             return False
         if isinstance(x, NormedRows):
-            return False                     # the norm kernel runs first; the product takes its rows
+            # rows left by the product before go straight in; else the norm kernel runs first
+            return x.pre is not None and m <= self.ACCUM_ROWS
         return x.dtype == torch.bfloat16 and x.data_ptr() % 16 == 0
 
     @staticmethod
@@ -268,18 +288,27 @@ class HipOps:
         """Launches the skinny kernel on rows m0 .. m0+mm of the bfloat16 matrix x; with ``k_split``
         the products over that many slices of K go to ``out[k_split, mm, n]``."""
         n, k = w.shape
-        xp = x.data_ptr() + m0 * k * 2
         width = n // 2 if epilogue == self._EPI_SWIGLU else n
         wptr, ldw = self._streamed(w)
+        if isinstance(x, NormedRows):           # rows that lack their norm's scale: see Prenormed
+            pre = x.pre
+            self._check(self.lib.llm_gemm_skinny_norm_bf16(
+                pre.raw.data_ptr(), wptr, out.data_ptr(), epilogue, _code(out.dtype), mm, n, k, ldw,
+                None, None, None, pre.ssq.data_ptr(), pre.ssq.shape[1], pre.eps, self._stream()),
+                "gemm_skinny_norm_bf16")
+            return
+        xp = x.data_ptr() + m0 * k * 2
         self._check(self.lib.llm_gemm_skinny_bf16(
             xp, wptr, out.data_ptr() + m0 * width * out.element_size(),
             epilogue, _code(out.dtype), mm, n, k, ldw, k_split, self._stream()), "gemm_skinny_bf16")
 
-    def linear(self, x, w, bias, out_dtype, residual=None):
+    def linear(self, x, w, bias, out_dtype, residual=None, then_norm=None):
         """x W^T (+ bias) as ``out_dtype``.  ``x`` is a matrix or a ``normed`` record.  With
         ``residual`` (the float32 stream, same shape as the result) the product is added into it
         where the kernel can do that, and None is returned; otherwise the result is returned and
-        the caller adds it."""
+        the caller adds it.  ``then_norm`` = (weight, eps) says that an RMS norm with these reads
+        ``residual`` next, before anything else touches it: where the product adds into the
+        stream at up to ``ACCUM_ROWS`` rows it then returns a ``Prenormed`` for ``normed``."""
         lazy = isinstance(x, NormedRows)
         m, k = (x.n_rows, x.res.shape[1]) if lazy else x.shape
         n, k2 = w.shape
@@ -301,6 +330,17 @@ class HipOps:
         if self._skinny_ok(x, w, m, k) and bias is None and not (residual is not None and m > self.ACCUM_ROWS):
             if residual is not None and m <= self.SKINNY_ROWS:
                 self._dev(residual, "residual stream", torch.float32, (m, n))
+                if then_norm is not None and self.fold_norms and n % 16 == 0 and not lazy:
+                    weight, eps = then_norm
+                    self._dev(weight, "norm weight", torch.float32, (n,))
+                    raw = torch.empty((m, n), dtype=torch.bfloat16, device=self.device)
+                    ssq = torch.empty((m, n // 16), dtype=torch.float32, device=self.device)
+                    wptr, ldw = self._streamed(w)
+                    self._check(self.lib.llm_gemm_skinny_norm_bf16(
+                        x.data_ptr(), wptr, residual.data_ptr(), self._EPI_ACCUM, _code(torch.float32),
+                        m, n, k, ldw, weight.data_ptr(), raw.data_ptr(), ssq.data_ptr(), None, 0, 0.0,
+                        self._stream()), "gemm_skinny_norm_bf16")
+                    return Prenormed(raw, ssq, weight, float(eps))
                 self._skinny(x, w, residual, self._EPI_ACCUM, 0, m)
                 return None
             if m <= self.SKINNY_ROWS or (out_dtype == torch.float32 and not lazy):
@@ -386,7 +426,10 @@ class HipOps:
         fused = (dtype == torch.bfloat16 and (adjacent or rot_dim == 0) and hd % 16 == 0
                  and m <= self.SKINNY_ROWS and m == ctx.n_tokens
                  and (not write or (kv is not None and kv.k_pages.dtype == torch.bfloat16)))
-        if fused and lazy:
+        pre = x.pre if lazy and fused and self._skinny_ok(x, w, m, k) else None
+        if pre is not None:
+            x, lazy = pre.raw, False             # rows that lack their norm's scale: see Prenormed
+        elif fused and lazy:
             x, lazy = self._materialise(x, dtype), False
         if fused and self._skinny_ok(x, w, m, k):
             self._weight(self._plain(w), "qkv weight")
@@ -416,7 +459,8 @@ class HipOps:
                 xp, wptr, bptr, q.data_ptr(), m, k, ldw, n_heads, n_kv, hd,
                 cptr, sptr, rot_dim, ctx.tok_pos.data_ptr(), ctx.tok_seq.data_ptr(),
                 ctx.seq_slot.data_ptr(), tptr, stride, kptr, vptr, 64, 1 if write else 0,
-                self._stream()), "gemm_skinny_rope_bf16")
+                pre.ssq.data_ptr() if pre is not None else None, pre.ssq.shape[1] if pre is not None else 0,
+                pre.eps if pre is not None else 0.0, self._stream()), "gemm_skinny_rope_bf16")
             return q
         qkv = self.linear(x, w, None, dtype)
         self.rope_kv_write(qkv, bias, n_heads, n_kv, hd, cos, sin, rot_dim, ctx, kv, write, adjacent)

@@ -73,6 +73,15 @@ class Stream:
     def __init__(self, res: torch.Tensor):
         self.res = res            # [tokens, width] float32
         self.delta = None         # [tokens, width] in the activation dtype, or None
+        self.pre = None           # what a product that added into ``res`` has left for the next norm
+
+    def put(self, out) -> None:
+        """Takes what a mixer or feed-forward returned: rows still to be added (a matrix), None
+        (it added them itself), or the record ``ops.linear(..., then_norm=)`` returned when it
+        added them and prepared the norm that comes next."""
+        is_rows = out is None or isinstance(out, torch.Tensor)
+        self.delta = out if is_rows else None
+        self.pre = None if is_rows else out
 
 
 class StepContext:
@@ -103,6 +112,11 @@ class StepContext:
         self.max_new = 0
         self.max_ctx = 0
         self.decode = False        # every sequence brings exactly one token
+        # (stream tensor, weight, eps) while the next thing to read that stream is an RMS norm
+        # with these, nothing else touching it in between: a product that adds into the stream
+        # may then prepare that norm (``ops.linear(..., then_norm=)``).  Set by blocks.
+        self.then_norm = None
+        self.norm_after_block = None   # the norm that reads the stream first after the running block, if known
         self.captured = False      # running under graph capture: host lists are not valid
         self._kv: Dict[int, KVView] = {}
         self._state: Dict[int, torch.Tensor] = {}
@@ -173,6 +187,11 @@ class Norm(Part):
     def add_norm(self, ctx: StepContext, stream: Stream, rows=None, lazy=False) -> torch.Tensor:
         raise NotImplementedError
 
+    def rms_terms(self):
+        """(weight, eps) if this is a plain RMS norm, y = x * weight * rsqrt(mean(x^2) + eps),
+        which a product before it may prepare; else None."""
+        return None
+
 
 class Block:
     """Arrangement of a mixer, a feed-forward and norms around the residual stream."""
@@ -184,3 +203,14 @@ class Block:
 
     def forward(self, ctx: StepContext, stream: Stream, entry) -> None:
         raise NotImplementedError
+
+    def entry_norm(self) -> Optional[Norm]:
+        """The norm that reads the stream first when this block runs, if nothing else touches
+        the stream before it; else None."""
+        return None
+
+    @staticmethod
+    def announce(ctx: StepContext, stream: Stream, norm: Optional[Norm]) -> None:
+        """Says (or, with None, takes back) that ``norm`` reads the stream next."""
+        terms = norm.rms_terms() if norm is not None else None
+        ctx.then_norm = (stream.res,) + tuple(terms) if terms else None

@@ -14,15 +14,23 @@ class PreNormBlock(Block):
             raise ConfigError("a prenorm block needs two norms, got %d" % len(norms))
         super().__init__(mixer, feed_forward, norms)
 
+    def entry_norm(self):
+        return self.norms[0]
+
     def forward(self, ctx: StepContext, stream: Stream, entry) -> None:
         mixer, ff = self.mixer, self.feed_forward
+        after = ctx.norm_after_block
         h = self.norms[0].add_norm(ctx, stream, lazy=mixer.takes_normed)
         if mixer.adds_to_stream:
-            stream.delta = mixer.forward(ctx, h, entry, residual=stream.res)
+            self.announce(ctx, stream, self.norms[1])
+            stream.put(mixer.forward(ctx, h, entry, residual=stream.res))
+            self.announce(ctx, stream, None)
         else:
-            stream.delta = mixer.forward(ctx, h, entry)
+            stream.put(mixer.forward(ctx, h, entry))
         h = self.norms[1].add_norm(ctx, stream, lazy=ff.takes_normed)
         if ff.adds_to_stream:
-            stream.delta = ff.forward(ctx, h, residual=stream.res)
+            self.announce(ctx, stream, after)
+            stream.put(ff.forward(ctx, h, residual=stream.res))
+            self.announce(ctx, stream, None)
         else:
-            stream.delta = ff.forward(ctx, h)
+            stream.put(ff.forward(ctx, h))

@@ -25,7 +25,12 @@ class Linear:
 
     def __call__(self, ctx, x, out_dtype=None, residual=None):
         """``x``: a matrix or an ``ops.normed`` record.  With ``residual`` the result may be added
-        into it, and None returned."""
+        into it, and None returned (or the record of a prepared norm: see ``Stream.put``)."""
         if residual is None:
             return ctx.ops.linear(x, self.prepared, self.bias, out_dtype or ctx.dtype)
+        hint = getattr(ctx, "then_norm", None)
+        if hint is not None and hint[0] is residual and getattr(ctx.ops, "folds_norms", False):
+            # an RMS norm reads the stream next: the product may prepare it, and then returns a record
+            return ctx.ops.linear(x, self.prepared, self.bias, out_dtype or ctx.dtype, residual=residual,
+                                  then_norm=hint[1:])
         return ctx.ops.linear(x, self.prepared, self.bias, out_dtype or ctx.dtype, residual=residual)

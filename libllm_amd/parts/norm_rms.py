@@ -29,8 +29,14 @@ class RMSNorm(Norm):
     def bind(self, tensors, ops, dtype):
         self.weight = tensors["weight"]
 
+    def rms_terms(self):
+        return self.weight, self.eps
+
     def add_norm(self, ctx: StepContext, stream: Stream, rows=None, lazy=False) -> torch.Tensor:
+        pre, stream.pre = stream.pre, None
         if lazy and stream.delta is None and hasattr(ctx.ops, "normed"):
+            if pre is not None:
+                return ctx.ops.normed(stream.res, self.weight, self.eps, rows, pre=pre)
             return ctx.ops.normed(stream.res, self.weight, self.eps, rows)
         out = ctx.ops.add_rmsnorm(stream.res, stream.delta, self.weight, self.eps, ctx.dtype, rows)
         stream.delta = None

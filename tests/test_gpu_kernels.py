@@ -281,6 +281,94 @@ def test_products_of_rows_still_to_be_normalised(ops, m, nk, gather):
         assert max_err(sw, g / (1 + torch.exp(-g)) * u) < 4 * BF16_2ULP
 
 
+@pytest.mark.parametrize("m", [1, 3, 8, 16])
+@pytest.mark.parametrize("nk", [(16, 8), (304, 520), (2048, 2048), (2048, 8192), (4096, 1032)])
+def test_product_prepares_the_norm_that_follows(ops, m, nk):
+    """A product that adds into the stream, told which RMS norm reads the stream next: the stream
+    gets the same bits as without, ``raw`` is the new stream times the norm's weight rounded once,
+    ``ssq`` holds the sums of squares over tiles of 16 columns; a row's values do not depend on
+    the other rows of the step."""
+    n, k = nk
+    x = rnd((m, k), torch.bfloat16, 90).cuda()
+    w = rnd((n, k), torch.bfloat16, 91).cuda()
+    pw = ops.prepare_weight(w)
+    nw = (1.0 + 0.3 * rnd((n,), torch.float32, 92)).cuda()
+    res = rnd((m, n), torch.float32, 93, 5.0).cuda()
+    res[0] *= 1e-3
+    plain = res.clone()
+    assert ops.linear(x, pw, None, torch.bfloat16, residual=plain) is None
+    pre = ops.linear(x, pw, None, torch.bfloat16, residual=res, then_norm=(nw, 1e-5))
+    assert pre is not None and pre.weight is nw and pre.eps == 1e-5
+    assert torch.equal(res, plain)
+    assert torch.equal(pre.raw, (res * nw).to(torch.bfloat16))
+    want = (res.double() ** 2).reshape(m, n // 16, 16).sum(-1)
+    assert tuple(pre.ssq.shape) == (m, n // 16) and max_err(pre.ssq, want) < 1e-6
+    one = rnd((m, n), torch.float32, 93, 5.0).cuda()
+    one[0] *= 1e-3
+    one = one[m - 1:].contiguous()
+    alone = ops.linear(x[m - 1:].contiguous(), pw, None, torch.bfloat16, residual=one, then_norm=(nw, 1e-5))
+    assert torch.equal(alone.raw[0], pre.raw[m - 1]) and torch.equal(alone.ssq[0], pre.ssq[m - 1])
+    # more rows than the product adds for, or a width that is no multiple of 16: no record
+    if m == 16:
+        big = rnd((17, n), torch.float32, 94).cuda()
+        out = ops.linear(rnd((17, k), torch.bfloat16, 95).cuda(), pw, None, torch.bfloat16, residual=big,
+                         then_norm=(nw, 1e-5))
+        assert out is None or isinstance(out, torch.Tensor)
+
+
+@pytest.mark.parametrize("m", [1, 5, 16])
+@pytest.mark.parametrize("width,n", [(2048, 3072), (2048, 16384), (528, 304), (4096, 1024)])
+def test_products_over_a_prepared_norm(ops, m, width, n):
+    """The product after a prepared norm takes ``raw`` as its rows and multiplies its sums by the
+    row's rsqrt(mean(x^2) + eps): plain product, SwiGLU and the rotary q|k|v product, against the
+    plain formulas in float64 and against the norm kernel followed by the same product."""
+    kin = 256
+    x = rnd((m, kin), torch.bfloat16, 96).cuda()
+    wo = ops.prepare_weight(rnd((width, kin), torch.bfloat16, 97, 0.5).cuda())
+    nw = (1.0 + 0.3 * rnd((width,), torch.float32, 98)).cuda()
+    res = rnd((m, width), torch.float32, 99, 4.0).cuda()
+    res[0] *= 1e-3
+    eps = 1e-5
+    pre = ops.linear(x, wo, None, torch.bfloat16, residual=res, then_norm=(nw, eps))
+    lazy = ops.normed(res, nw, eps, pre=pre)
+    assert lazy.pre is pre
+    assert ops.normed(res, nw, 1e-6, pre=pre).pre is None                 # another norm than the one prepared
+    assert ops.normed(res, nw.clone(), eps, pre=pre).pre is None
+    assert ops.normed(res, nw, eps, torch.arange(m, dtype=torch.int32, device="cuda"), pre=pre).pre is None
+    w = rnd((n, width), torch.bfloat16, 100).cuda()
+    pw = ops.prepare_weight(w)
+    rd = res.double()
+    h = rd * nw.double() / torch.sqrt((rd * rd).mean(-1, keepdim=True) + eps)
+    ref = h @ w.double().t()
+    hb = ops.add_rmsnorm(res, None, nw, eps, torch.bfloat16)              # the norm kernel's rows
+    for out_dtype in DTYPES:
+        out = ops.linear(lazy, pw, None, out_dtype)
+        assert out.dtype == out_dtype and max_err(out, ref) < (BF16_2ULP if out_dtype == torch.bfloat16 else 2.0 ** -8)
+    assert max_err(ops.linear(lazy, pw, None, torch.float32), ops.linear(hb, pw, None, torch.float32)) < 2.0 ** -7
+    if n % 32 == 0:
+        g, u = ref[:, :n // 2], ref[:, n // 2:]
+        sw = ops.linear_swiglu(lazy, pw, torch.bfloat16)
+        assert max_err(sw, g / (1 + torch.exp(-g)) * u) < 4 * BF16_2ULP
+        assert max_err(sw, ops.linear_swiglu(hb, pw)) < 4 * BF16_2ULP
+    # the rotary product: the same queries and cache as from the norm kernel's rows, up to rounding
+    hd = 64
+    if n % hd == 0 and n // hd >= 3:
+        n_kv = max(1, n // hd // 6)
+        n_heads = n // hd - 2 * n_kv
+        seqs = [(i, 3 * i, 1) for i in range(m)]
+        ctx = make_ctx(ops, torch.bfloat16, seqs)
+        cos = torch.cos(rnd((64, hd // 2), torch.float32, 101)).cuda()
+        sin = torch.sin(rnd((64, hd // 2), torch.float32, 101)).cuda()
+        outs = []
+        for rows in (lazy, hb):
+            kv = make_kv("cuda", torch.bfloat16, m, 1, n_kv, hd, seed=1)
+            q = ops.qkv_rope(rows, pw, None, n_heads, n_kv, hd, cos, sin, hd, ctx, kv, True, True, torch.bfloat16)
+            outs.append((q[:, :n_heads * hd].clone(), kv.k_pages.clone(), kv.v_pages.clone()))
+        for a, b in zip(*outs):
+            assert max_err(a, b) < BF16_2ULP
+        assert float(outs[0][1].float().abs().max()) > 0
+
+
 @pytest.mark.parametrize("m", [17, 33, 40, 64])
 @pytest.mark.parametrize("nk", [(128, 2048), (2048, 2048), (2048, 8192), (3072, 3072), (200, 1536)])
 def test_products_in_slices_of_k(ops, monkeypatch, m, nk):

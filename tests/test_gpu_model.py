@@ -182,6 +182,37 @@ def test_padding_changes_nothing(models):
     assert np.array_equal(a, b[:, :5])
 
 
+@pytest.mark.parametrize("name", list(CONFIGS))
+def test_norms_between_products_get_no_kernel(models, name):
+    """Decoding up to 16 rows in bfloat16, the product that adds into the stream prepares the RMS
+    norm after it and the next product applies the row's scale: the norm kernel then runs only
+    for the first norm of a step and the last.  Logits against the plain implementation, and
+    against an engine that runs every norm as a kernel."""
+    from libllm_amd.runtime import load_engine
+    path, cfg, weights = models[name]
+    requests = make_requests(cfg, [9, 30, 17, 6], seed=45)
+    folded = load_engine(path, dtype="bfloat16", max_tokens=1024, use_graphs=False)
+    kernels = load_engine(path, dtype="bfloat16", max_tokens=1024, use_graphs=False)
+    kernels.ops.fold_norms = False
+    calls = {}
+    for tag, e in (("folded", folded), ("kernels", kernels)):
+        real = e.ops.add_rmsnorm
+        def counted(*a, _real=real, _tag=tag, **k):
+            calls[_tag] = calls.get(_tag, 0) + 1
+            return _real(*a, **k)
+        e.ops.add_rmsnorm = counted
+    a, b = _decode_rows(folded, requests, 4), _decode_rows(kernels, requests, 4)
+    n_layers = len(folded.model.spec.schedule)
+    prompt = 2 * n_layers                                       # the prompt step: more than 16 rows, no logits wanted
+    assert calls["kernels"] == prompt + 4 * (2 * n_layers + 1)
+    assert calls["folded"] == prompt + 4 * 2
+    assert_logits_close(a, b.astype(np.float64), "bfloat16", "folded norms against norm kernels")
+    for i, (rid, toks) in enumerate(requests.items()):
+        ref = oracle(name, cfg, weights, toks)
+        for step in range(4):                                   # step s fed token -(4 - s): logits at that position
+            assert_logits_close(a[step, i][None], ref[len(toks) - 4 + step][None], "bfloat16", "%s step %d" % (rid, step))
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_batch_order_changes_nothing(models, dtype):
     """The same requests in the opposite order take other slots and other rows of every step.
