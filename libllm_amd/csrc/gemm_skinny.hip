@@ -227,18 +227,19 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
       }
     }
   }
+  // The sums of squares of a row of X that still lacks its scale: TPR threads a row, each asks
+  // for every TPR-th one now and adds them after the loop, when they have long arrived.
+  constexpr int TPR = NT / 16, SS_AHEAD = 8;
+  float e_ss[SS_AHEAD];
+  const int ss_row = tid / TPR, ss_part = tid % TPR;
   if constexpr (MT == 1) {                       // (the host asks for it with up to 16 rows only)
+    static_assert(TPR <= 64 && (TPR & (TPR - 1)) == 0, "the threads of a row lie in one wave");
     if (norm.ssq_in != nullptr) {
-      // TPR threads a row add its sums of squares: each every TPR-th one, then across the threads
-      constexpr int TPR = NT / 16;
-      static_assert(TPR <= 64 && (TPR & (TPR - 1)) == 0, "the threads of a row lie in one wave");
-      const int row = tid / TPR, part = tid % TPR;
-      float ss = 0.f;
-      if (row < M)
-        for (int p = part; p < norm.parts_in; p += TPR) ss += norm.ssq_in[(size_t)row * norm.parts_in + p];
 #pragma unroll
-      for (int off = TPR / 2; off >= 1; off >>= 1) ss += __shfl_xor(ss, off, 64);
-      if (part == 0) s_scale[row] = rsqrtf(ss / (float)K + norm.eps);   // read after the loop's barriers
+      for (int i = 0; i < SS_AHEAD; ++i) {
+        const int p = ss_part + i * TPR;
+        e_ss[i] = (ss_row < M && p < norm.parts_in) ? norm.ssq_in[(size_t)ss_row * norm.parts_in + p] : 0.f;
+      }
     }
   }
 #define SK_STEP(C, CUR, NXT)                    \
@@ -255,6 +256,20 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
     SK_STEP(c + 2, a[2], a[1])
   }
 #undef SK_STEP
+
+  if constexpr (MT == 1) {
+    if (norm.ssq_in != nullptr) {
+      float ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < SS_AHEAD; ++i) ss += e_ss[i];
+      if (ss_row < M)                            // rows wider than 16 * SS_AHEAD * TPR columns
+        for (int p = ss_part + SS_AHEAD * TPR; p < norm.parts_in; p += TPR)
+          ss += norm.ssq_in[(size_t)ss_row * norm.parts_in + p];
+#pragma unroll
+      for (int off = TPR / 2; off >= 1; off >>= 1) ss += __shfl_xor(ss, off, 64);
+      if (ss_part == 0) s_scale[ss_row] = rsqrtf(ss / (float)K + norm.eps);   // read behind the next barrier
+    }
+  }
 
   // ---- add the partial sums of the 8 waves in order, apply the epilogue, store: one output tile
   // of every row group a round (a gate and its up tile together), so that the buffer stays small
