@@ -388,7 +388,9 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(
 // if the group is larger).  The pages of the sequence are dealt out evenly to all waves of all
 // blocks of a (sequence, kv head); a wave loads a whole page (keys and values) into registers
 // before it computes; several blocks share a compute unit, so one's loads overlap another's
-// arithmetic (keeping a second page in flight per wave cost more in occupancy than it gained).
+// arithmetic.  Where the whole grid fits at two blocks a compute unit, a wave also asks for its
+// next page while it works on this one (AHEAD); with more blocks than that the registers this
+// takes cost more in blocks per unit than the overlap gains.
 // The waves of a block merge their (O, m, l)
 // through shared memory; with several blocks each writes its merged partial to global memory and
 // a second kernel merges the partials in block order.
@@ -399,8 +401,7 @@ struct PageFrags {
 };
 
 template <int HD>
-__device__ __forceinline__ void load_page(const bf16_t* __restrict__ kpage,
-                                          const bf16_t* __restrict__ vpage, PageFrags<HD>& f) {
+__device__ __forceinline__ void load_keys(const bf16_t* __restrict__ kpage, PageFrags<HD>& f) {
   constexpr int KS = (HD + 31) / 32;
   const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
 #pragma unroll
@@ -413,6 +414,11 @@ __device__ __forceinline__ void load_page(const bf16_t* __restrict__ kpage,
       f.k[t4][ks] = (d < HD) ? frag_load(krow + d) : frag_zero();
     }
   }
+}
+
+template <int HD>
+__device__ __forceinline__ void load_values(const bf16_t* __restrict__ vpage, PageFrags<HD>& f) {
+  const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
 #pragma unroll
   for (int dt = 0; dt < HD / 16; ++dt) {
     const bf16_t* vrow = vpage + (size_t)(dt * 16 + r) * PAGE + 8 * g;
@@ -421,14 +427,13 @@ __device__ __forceinline__ void load_page(const bf16_t* __restrict__ kpage,
   }
 }
 
-// Same arithmetic as attn_page, on fragments already loaded.
+// Same arithmetic as attn_page, on fragments already loaded, in two halves: the scores, after
+// which the keys' registers are free for the next page's, and the rest, after which the values' are.
 template <int HD>
-__device__ __forceinline__ void compute_page(const PageFrags<HD>& f, const Frag (&q)[(HD + 31) / 32],
-                                             float scale_log2, int key0, int kmin, int kmax,
-                                             AttnState<HD>& st) {
+__device__ __forceinline__ void page_scores(const PageFrags<HD>& f, const Frag (&q)[(HD + 31) / 32],
+                                            int key0, int kmin, int kmax, f32x4 (&s)[4]) {
   constexpr int KS = (HD + 31) / 32;
   const int lane = threadIdx.x & 63, g = lane >> 4;
-  f32x4 s[4];
 #pragma unroll
   for (int t4 = 0; t4 < 4; ++t4) {
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
@@ -441,6 +446,11 @@ __device__ __forceinline__ void compute_page(const PageFrags<HD>& f, const Frag 
     }
     s[t4] = acc;
   }
+}
+
+template <int HD>
+__device__ __forceinline__ void page_values(const PageFrags<HD>& f, const f32x4 (&s)[4], float scale_log2,
+                                            AttnState<HD>& st) {
   const float mx = max_over_lane_groups(max_of_16(s));
   const float m_new = max2(st.m, mx * scale_log2);
   const float m_safe = (m_new > -INFINITY) ? m_new : 0.f;      // nothing seen yet: every p is 0
@@ -472,7 +482,7 @@ __device__ __forceinline__ void compute_page(const PageFrags<HD>& f, const Frag 
   }
 }
 
-template <int HD, int WAVES>
+template <int HD, int WAVES, bool AHEAD>
 __global__ __launch_bounds__(WAVES * 64, (HD <= 128) ? 2 : 1) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ v_pages, const int* __restrict__ table, int table_stride,
@@ -502,12 +512,31 @@ __global__ __launch_bounds__(WAVES * 64, (HD <= 128) ? 2 : 1) void attn_decode_k
     attn_init<HD>(st);
     const int lo = valid ? kmin : 0x7fffffff, hi = valid ? pos : -1;
     {
+      PageFrags<HD> f;
       for (int pg = p0; pg < p1; ++pg) {
         const size_t base = ((size_t)trow[pg] * n_kv + kvh) * PAGE * HD;
         if (HD <= 128) {
-          PageFrags<HD> f;
-          load_page<HD>(k_pages + base, v_pages + base, f);
-          compute_page<HD>(f, qf, scale_log2, pg * PAGE, lo, hi, st);
+          f32x4 s[4];
+          if (AHEAD) {
+            // The next page's keys are asked for as soon as this page's scores stand, its values
+            // as soon as this page's are used, so that a wave's pages overlap.  The compiler
+            // takes further registers for it (169 instead of 119 at head size 64), which leaves
+            // two blocks a compute unit: the host asks for this when the grid fits in that.
+            if (pg == p0) {
+              load_keys<HD>(k_pages + base, f);
+              load_values<HD>(v_pages + base, f);
+            }
+            const size_t next = (pg + 1 < p1) ? ((size_t)trow[pg + 1] * n_kv + kvh) * PAGE * HD : 0;
+            page_scores<HD>(f, qf, pg * PAGE, lo, hi, s);
+            if (pg + 1 < p1) load_keys<HD>(k_pages + next, f);
+            page_values<HD>(f, s, scale_log2, st);
+            if (pg + 1 < p1) load_values<HD>(v_pages + next, f);
+          } else {
+            load_keys<HD>(k_pages + base, f);
+            load_values<HD>(v_pages + base, f);
+            page_scores<HD>(f, qf, pg * PAGE, lo, hi, s);
+            page_values<HD>(f, s, scale_log2, st);
+          }
         } else {
           attn_page<HD>(k_pages + base, v_pages + base, qf, scale_log2, pg * PAGE, lo, hi, st);
         }
@@ -639,6 +668,19 @@ extern "C" int llm_attention_mfma_supported(int hd) {
   return 0;
 }
 
+static int compute_units() {
+  static int units = 0;                     // of the current device, asked once
+  if (units == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      units = n;
+    else
+      units = 256;
+  }
+  return units;
+}
+
 static bool attn_args_ok(const void* q, int q_stride, const void* k, const void* v, int n_heads,
                          int n_kv, int hd, int window) {
   if (n_heads <= 0 || n_kv <= 0 || n_heads % n_kv || window < 0) return false;
@@ -698,13 +740,21 @@ extern "C" int llm_attention_decode_bf16(const void* q, int q_stride, const void
   if (n_blocks > 1 && (!part_o || !part_ml)) return LLM_ERR_ARG;
   const float scale_log2 = scale * 1.4426950408889634f;
   dim3 grid(n_blocks, n_kv, n_seqs);
+  // pages overlapped within a wave where all blocks are resident at two a compute unit
+  const bool ahead = hd <= 128 && (long long)n_blocks * n_kv * n_seqs <= 2LL * compute_units();
 #define CASE(D)                                                                                   \
   if (hd == D) {                                                                                  \
     constexpr int WAVES = (D > 128) ? 2 : 4;                                                      \
-    attn_decode_kernel<D, WAVES><<<grid, WAVES * 64, 0, stream>>>(                                \
-        (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, table,        \
-        table_stride, seq_slot, seq_pos0, part_o, part_ml, (bf16_t*)out, n_heads, n_kv,           \
-        scale_log2, window);                                                                      \
+    if (ahead)                                                                                    \
+      attn_decode_kernel<D, WAVES, true><<<grid, WAVES * 64, 0, stream>>>(                        \
+          (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, table,      \
+          table_stride, seq_slot, seq_pos0, part_o, part_ml, (bf16_t*)out, n_heads, n_kv,         \
+          scale_log2, window);                                                                    \
+    else                                                                                          \
+      attn_decode_kernel<D, WAVES, false><<<grid, WAVES * 64, 0, stream>>>(                       \
+          (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, table,      \
+          table_stride, seq_slot, seq_pos0, part_o, part_ml, (bf16_t*)out, n_heads, n_kv,         \
+          scale_log2, window);                                                                    \
     if (n_blocks > 1) {                                                                           \
       if (hipGetLastError() != hipSuccess) return LLM_ERR_LAUNCH;                                 \
       const dim3 cgrid(n_heads, n_seqs);                                                          \
