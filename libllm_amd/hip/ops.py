@@ -99,8 +99,8 @@ class HipOps:
     ACCUM_ROWS = 16         # most rows for which a product adds into the stream itself
     SPLIT_ROWS = 64         # beyond those and up to here it goes in slices of K that the next norm adds; then the library's
     DECODE_BLOCKS = 768     # blocks of the decode attention grid beyond which sequences are not split further
-    DECODE_BLOCKS_AHEAD = 512   # the same where a wave would get DECODE_AHEAD_PAGES pages or more: two blocks a
-    DECODE_AHEAD_PAGES = 6      # compute unit, at which the kernel overlaps a wave's pages (head sizes up to 128)
+    DECODE_BLOCKS_AHEAD = 512   # the same where a wave would get DECODE_AHEAD_PAGES pages or more and the sequences
+    DECODE_AHEAD_PAGES = 6      # fill such a grid: two blocks a compute unit, at which the kernel overlaps a wave's pages
     PROMPT_TILE_BLOCKS = (1024, 768)   # blocks of 128 rows from which a wave of prompt attention takes two tiles of rows: heads up to 64 wide, up to 128 (wider ones never: one wave a unit would be left)
     _EPI_NONE, _EPI_SWIGLU, _EPI_ACCUM = 0, 1, 2
 
@@ -540,7 +540,9 @@ class HipOps:
                 # compute unit; the kernel gives every wave ceil(pages / waves) pages in a row, so
                 # blocks beyond ceil(pages / (that * waves)) would get none: they are not launched
                 budget = self.DECODE_BLOCKS
-                if hd <= 128 and pages * m * n_kv >= self.DECODE_AHEAD_PAGES * self.DECODE_BLOCKS_AHEAD * waves:
+                ahead = self.DECODE_BLOCKS_AHEAD // (m * n_kv) * (m * n_kv)      # blocks the smaller grid would have
+                if (hd <= 128 and pages * m * n_kv >= self.DECODE_AHEAD_PAGES * self.DECODE_BLOCKS_AHEAD * waves
+                        and ahead * 16 >= self.DECODE_BLOCKS_AHEAD * 15):
                     budget = self.DECODE_BLOCKS_AHEAD
                 n_blocks = max(1, min(-(-pages // waves), max(1, budget // (m * n_kv))))
                 per_wave = -(-pages // (n_blocks * waves))
