@@ -770,6 +770,29 @@ def test_attention_decode_over_many_pages(ops, ctx_len, far):
     assert max_err(out, ref) < BF16_2ULP
 
 
+@pytest.mark.parametrize("hd", [64, 128])
+@pytest.mark.parametrize("blocks", [1, 3, 4096])
+def test_attention_decode_pages_of_a_wave(ops, monkeypatch, hd, blocks):
+    """With few blocks a wave walks many pages, asking for the next while it works on one (grids
+    of up to two blocks a compute unit); with many sequences and kv heads the grid is larger and
+    the kernel's other form runs.  One far key dominates; a window cuts the walk short."""
+    monkeypatch.setattr(ops, "DECODE_BLOCKS", blocks)
+    monkeypatch.setattr(ops, "DECODE_BLOCKS_AHEAD", min(blocks, 512))
+    for window in (0, 700):
+        out, ref = run_attention(ops, torch.bfloat16, 8, 2, hd, [(0, 2100, 1), (1, 2030, 1)], window=window,
+                                 seed=blocks, boost=(2000, 10.0))
+        assert max_err(out, ref) < BF16_2ULP
+
+
+def test_attention_decode_on_a_large_grid(ops):
+    """More (sequence, kv head) pairs than two blocks a compute unit: the form of the kernel that
+    loads a page, then computes.  Against the oracle."""
+    n_kv, seqs = 16, [(i, 70 + 9 * i, 1) for i in range(40)]
+    assert len(seqs) * n_kv > 512
+    out, ref = run_attention(ops, torch.bfloat16, 16, n_kv, 64, seqs, seed=8)
+    assert max_err(out, ref) < BF16_2ULP
+
+
 def test_attention_single_token_is_value(ops):
     # one query, no past: the output is the value itself
     out, ref = run_attention(ops, torch.float32, 4, 4, 32, [(0, 0, 1)])
