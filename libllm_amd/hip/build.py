@@ -27,9 +27,9 @@ LIB_NAME = "libllm_amd_hip.so"
 # left to itself the compiler keeps them in accumulation registers and moves them out and back
 # for every other instruction that touches them, two moves a value and page in the attention
 # kernels, where instruction issue is what bounds the time.
+OPTIONAL_FLAGS = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]    # left out for a compiler that does not know the switch
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17",
-         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-         "-mllvm", "-amdgpu-mfma-vgpr-form=1"]
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"] + OPTIONAL_FLAGS
 
 _lib: Optional[ctypes.CDLL] = None
 
@@ -112,6 +112,12 @@ def build(force: bool = True, verbose: bool = True) -> str:
         obj = os.path.join(objdir, os.path.basename(src)[:-4] + ".o")
         cmd = [hipcc] + FLAGS + ["-I", CSRC, "-c", src, "-o", obj]
         proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if proc.returncode != 0 and OPTIONAL_FLAGS[-1].split("=")[0].lstrip("-") in proc.stdout:
+            if verbose:
+                _say("  this hipcc does not know %s: compiling %s without it (the attention kernels "
+                     "run somewhat slower)" % (OPTIONAL_FLAGS[-1], os.path.basename(src)))
+            cmd = [hipcc] + FLAGS[:-len(OPTIONAL_FLAGS)] + ["-I", CSRC, "-c", src, "-o", obj]
+            proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         if proc.returncode != 0:
             raise KernelError("hipcc failed on %s:\n%s" % (os.path.basename(src), proc.stdout[-4000:]))
         if verbose:
