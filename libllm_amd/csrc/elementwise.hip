@@ -81,11 +81,11 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_reg_kernel(float* __restrict__
     wv[j] = in ? *reinterpret_cast<const float4*>(w + i) : make_float4(0.f, 0.f, 0.f, 0.f);
     if (d && in) {
       for (int q = 0; q < n_delta; ++q) {                  // several deltas are added in this order
-        const TD* dq = d + q * delta_stride + i;
-        v[j].x += Conv<TD>::load(dq);
-        v[j].y += Conv<TD>::load(dq + 1);
-        v[j].z += Conv<TD>::load(dq + 2);
-        v[j].w += Conv<TD>::load(dq + 3);
+        const float4 dv = Conv4<TD>::load(d + q * delta_stride + i);
+        v[j].x += dv.x;
+        v[j].y += dv.y;
+        v[j].z += dv.z;
+        v[j].w += dv.w;
       }
       *reinterpret_cast<float4*>(x + i) = v[j];
     }
@@ -99,12 +99,9 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_reg_kernel(float* __restrict__
 #pragma unroll
   for (int j = 0; j < NV; ++j) {
     const int i = (threadIdx.x + j * NT) * 4;
-    if (i < H) {
-      Conv<TO>::store(o + i, v[j].x * wv[j].x * inv);
-      Conv<TO>::store(o + i + 1, v[j].y * wv[j].y * inv);
-      Conv<TO>::store(o + i + 2, v[j].z * wv[j].z * inv);
-      Conv<TO>::store(o + i + 3, v[j].w * wv[j].w * inv);
-    }
+    if (i < H)
+      Conv4<TO>::store(o + i, make_float4(v[j].x * wv[j].x * inv, v[j].y * wv[j].y * inv,
+                                          v[j].z * wv[j].z * inv, v[j].w * wv[j].w * inv));
   }
 }
 
@@ -115,7 +112,8 @@ extern "C" int llm_add_rmsnorm(float* res, const void* delta, int delta_dtype, i
   if (n_out <= 0) return LLM_OK;
   if (H <= 0 || (delta != nullptr && n_delta < 1)) return LLM_ERR_ARG;
   constexpr int NT = 256;
-  const bool reg = (H % 4 == 0) && H <= NT * 4 * 4 && ((((uintptr_t)res) | ((uintptr_t)w)) & 15) == 0;
+  const bool reg = (H % 4 == 0) && H <= NT * 4 * 4 && delta_stride % 4 == 0 &&
+                   ((((uintptr_t)res) | ((uintptr_t)w) | ((uintptr_t)delta) | ((uintptr_t)out)) & 15) == 0;
   const bool reg2 = reg && H <= NT * 4 * 2;
 #define LAUNCH(TD, TO) do {                                                                         \
   if (reg2)                                                                                         \
