@@ -152,6 +152,75 @@ def test_first_tokens(models, tmp_path, dtype):
         check(name, cfg, weights, requests, traces.collect(steps, str(out_dir), cfg.vocab), dtype)
 
 
+@pytest.fixture(scope="module")
+def long_models(tmp_path_factory):
+    """The tiny configurations with position limits beyond a thousand, so that one request of a
+    batch can be long while the others are short."""
+    base = tmp_path_factory.mktemp("long_models")
+    out = {}
+    for name, limit in (("A", 1536), ("B", 2304), ("C", 1100)):
+        cfg = dict(CONFIGS[name], max_position_embeddings=limit)
+        path = make_model(base, cfg, seed=5 + len(out), name=name)
+        cfg_json, weights = files.read_model_dir(path)
+        out[name] = (path, llama.PlainConfig(cfg_json), weights)
+    return out
+
+
+EDGE_LENGTHS = [1, 2, 15, 16, 17, 31, 33, 63, 64, 65, 127, 128, 129, 191, 192, 193, 255, 256, 257]
+
+
+def random_trace(rng, cfg):
+    """One to three batches after one another.  A batch has up to 33 requests that start together,
+    lengths drawn around page and tile borders, sometimes one of about a thousand tokens among
+    them.  Half the time the prompts come in chunks of unequal sizes, a chunk for every request
+    that still has prompt left; then one token a step, the shorter requests ending earlier."""
+    steps, requests = [], {}
+    for _ in range(int(rng.integers(1, 4))):
+        group = {}
+        long_one = rng.random() < 0.4
+        for i in range(int(rng.choice([1, 2, 3, 4, 5, 7, 8, 9, 13, 16, 17, 25, 33]))):
+            if long_one and i == 0:
+                n = int(rng.integers(900, cfg.max_pos))
+            elif rng.random() < 0.5:
+                n = int(rng.choice(EDGE_LENGTHS)) + 64 * int(rng.integers(0, 2))
+            else:
+                n = int(rng.integers(1, 300))
+            group["q%d" % (len(requests) + len(group))] = rng.integers(0, cfg.vocab, size=min(n, cfg.max_pos)).tolist()
+        requests.update(group)
+        sub = traces.batches([group], {r: int(rng.integers(0, min(len(t), 40))) for r, t in group.items()})
+        if rng.random() < 0.5:
+            left = {e["id"]: list(e["tokens"]) for e in sub[0]["entries"]}
+            chunks = []
+            while any(left.values()):
+                entries = []
+                for r in left:
+                    if left[r]:
+                        k = int(rng.choice([1, 3, 16, 63, 64, 65, 100, 400]))
+                        entries.append({"id": r, "tokens": left[r][:k], "want": list(range(len(left[r][:k])))})
+                        left[r] = left[r][k:]
+                chunks.append({"entries": entries, "end": []})
+            for r in sub[0]["end"]:                          # a request that is all prompt ends with its last chunk
+                [c for c in chunks if any(e["id"] == r for e in c["entries"])][-1]["end"].append(r)
+            sub = chunks + sub[1:]
+        for s in sub:
+            s["step"] = len(steps)
+            steps.append(s)
+    return steps, requests
+
+
+@pytest.mark.parametrize("case", range(12))
+def test_random_traces(long_models, tmp_path, case):
+    """Drawn batches, cuts and cache sizes (see random_trace) in both dtypes, with and without
+    captured graphs, every position of every request against the plain implementation."""
+    name, dtype, use_graphs = "ABC"[case % 3], DTYPES[(case // 3) % 2], case < 9
+    path, cfg, weights = long_models[name]
+    rng = np.random.default_rng(1000 + case)
+    steps, requests = random_trace(rng, cfg)
+    spare = int(rng.choice([0, 0, 64, 640]))
+    run_replay(path, dtype, steps, tmp_path, max_tokens=traces.max_tokens_needed(steps) + spare, use_graphs=use_graphs)
+    check("long" + name, cfg, weights, requests, traces.collect(steps, str(tmp_path), cfg.vocab), dtype)
+
+
 def _decode_rows(engine, requests, n_last):
     from libllm_amd.engine import StepEntry
     engine.step([StepEntry(r, t[:-n_last], []) for r, t in requests.items()])
