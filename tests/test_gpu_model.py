@@ -221,6 +221,43 @@ def test_random_traces(long_models, tmp_path, case):
     check("long" + name, cfg, weights, requests, traces.collect(steps, str(tmp_path), cfg.vocab), dtype)
 
 
+BENCH_SHAPES = {
+    "1b": dict(hidden_size=2048, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
+               intermediate_size=8192, tie_word_embeddings=True, factor=32.0),
+    "8b": dict(hidden_size=4096, num_attention_heads=32, num_key_value_heads=8, head_dim=128,
+               intermediate_size=14336, tie_word_embeddings=False, factor=8.0),
+}
+
+
+@pytest.mark.parametrize("shape", list(BENCH_SHAPES))
+def test_layers_of_the_measured_shapes(tmp_path, shape):
+    """Two layers of the sizes that the measurements run (a smaller vocabulary, no power of two)
+    against the plain implementation.  The launcher picks the form of a product and of attention
+    by the sizes and by the rows of a step, so the tiny configurations do not reach every form:
+    batches of 1, 8, 20, 48 and 64 decode through each form of the skinny product, the prompts of
+    700 tokens go through the library's products and the two-tile prompt attention."""
+    sh = dict(BENCH_SHAPES[shape])
+    cfg_dict = {"model_type": "llama", "num_hidden_layers": 2, "vocab_size": 8009, "rope_theta": 500000.0,
+                "rope_scaling": {"rope_type": "llama3", "factor": sh.pop("factor"), "low_freq_factor": 1.0,
+                                 "high_freq_factor": 4.0, "original_max_position_embeddings": 8192},
+                "rms_norm_eps": 1e-5, "max_position_embeddings": 4096, "hidden_act": "silu",
+                "eos_token_id": 2, **sh}
+    path = make_model(tmp_path, cfg_dict, seed=3, std=0.02, norm_std=0.1, name=shape)
+    cfg_json, weights = files.read_model_dir(path)
+    cfg = llama.PlainConfig(cfg_json)
+    rng = np.random.default_rng(1)
+    for batch, prompt, decode, dtypes in ((1, 40, 5, DTYPES), (8, 30, 5, DTYPES), (20, 20, 3, DTYPES),
+                                          (48, 10, 3, ["bfloat16"]), (64, 8, 3, DTYPES), (3, 700, 2, ["bfloat16"])):
+        group = {"s%d_%d" % (batch, i): rng.integers(0, cfg.vocab, size=prompt + int(rng.integers(0, 9)) + decode).tolist()
+                 for i in range(batch)}
+        steps = traces.batches([group], {r: decode for r in group})
+        checked = dict(list(group.items())[:3] + list(group.items())[-1:])
+        for dtype in dtypes:
+            out_dir = tmp_path / ("%s_%d_%s" % (shape, batch, dtype))
+            run_replay(path, dtype, steps, out_dir, max_tokens=traces.max_tokens_needed(steps) + 64)
+            check(shape, cfg, weights, checked, traces.collect(steps, str(out_dir), cfg.vocab), dtype)
+
+
 def _decode_rows(engine, requests, n_last):
     from libllm_amd.engine import StepEntry
     engine.step([StepEntry(r, t[:-n_last], []) for r, t in requests.items()])
