@@ -258,6 +258,50 @@ def test_layers_of_the_measured_shapes(tmp_path, shape):
             check(shape, cfg, weights, checked, traces.collect(steps, str(out_dir), cfg.vocab), dtype)
 
 
+ODD = {
+    "width 100, feed-forward 150, vocabulary 101": dict(hidden_size=100, num_attention_heads=5, num_key_value_heads=5,
+                                                        intermediate_size=150, vocab_size=101),
+    "odd width 65, vocabulary 3": dict(hidden_size=65, intermediate_size=91, vocab_size=3),
+    "head size 80": dict(hidden_size=160, num_attention_heads=2, num_key_value_heads=1, head_dim=80),
+    "head size 112": dict(hidden_size=112, num_attention_heads=2, num_key_value_heads=2, head_dim=112),
+    "head size 256": dict(hidden_size=256, num_attention_heads=2, num_key_value_heads=1, head_dim=256),
+    "head size 24": dict(hidden_size=96, num_attention_heads=4, num_key_value_heads=2, head_dim=24),
+    "seven heads, seven kv heads": dict(hidden_size=112, num_attention_heads=7, num_key_value_heads=7),
+    "a group of 20 heads": dict(hidden_size=80, num_attention_heads=20, num_key_value_heads=1),
+    "a group of 40 heads": dict(hidden_size=80, num_attention_heads=40, num_key_value_heads=1, head_dim=32),
+    "one layer, one head": dict(num_hidden_layers=1, hidden_size=16, num_attention_heads=1, num_key_value_heads=1,
+                                intermediate_size=8, vocab_size=9),
+    "feed-forward of one, vocabulary 70001": dict(intermediate_size=1, vocab_size=70001),
+}
+
+
+@pytest.mark.parametrize("what", list(ODD))
+def test_odd_sizes_end_to_end(tmp_path, what):
+    """Sizes that a configuration may have and no released model has, through the whole engine in
+    both dtypes: a batch of up to 18 unequal prompts, then six tokens each."""
+    cfg_dict = dict(TINY_A, max_position_embeddings=512, **ODD[what])
+    path = make_model(tmp_path, cfg_dict, seed=len(what), name="odd")
+    cfg_json, weights = files.read_model_dir(path)
+    cfg = llama.PlainConfig(cfg_json)
+    lengths = [70, 9, 131, 20, 1, 64, 33, 200, 5, 17, 90, 40, 3, 66, 128, 12, 7, 100]
+    requests = make_requests(cfg, lengths[:18 if len(what) % 2 else 5], seed=len(what))
+    steps = traces.batches([requests], {r: min(6, len(t) - 1) for r, t in requests.items()})
+    for dtype in DTYPES:
+        out_dir = tmp_path / dtype
+        run_replay(path, dtype, steps, out_dir)
+        check(what, cfg, weights, requests, traces.collect(steps, str(out_dir), cfg.vocab), dtype)
+
+
+def test_a_head_size_beyond_the_kernels_is_refused(tmp_path):
+    from libllm_amd.errors import KernelError
+    from libllm_amd.engine import StepEntry
+    from libllm_amd.runtime import load_engine
+    path = make_model(tmp_path, dict(TINY_A, hidden_size=272, num_attention_heads=1, num_key_value_heads=1,
+                                     head_dim=272), seed=1, name="wide_head")
+    with pytest.raises(KernelError, match="head_dim 272"):
+        load_engine(path, dtype="bfloat16", max_tokens=64).step([StepEntry("a", [1, 2, 3], [2])])
+
+
 def _decode_rows(engine, requests, n_last):
     from libllm_amd.engine import StepEntry
     engine.step([StepEntry(r, t[:-n_last], []) for r, t in requests.items()])
