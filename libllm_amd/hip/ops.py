@@ -101,7 +101,14 @@ class HipOps:
     DECODE_BLOCKS = 768     # blocks of the decode attention grid beyond which sequences are not split further
     DECODE_BLOCKS_AHEAD = 512   # the same where a wave would get DECODE_AHEAD_PAGES pages or more and the sequences
     DECODE_AHEAD_PAGES = 6      # fill such a grid: two blocks a compute unit, at which the kernel overlaps a wave's pages
-    PROMPT_TILE_BLOCKS = (1024, 768)   # blocks of 128 rows from which a wave of prompt attention takes two tiles of rows: heads up to 64 wide, up to 128 (wider ones never: one wave a unit would be left)
+    # New rows of the step's longest sequence from which a wave of prompt attention takes two
+    # tiles of rows: heads up to 64 wide, up to 128 (wider ones never: one wave a unit would be
+    # left).  A block's walk over the pages of its rows is what a short prompt waits for, and two
+    # tiles make every walk longer; from here on the pages staged half as often outweigh that
+    # (head size 64: 67.3 against 68.6 us at 3,072 rows, 109.4 against 104.0 at 4,096; head size
+    # 128: 59.7 against 64.2 at 2,048, 124.9 against 108.1 at 3,072).  More sequences of the same
+    # lengths do not move the crossing (4 x 1,024 rows: 39.1 against 43.0).
+    PROMPT_TILE_ROWS = (3584, 2560)
     _EPI_NONE, _EPI_SWIGLU, _EPI_ACCUM = 0, 1, 2
 
     def __init__(self, device: Optional[str] = None):
@@ -557,8 +564,7 @@ class HipOps:
             else:
                 tiles = self.prompt_tiles
                 if not tiles:
-                    blocks = -(-ctx.max_new // 128) * n_heads * ctx.n_seqs
-                    tiles = 2 if hd <= 128 and blocks >= self.PROMPT_TILE_BLOCKS[0 if hd <= 64 else 1] else 1
+                    tiles = 2 if hd <= 128 and ctx.max_new >= self.PROMPT_TILE_ROWS[0 if hd <= 64 else 1] else 1
                 self._check(self.lib.llm_attention_prefill_bf16(
                     qkv.data_ptr(), width, kv.k_pages.data_ptr(), kv.v_pages.data_ptr(),
                     table.data_ptr(), table.shape[1], 64, ctx.seq_start.data_ptr(),

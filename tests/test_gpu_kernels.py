@@ -739,12 +739,12 @@ def test_prompt_attention_tiles_of_rows(ops, hd, window, tiles):
     assert max_err(out, ref) < BF16_2ULP
 
 
-def test_prompt_attention_takes_two_tiles_when_blocks_are_many(ops):
-    """Left to itself the launcher takes two tiles a wave from 1,024 blocks of 128 rows on; a row's
-    bits do not depend on it."""
-    n_heads, n_kv, hd, rows = 32, 8, 64, 2048
-    seqs = [(0, 0, rows), (1, 64, rows - 100)]
-    assert -(-rows // 128) * n_heads * len(seqs) >= ops.PROMPT_TILE_BLOCKS[0]
+def test_prompt_attention_takes_two_tiles_for_long_prompts(ops):
+    """Left to itself the launcher takes two tiles a wave where the longest sequence brings 3,584
+    rows or more (head size 64); a row's bits do not depend on it."""
+    n_heads, n_kv, hd, rows = 32, 8, 64, 3600
+    seqs = [(0, 0, rows), (1, 64, 500)]
+    assert rows >= ops.PROMPT_TILE_ROWS[0]
     ctx = make_ctx(ops, torch.bfloat16, seqs)
     kv = make_kv("cuda", torch.bfloat16, 2, (rows + 64) // PAGE + 1, n_kv, hd, seed=2)
     kv.k_pages.normal_(); kv.v_pages.normal_()

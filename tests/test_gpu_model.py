@@ -235,7 +235,7 @@ def test_layers_of_the_measured_shapes(tmp_path, shape):
     against the plain implementation.  The launcher picks the form of a product and of attention
     by the sizes and by the rows of a step, so the tiny configurations do not reach every form:
     batches of 1, 8, 20, 48 and 64 decode through each form of the skinny product, the prompts of
-    700 tokens go through the library's products and the two-tile prompt attention."""
+    700 tokens go through the library's products."""
     sh = dict(BENCH_SHAPES[shape])
     cfg_dict = {"model_type": "llama", "num_hidden_layers": 2, "vocab_size": 8009, "rope_theta": 500000.0,
                 "rope_scaling": {"rope_type": "llama3", "factor": sh.pop("factor"), "low_freq_factor": 1.0,
