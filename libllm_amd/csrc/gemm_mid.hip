@@ -1,0 +1,278 @@
+// C[M,N] = X[M,K] * W[N,K]^T for 65 to 128 rows: still bound by the one pass over W, but with too
+// many rows for a block to stage all of them per 16 rows of W, as the product for few rows does.
+// bfloat16 inputs, float32 accumulation on the matrix cores.
+//
+// A block of 4 waves owns 64 rows of W over all of K or one slice of it: two pairs of waves with
+// two tiles of 16 rows each (what a wave reads of X from shared memory serves both tiles; that
+// traffic is what bounds this kernel), the first wave of a pair taking the first two steps (of
+// 32 elements) of every chunk of 128, the second the other two.  W is the copy tiled for the
+// matrix cores (llm_pack_weight): a wave's fragment of a step is 1 KiB in a row, and goes from
+// global memory straight to registers, five chunks ahead.  The rows of X go through shared
+// memory, a chunk at a time, in two buffers filled in turns (one barrier a chunk), and four
+// more waves do nothing but that: a wave's loads complete in the order they were asked for, so a
+// wave that waited for the rows of the next chunk would wait for every fragment of W asked for
+// before them (with every wave doing both, a chunk took 1.9 us instead of 1.5).  The four waves
+// that compute read the rows as B operands, so
+// lane l ends with
+// C[m = 16 mt + l % 16][n = 4 (l / 16) + e] for the 16 rows n of a tile of W.  The two waves of a
+// pair add their sums through shared memory, first wave first: a row's bits do not depend on the
+// other rows.
+//
+// Epilogues: plain store as bfloat16; with slices of K (grid height > 1), float32 matrices
+// [slice, M, N] that the caller adds in order; or SwiGLU over a stacked [gate; up] weight
+// (src/flint/cuda/swiglu.cu:44-49): a wave's two tiles are a gate tile and the up tile of the
+// same columns, gate and up rounded to bfloat16 first, as the unfused path stores them.
+#include "mfma.h"
+
+#define MID_EPI_NONE 0
+#define MID_EPI_SWIGLU 1
+#define MID_CK 128          // elements of K per chunk
+#define MID_STEPS 4         // steps of 32 per chunk
+#define MID_STAGES 6        // chunks of W in registers
+#define MID_WK 2            // waves that share a tile of W, splitting each chunk's steps
+#define MID_NT 512          // threads of a block: four waves that compute, four that stage X
+#define MID_RT 2            // tiles of W a wave owns
+
+template <int MT, int EPI, typename OutT>
+__global__ __launch_bounds__(MID_NT) void gemm_mid_kernel(const bf16_t* __restrict__ X,
+                                                             const bf16_t* __restrict__ W,
+                                                             OutT* __restrict__ C, int M, int N, int K,
+                                                             int ldx, int w_steps, int n_out) {
+  constexpr int ROW_B = MID_CK * 2;                  // bytes of a staged row: 16 pieces of 16 bytes, swizzled
+  constexpr int BUF = 16 * MT * ROW_B;
+  constexpr int PASSES = MT;                         // 256 threads carry 16 rows a pass
+  constexpr int US = MID_STEPS / MID_WK;             // steps of a chunk that a wave takes
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2 * BUF];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int wn = wave >> 1, wk = wave & 1;
+  const int r = lane & 15, g = lane >> 4;
+  const int k0 = blockIdx.y * K;                     // this block's slice of K (K elements, a multiple of 32 if sliced)
+  X += k0;
+  const int n_chunks = K / MID_CK;                   // K is a multiple of the chunk
+
+  // first rows of W of this wave's tiles
+  int tile_row[MID_RT];
+  const bf16_t* wp[MID_RT];
+#pragma unroll
+  for (int rt = 0; rt < MID_RT; ++rt) {
+    if (EPI == MID_EPI_SWIGLU)
+      tile_row[rt] = rt * n_out + (blockIdx.x * 2 + wn) * 16;
+    else
+      tile_row[rt] = ((blockIdx.x * 2 + wn) * MID_RT + rt) * 16;
+    int t = tile_row[rt] / 16;
+    if (t > (N - 1) / 16) t = (N - 1) / 16;          // tiles past the end read the last one; not stored
+    wp[rt] = W + ((size_t)t * w_steps * 64 + lane) * 8 + (size_t)(k0 / 32) * 512;
+  }
+
+  f32x4 acc[MID_RT][MT];
+#pragma unroll
+  for (int rt = 0; rt < MID_RT; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[rt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  float* ex = reinterpret_cast<float*>(lds);
+  if (wave >= 4) {
+    // ---- the waves that stage X: chunk c + 1 goes to its buffer while chunk c is computed on; the
+    // loads are asked for two chunks before.  A row's 16 pieces are stored at piece ^ (row % 16):
+    // the 16 lanes of a read, one row each, then fall into 16 different groups of banks.
+    const int t2 = tid - 256, x_col = t2 & 15, x_row0 = t2 >> 4;
+    uint4 xr[2][PASSES];
+    // (Rows past M and chunks past the end are zeros.  Loads without a condition, rows and chunks
+    // clamped instead, let the compiler count the loads in flight and wait for fewer: measured
+    // twice as slow, 60 against 25 us at 128 x 2,048 x 16,384.)
+    const int last = n_chunks - 1;
+    auto load_x = [&](int chunk, uint4 (&dst)[PASSES]) {
+      const int k = chunk * MID_CK + x_col * 8;
+#pragma unroll
+      for (int p = 0; p < PASSES; ++p) {
+        const int row = x_row0 + p * 16;
+        dst[p] = (row < M && chunk <= last) ? *reinterpret_cast<const uint4*>(X + (size_t)row * ldx + k)
+                                            : make_uint4(0u, 0u, 0u, 0u);
+      }
+    };
+    auto store_x = [&](int buf, uint4 (&src)[PASSES]) {
+#pragma unroll
+      for (int p = 0; p < PASSES; ++p) {
+        const int row = x_row0 + p * 16;
+        *reinterpret_cast<uint4*>(lds + buf * BUF + row * ROW_B + ((x_col ^ (row & 15)) * 16)) = src[p];
+      }
+    };
+    load_x(0, xr[0]);
+    load_x(1, xr[1]);
+    store_x(0, xr[0]);
+    load_x(2, xr[0]);
+#define MID_STAGE(C, CUR)                  \
+  __syncthreads();                         \
+  store_x(((C) + 1) & 1, CUR);             \
+  load_x((C) + 3, CUR);                    \
+  if ((C) + 1 >= n_chunks) break;
+    for (int c = 0;; c += 2) {
+      MID_STAGE(c, xr[1])
+      MID_STAGE(c + 1, xr[0])
+    }
+#undef MID_STAGE
+    __syncthreads();
+    __syncthreads();
+    return;
+  }
+
+  Frag a[MID_STAGES][US][MID_RT];
+  const int last = n_chunks - 1;
+  auto load_w = [&](int chunk, Frag (&dst)[US][MID_RT]) {
+    const int s0 = chunk * MID_STEPS + wk * US;
+#pragma unroll
+    for (int u = 0; u < US; ++u)
+#pragma unroll
+      for (int rt = 0; rt < MID_RT; ++rt)
+        dst[u][rt] = chunk <= last ? frag_load(wp[rt] + (size_t)(s0 + u) * 512) : frag_zero();
+  };
+  auto compute = [&](int buf, Frag (&src)[US][MID_RT]) {
+#pragma unroll
+    for (int u = 0; u < US; ++u) {
+      const int piece = (wk * US + u) * 4 + g;
+      Frag b[MT];                                      // all of a step's reads before its matrix instructions
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        b[mt].u = *reinterpret_cast<const uint4*>(lds + buf * BUF + (mt * 16 + r) * ROW_B + ((piece ^ r) * 16));
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+#pragma unroll
+        for (int rt = 0; rt < MID_RT; ++rt) acc[rt][mt] = mfma_bf16(src[u][rt], b[mt], acc[rt][mt]);
+    }
+  };
+
+#pragma unroll
+  for (int c = 0; c < MID_STAGES - 1; ++c) load_w(c, a[c]);
+  // iteration c: chunk c of X lies in buffer c % 2
+#define MID_STEP(C, CUR, NXT)                 \
+  __syncthreads();                            \
+  load_w((C) + MID_STAGES - 1, NXT);          \
+  compute((C) & 1, CUR);                      \
+  if ((C) + 1 >= n_chunks) break;
+  for (int c = 0;; c += 6) {
+    MID_STEP(c, a[0], a[5])
+    MID_STEP(c + 1, a[1], a[0])
+    MID_STEP(c + 2, a[2], a[1])
+    MID_STEP(c + 3, a[3], a[2])
+    MID_STEP(c + 4, a[4], a[3])
+    MID_STEP(c + 5, a[5], a[4])
+  }
+#undef MID_STEP
+
+  // ---- the second wave of a pair hands its sums to the first through shared memory
+  __syncthreads();                                     // every wave is done with the staged rows
+  if (wk == 1) {
+#pragma unroll
+    for (int rt = 0; rt < MID_RT; ++rt)
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt)
+        *reinterpret_cast<float4*>(ex + (((wn * MID_RT + rt) * MT + mt) * 64 + lane) * 4) =
+            make_float4(acc[rt][mt][0], acc[rt][mt][1], acc[rt][mt][2], acc[rt][mt][3]);
+  }
+  __syncthreads();
+  if (wk == 1) return;
+#pragma unroll
+  for (int rt = 0; rt < MID_RT; ++rt)
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const float4 v = *reinterpret_cast<const float4*>(ex + (((wn * MID_RT + rt) * MT + mt) * 64 + lane) * 4);
+      acc[rt][mt] += f32x4{v.x, v.y, v.z, v.w};
+    }
+
+  if (EPI == MID_EPI_SWIGLU) {
+    const int n = tile_row[0] + 4 * g;                 // output column: the gate tile's rows
+    if (n >= n_out) return;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = mt * 16 + r;
+      if (m >= M) continue;
+      float v[4];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const float gt = bf16_to_f32(f32_to_bf16(acc[0][mt][e])), u = bf16_to_f32(f32_to_bf16(acc[1][mt][e]));
+        v[e] = u * gt / (1.0f + expf(-gt));
+      }
+      uint2 pk;
+      pk.x = pack2_bf16(v[0], v[1]);
+      pk.y = pack2_bf16(v[2], v[3]);
+      *reinterpret_cast<uint2*>(C + (size_t)m * n_out + n) = pk;       // n_out is a multiple of 16
+    }
+    return;
+  }
+
+#pragma unroll
+  for (int rt = 0; rt < MID_RT; ++rt) {
+    const int n = tile_row[rt] + 4 * g;
+    if (n >= N) continue;
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) {
+      const int m = mt * 16 + r;
+      if (m >= M) continue;
+      const f32x4 sum = acc[rt][mt];
+      OutT* dst = C + ((size_t)blockIdx.y * M + m) * N + n;
+      if (n + 3 < N && (N & 3) == 0) {
+        if (sizeof(OutT) == 2) {
+          uint2 pk;
+          pk.x = pack2_bf16(sum[0], sum[1]);
+          pk.y = pack2_bf16(sum[2], sum[3]);
+          *reinterpret_cast<uint2*>(dst) = pk;
+        } else {
+          *reinterpret_cast<float4*>(dst) = make_float4(sum[0], sum[1], sum[2], sum[3]);
+        }
+      } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (n + e < N) Conv<OutT>::store(dst + e, sum[e]);
+      }
+    }
+  }
+}
+
+template <int EPI, typename OutT>
+static int launch_mid(const bf16_t* X, const bf16_t* W, void* C, int M, int N, int K, int ldx,
+                      int k_split, hipStream_t stream) {
+  const int n_out = (EPI == MID_EPI_SWIGLU) ? N / 2 : N;
+  const int per_block = (EPI == MID_EPI_SWIGLU) ? 32 : 64;
+  const dim3 grid((n_out + per_block - 1) / per_block, k_split);
+  const int w_steps = (K + 31) / 32;
+#define MID_CASE(T)                                                                                  \
+  case T:                                                                                            \
+    gemm_mid_kernel<T, EPI, OutT><<<grid, MID_NT, 0, stream>>>(X, W, (OutT*)C, M, N, K / k_split, ldx,  \
+                                                            w_steps, n_out);                         \
+    break;
+  switch ((M + 15) / 16) {
+    MID_CASE(5)
+    MID_CASE(6)
+    MID_CASE(7)
+    MID_CASE(8)
+    default: return LLM_ERR_ARG;
+  }
+#undef MID_CASE
+  return llm_launch_status();
+}
+
+// X [M, K] bfloat16 with rows ldx apart, 65 <= M <= 128; W the tiled copy of a [N, K] matrix.
+// epilogue 0: C [M, N] bfloat16, or with k_split > 1 float32 [k_split, M, N], the products over
+// the slices of K; K is a multiple of 128 * k_split; epilogue 1: C [M, N/2] bfloat16, SwiGLU over
+// W = [Wg; Wu], N/2 a multiple of 16.
+extern "C" int llm_gemm_mid_bf16(const void* X, int ldx, const void* W_tiled, void* C, int epilogue,
+                                 int out_dtype, int M, int N, int K, int k_split, hipStream_t stream) {
+  if (M < 65 || M > 128 || N <= 0 || K <= 0 || (K & 7) || ldx < K || (ldx & 7) || k_split < 1)
+    return LLM_ERR_ARG;
+  if (X == nullptr || W_tiled == nullptr || C == nullptr) return LLM_ERR_ARG;
+  if ((((uintptr_t)X) | ((uintptr_t)W_tiled) | ((uintptr_t)C)) & 15) return LLM_ERR_ARG;
+  if (k_split > 65535 || K % (k_split * MID_CK) != 0) return LLM_ERR_ARG;
+  if (epilogue == MID_EPI_NONE) {
+    if (k_split == 1 && out_dtype == LLM_DTYPE_BF16)
+      return launch_mid<MID_EPI_NONE, bf16_t>((const bf16_t*)X, (const bf16_t*)W_tiled, C, M, N, K, ldx, 1, stream);
+    if (out_dtype == LLM_DTYPE_F32)
+      return launch_mid<MID_EPI_NONE, float>((const bf16_t*)X, (const bf16_t*)W_tiled, C, M, N, K, ldx, k_split, stream);
+    return LLM_ERR_ARG;
+  }
+  if (epilogue == MID_EPI_SWIGLU) {
+    if ((N & 31) || out_dtype != LLM_DTYPE_BF16 || k_split != 1) return LLM_ERR_ARG;
+    return launch_mid<MID_EPI_SWIGLU, bf16_t>((const bf16_t*)X, (const bf16_t*)W_tiled, C, M, N, K, ldx, 1, stream);
+  }
+  return LLM_ERR_ARG;
+}

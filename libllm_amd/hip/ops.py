@@ -43,6 +43,7 @@ _SIGNATURES = {
     "llm_attention_ref": [_vp, _i, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i, _i,
                           _f, _i, _vp],
     "llm_gemm_skinny_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
+    "llm_gemm_mid_bf16": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
     "llm_gemm_skinny_norm_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _f, _vp],
     "llm_attention_mfma_supported": [_i],
     "llm_attention_prefill_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i,
@@ -98,6 +99,15 @@ class HipOps:
     SKINNY_ROWS = 64        # most rows the streaming matrix product takes at once; beyond, the library's
     ACCUM_ROWS = 16         # most rows for which a product adds into the stream itself
     SPLIT_ROWS = 64         # beyond those and up to here it goes in slices of K that the next norm adds; then the library's
+    # 65 to MID_ROWS rows: a streaming product of their own for weights with a tiled copy; beyond,
+    # the library's.  Whole engines compared in one process, prompt steps of 65 to 128 tokens: 3.54
+    # against 4.17 ms at the 3B shape, 6.19 against 7.01 at 8B; decode batches of 96: 3.92 against
+    # 5.25 and 6.25 against 7.05.  At the 1B shape the library's products for the two small
+    # weights and for gate/up at 128 rows are as fast or 1 % faster: hence the two limits below.
+    MID_ROWS = 128
+    MID_MIN_WEIGHT = 3072 * 3072    # elements of a weight from which a product that adds into the stream takes it (in slices of K)
+    MID_SWIGLU_K = 3072             # width from which gate/up takes it at more than MID_SWIGLU_ROWS rows
+    MID_SWIGLU_ROWS = 96
     DECODE_BLOCKS = 768     # blocks of the decode attention grid beyond which sequences are not split further
     DECODE_BLOCKS_AHEAD = 512   # the same where a wave would get DECODE_AHEAD_PAGES pages or more and the sequences
     DECODE_AHEAD_PAGES = 6      # fill such a grid: two blocks a compute unit, at which the kernel overlaps a wave's pages
@@ -130,6 +140,7 @@ class HipOps:
         self.fast_attention = True      # bfloat16 attention on the matrix cores (else the plain kernel, as for float32)
         self.pack_weights = True        # keep a tiled copy of every weight for the skinny product
         self.fast_gemm = True           # the skinny product for few rows (else the library's for every product)
+        self.mid_gemm = True            # the product for 65 to 128 rows (else the library's)
         self.fold_norms = True          # up to ACCUM_ROWS rows, a norm between two products gets no kernel of its own
         self.prompt_tiles = 0           # tiles of rows a wave of prompt attention takes (1 or 2; 0: by the number of blocks)
 
@@ -293,6 +304,29 @@ class HipOps:
             ks -= 1
         return ks
 
+    def _mid_ok(self, x, w, m, k):
+        return (self.fast_gemm and self.mid_gemm and isinstance(w, PreparedWeight)
+                and self.SKINNY_ROWS < m <= self.MID_ROWS and not isinstance(x, NormedRows)
+                and x.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1 and x.stride(0) >= k
+                and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and k % 128 == 0)
+
+    @staticmethod
+    def _k_split_mid(n, k):
+        """Slices of K for a product of 65 to 128 rows whose result the next norm adds: enough for
+        about a block a compute unit at 64 weight rows a block, each at least 256 long and a
+        multiple of 128."""
+        ks = max(1, min(16, 256 // max(1, -(-n // 64))))
+        while ks > 1 and (k % (ks * 128) or k // ks < 256):
+            ks -= 1
+        return ks
+
+    def _mid(self, x, w, out, epilogue, k_split=1):
+        n, k = w.shape
+        self._check(self.lib.llm_gemm_mid_bf16(
+            x.data_ptr(), x.stride(0), w.tiled.data_ptr(), out.data_ptr(), epilogue, _code(out.dtype),
+            x.shape[0], n, k, k_split, self._stream()), "gemm_mid_bf16")
+        return out
+
     def _skinny(self, x, w, out, epilogue, m0=0, mm=None, k_split=1):
         """Launches the skinny kernel on rows m0 .. m0+mm of the bfloat16 matrix x; with ``k_split``
         the products over that many slices of K go to ``out[k_split, mm, n]``."""
@@ -364,6 +398,14 @@ class HipOps:
             x = self._materialise(x, torch.float32 if w.dtype == torch.float32 else torch.bfloat16)
             if self._skinny_ok(x, w, m, k) and bias is None:
                 return self.linear(x, w, None, out_dtype, residual)
+        if self._mid_ok(x, w, m, k) and bias is None and out_dtype != torch.float32:
+            # (without slices of K, for a product that does not add into the stream, it has too few
+            # blocks for the q|k|v weights and loses to the library: 16.7 against 13.0 us at 128 rows)
+            if residual is not None and n * k >= self.MID_MIN_WEIGHT:
+                # K in slices for enough blocks; the norm kernel that follows adds them, in order
+                ks = self._k_split_mid(n, k)
+                return self._mid(x, w, torch.empty((ks, m, n), dtype=torch.float32, device=self.device),
+                                 self._EPI_NONE, ks)
         w = self._plain(w)
         if w.dtype == torch.float32:
             if w.stride(0) != k:
@@ -406,6 +448,11 @@ class HipOps:
                 raise KernelError("linear_swiglu: a normed record needs the activation dtype")
             x = self._materialise(x, dtype)
             return self.linear_swiglu(x, w, dtype)
+        if (self._mid_ok(x, w, m, k) and inter % 16 == 0 and dtype == torch.bfloat16
+                and (m <= self.MID_SWIGLU_ROWS or k >= self.MID_SWIGLU_K)):
+            self._weight(self._plain(w), "linear weight")
+            return self._mid(x, w, torch.empty((m, inter), dtype=torch.bfloat16, device=self.device),
+                             self._EPI_SWIGLU)
         return self.silu_mul(self.linear(x, w, None, x.dtype))
 
     def silu_mul(self, gu):

@@ -412,6 +412,72 @@ def test_products_in_slices_of_k(ops, monkeypatch, m, nk):
         ops._skinny(x, w, plain, ops._EPI_NONE, 0, m, k_split=7)
 
 
+# ---------------------------------------------------------------- the product for 65 to 128 rows
+@pytest.mark.parametrize("m", [65, 80, 97, 128])
+@pytest.mark.parametrize("nk", [(64, 128), (48, 256), (1000, 640), (3072, 3072), (2048, 8192)])
+def test_gemm_mid(ops, m, nk):
+    """Plain as bfloat16, and in slices of K as float32 matrices, against float64; weights whose
+    rows are no multiple of 64 or of 16, one chunk of K and many."""
+    n, k = nk
+    x = rnd((m, k), torch.bfloat16, 3).cuda()
+    w = ops.prepare_weight(rnd((n, k), torch.bfloat16, 4, scale=0.05).cuda())
+    ref = x.double() @ w.w.double().t()
+    out = ops._mid(x, w, torch.empty((m, n), dtype=torch.bfloat16, device="cuda"), ops._EPI_NONE)
+    assert close(out, ref, torch.bfloat16)
+    for ks in sorted({1, 2 if (k // 128) % 2 == 0 else 1, k // 128}):
+        parts = ops._mid(x, w, torch.empty((ks, m, n), dtype=torch.float32, device="cuda"), ops._EPI_NONE, ks)
+        total = parts[0].clone()
+        for j in range(1, ks):
+            total += parts[j]
+        assert close(total, ref, torch.float32)
+
+
+@pytest.mark.parametrize("m", [66, 128])
+@pytest.mark.parametrize("ik", [(32, 128), (208, 384), (8192, 2048)])
+def test_gemm_mid_swiglu(ops, m, ik):
+    """silu(gate) * up over a stacked weight, gate and up rounded to bfloat16 first as the
+    unfused path stores them: the same bits as the library's product and the SiLU-mul kernel
+    give wherever the two products agree on every rounded gate and up, close everywhere."""
+    inter, k = ik
+    x = rnd((m, k), torch.bfloat16, 5).cuda()
+    w = ops.prepare_weight(rnd((2 * inter, k), torch.bfloat16, 6, scale=0.05).cuda())
+    out = ops._mid(x, w, torch.empty((m, inter), dtype=torch.bfloat16, device="cuda"), ops._EPI_SWIGLU)
+    gu = (x.double() @ w.w.double().t()).bfloat16().double()
+    g, u = gu[:, :inter], gu[:, inter:]
+    ref = u * g / (1 + torch.exp(-g))
+    err = ((out.double() - ref).abs() / (ref.abs() + ref.abs().mean())).max().item()
+    assert err < 0.02, err
+
+
+def test_gemm_mid_rows_do_not_depend_on_the_batch(ops):
+    """A row's sums are added along K by the same two waves in the same order whatever the other
+    rows are: the same bits at 65, 100 and 128 rows, and with the row at another place."""
+    n, k = 1024, 1024
+    x = rnd((128, k), torch.bfloat16, 7).cuda()
+    w = ops.prepare_weight(rnd((n, k), torch.bfloat16, 8, scale=0.05).cuda())
+    full = ops._mid(x, w, torch.empty((128, n), dtype=torch.bfloat16, device="cuda"), ops._EPI_NONE)
+    for m in (65, 100):
+        part = ops._mid(x[:m].contiguous(), w, torch.empty((m, n), dtype=torch.bfloat16, device="cuda"), ops._EPI_NONE)
+        assert torch.equal(part, full[:m])
+    moved = torch.cat([x[64:], x[:64]]).contiguous()
+    out = ops._mid(moved, w, torch.empty((128, n), dtype=torch.bfloat16, device="cuda"), ops._EPI_NONE)
+    assert torch.equal(out[:64], full[64:]) and torch.equal(out[64:], full[:64])
+
+
+def test_gemm_mid_refuses(ops):
+    from libllm_amd.errors import KernelError
+    w = ops.prepare_weight(rnd((64, 256), torch.bfloat16, 1).cuda())
+    x = rnd((128, 256), torch.bfloat16, 2).cuda()
+    for rows, ks in ((64, 1), (129, 1), (100, 3)):                     # too few rows, too many, slices that do not divide K
+        with pytest.raises(KernelError):
+            xs = torch.cat([x, x])[:rows].contiguous()
+            ops._mid(xs, w, torch.empty((ks, rows, 64), dtype=torch.float32, device="cuda"), ops._EPI_NONE, ks)
+    w2 = ops.prepare_weight(rnd((64, 200), torch.bfloat16, 1).cuda())    # K no multiple of the chunk
+    assert not ops._mid_ok(rnd((100, 200), torch.bfloat16, 2).cuda(), w2, 100, 200)
+    with pytest.raises(KernelError):
+        ops._mid(rnd((100, 200), torch.bfloat16, 2).cuda(), w2, torch.empty((100, 64), dtype=torch.bfloat16, device="cuda"), ops._EPI_NONE)
+
+
 def test_large_bf16_product(ops):
     x = rnd((300, 256), torch.bfloat16, 3).cuda()
     w = rnd((520, 256), torch.bfloat16, 4).cuda()

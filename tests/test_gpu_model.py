@@ -549,12 +549,14 @@ def test_library_products_inside_prompt_graphs(rows):
     assert list(engines[0]._prompt_graphs) == [(rows, 2)] and not engines[1]._prompt_graphs
 
 
+@pytest.mark.parametrize("n_prompts", [40, 96])
 @pytest.mark.parametrize("widths", [(2048, 32, 64, 8192), (4096, 32, 128, 14336)])
-def test_decode_graphs_of_many_rows(widths):
+def test_decode_graphs_of_many_rows(widths, n_prompts):
     """From 17 rows on the products that add into the stream are computed over slices of K, which
-    the next norm kernel adds.  Layers of real width: a graph of 48 rows replayed twelve times, an
-    engine without graphs stepping beside it, other work and a synchronisation between the
-    replays; every replay gives the bits of the eager step."""
+    the next norm kernel adds; from 65 rows on by the product for 65 to 128 rows, or the
+    library's.  Layers of real width: a graph of 48 or 96 rows replayed twelve times, an engine
+    without graphs stepping beside it, other work and a synchronisation between the replays;
+    every replay gives the bits of the eager step."""
     import torch
     from libllm_amd.config import config_from_dict
     from libllm_amd.engine import StepEntry
@@ -566,9 +568,10 @@ def test_decode_graphs_of_many_rows(widths):
         "rope_theta": 500000.0, "rms_norm_eps": 1e-5, "tie_word_embeddings": True,
         "max_position_embeddings": 4096, "hidden_act": "silu", "bos_token_id": 1, "eos_token_id": 2})
     rng = np.random.default_rng(3)
-    prompts = {i: rng.integers(3, 4096, size=int(n)).tolist() for i, n in enumerate(rng.integers(3, 40, size=40))}
-    engines = [random_engine(cfg, seed=5, dtype="bfloat16", max_tokens=8192, use_graphs=g) for g in (True, False)]
-    assert engines[0].ops.ACCUM_ROWS < 40 <= engines[0].ops.SPLIT_ROWS
+    prompts = {i: rng.integers(3, 4096, size=int(n)).tolist() for i, n in enumerate(rng.integers(3, 40, size=n_prompts))}
+    engines = [random_engine(cfg, seed=5, dtype="bfloat16", max_tokens=16384, use_graphs=g) for g in (True, False)]
+    ops = engines[0].ops
+    assert ops.ACCUM_ROWS < 40 <= ops.SPLIT_ROWS < 96 <= ops.MID_ROWS and ops.mid_gemm
     for e in engines:
         e.step([StepEntry(r, t, []) for r, t in prompts.items()])
     scratch = torch.randn((512, 512), device="cuda")
@@ -580,7 +583,7 @@ def test_decode_graphs_of_many_rows(widths):
             scratch = (scratch @ scratch).clamp_(-1, 1)         # the program's own eager work
             torch.cuda.synchronize()
         assert torch.equal(outs[0], outs[1]), "replay %d differs from the eager step" % k
-    assert [key[0] for key in engines[0]._graphs] == [48] and not engines[1]._graphs
+    assert [key[0] for key in engines[0]._graphs] == [48 if n_prompts == 40 else 96] and not engines[1]._graphs
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
