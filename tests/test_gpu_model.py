@@ -234,8 +234,9 @@ def test_layers_of_the_measured_shapes(tmp_path, shape):
     """Two layers of the sizes that the measurements run (a smaller vocabulary, no power of two)
     against the plain implementation.  The launcher picks the form of a product and of attention
     by the sizes and by the rows of a step, so the tiny configurations do not reach every form:
-    batches of 1, 8, 20, 48 and 64 decode through each form of the skinny product, the prompts of
-    700 tokens go through the library's products."""
+    batches of 1, 8, 20, 48 and 64 decode through each form of the skinny product, batches of 96
+    and 128 and a prompt of 100 tokens through the product for 65 to 128 rows, the prompts of 700
+    tokens through the library's products."""
     sh = dict(BENCH_SHAPES[shape])
     cfg_dict = {"model_type": "llama", "num_hidden_layers": 2, "vocab_size": 8009, "rope_theta": 500000.0,
                 "rope_scaling": {"rope_type": "llama3", "factor": sh.pop("factor"), "low_freq_factor": 1.0,
@@ -247,7 +248,8 @@ def test_layers_of_the_measured_shapes(tmp_path, shape):
     cfg = llama.PlainConfig(cfg_json)
     rng = np.random.default_rng(1)
     for batch, prompt, decode, dtypes in ((1, 40, 5, DTYPES), (8, 30, 5, DTYPES), (20, 20, 3, DTYPES),
-                                          (48, 10, 3, ["bfloat16"]), (64, 8, 3, DTYPES), (3, 700, 2, ["bfloat16"])):
+                                          (48, 10, 3, ["bfloat16"]), (64, 8, 3, DTYPES), (3, 700, 2, ["bfloat16"]),
+                                          (96, 6, 3, ["bfloat16"]), (1, 100, 2, ["bfloat16"]), (128, 1, 2, ["bfloat16"])):
         group = {"s%d_%d" % (batch, i): rng.integers(0, cfg.vocab, size=prompt + int(rng.integers(0, 9)) + decode).tolist()
                  for i in range(batch)}
         steps = traces.batches([group], {r: decode for r in group})
