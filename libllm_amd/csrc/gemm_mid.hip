@@ -33,6 +33,16 @@
 #define MID_NT 512          // threads of a block: four waves that compute, four that stage X
 #define MID_RT 2            // tiles of W a wave owns
 
+// Loads whose completion this file counts itself.  With ordinary loads the compiler makes a wave
+// wait for all of its loads once a chunk (it does not count loads across the loop's branches),
+// which puts a trip to memory into every chunk.  The compiler does not see these, so every wave
+// issues the same number per chunk, also past the end (there from one line that all lanes share),
+// and waits by count.
+typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void load16_uncounted(u32x4v& dst, const void* p) {
+  asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(dst) : "v"(p) : "memory");
+}
+
 template <int MT, int EPI, typename OutT>
 __global__ __launch_bounds__(MID_NT) void gemm_mid_kernel(const bf16_t* __restrict__ X,
                                                              const bf16_t* __restrict__ W,
@@ -77,33 +87,38 @@ __global__ __launch_bounds__(MID_NT) void gemm_mid_kernel(const bf16_t* __restri
     // loads are asked for two chunks before.  A row's 16 pieces are stored at piece ^ (row % 16):
     // the 16 lanes of a read, one row each, then fall into 16 different groups of banks.
     const int t2 = tid - 256, x_col = t2 & 15, x_row0 = t2 >> 4;
-    uint4 xr[2][PASSES];
-    // (Rows past M and chunks past the end are zeros.  Loads without a condition, rows and chunks
-    // clamped instead, let the compiler count the loads in flight and wait for fewer: measured
-    // twice as slow, 60 against 25 us at 128 x 2,048 x 16,384.)
+    static_assert(PASSES <= 8, "the waits below name eight registers");
+    u32x4v xr[2][8];
     const int last = n_chunks - 1;
-    auto load_x = [&](int chunk, uint4 (&dst)[PASSES]) {
+    auto load_x = [&](int chunk, u32x4v (&dst)[8]) {
       const int k = chunk * MID_CK + x_col * 8;
 #pragma unroll
-      for (int p = 0; p < PASSES; ++p) {
+      for (int p = 0; p < 8; ++p) {
         const int row = x_row0 + p * 16;
-        dst[p] = (row < M && chunk <= last) ? *reinterpret_cast<const uint4*>(X + (size_t)row * ldx + k)
-                                            : make_uint4(0u, 0u, 0u, 0u);
+        const bf16_t* src = (p < PASSES && row < M && chunk <= last) ? X + (size_t)row * ldx + k : X;
+        load16_uncounted(dst[p], src);
       }
     };
-    auto store_x = [&](int buf, uint4 (&src)[PASSES]) {
+    auto store_x = [&](int buf, u32x4v (&src)[8]) {
 #pragma unroll
       for (int p = 0; p < PASSES; ++p) {
         const int row = x_row0 + p * 16;
-        *reinterpret_cast<uint4*>(lds + buf * BUF + row * ROW_B + ((x_col ^ (row & 15)) * 16)) = src[p];
+        *reinterpret_cast<u32x4v*>(lds + buf * BUF + row * ROW_B + ((x_col ^ (row & 15)) * 16)) = src[p];
       }
     };
+    // all but the newest eight loads have arrived: the registers named are then valid
+#define MID_WAIT_X(R)                                                                              \
+  asm volatile("s_waitcnt vmcnt(8)"                                                                \
+               : "+v"(R[0]), "+v"(R[1]), "+v"(R[2]), "+v"(R[3]), "+v"(R[4]), "+v"(R[5]), "+v"(R[6]), \
+                 "+v"(R[7])::"memory")
     load_x(0, xr[0]);
     load_x(1, xr[1]);
+    MID_WAIT_X(xr[0]);
     store_x(0, xr[0]);
     load_x(2, xr[0]);
 #define MID_STAGE(C, CUR)                  \
   __syncthreads();                         \
+  MID_WAIT_X(CUR);                         \
   store_x(((C) + 1) & 1, CUR);             \
   load_x((C) + 3, CUR);                    \
   if ((C) + 1 >= n_chunks) break;
@@ -112,22 +127,25 @@ __global__ __launch_bounds__(MID_NT) void gemm_mid_kernel(const bf16_t* __restri
       MID_STAGE(c + 1, xr[0])
     }
 #undef MID_STAGE
+#undef MID_WAIT_X
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // nothing of this wave's is in flight when it ends
     __syncthreads();
     __syncthreads();
     return;
   }
 
-  Frag a[MID_STAGES][US][MID_RT];
+  static_assert(US == 2 && MID_RT == 2 && MID_STAGES == 6, "the waits below name four registers and count twenty loads");
+  u32x4v a[MID_STAGES][US][MID_RT];
   const int last = n_chunks - 1;
-  auto load_w = [&](int chunk, Frag (&dst)[US][MID_RT]) {
+  auto load_w = [&](int chunk, u32x4v (&dst)[US][MID_RT]) {
     const int s0 = chunk * MID_STEPS + wk * US;
 #pragma unroll
     for (int u = 0; u < US; ++u)
 #pragma unroll
       for (int rt = 0; rt < MID_RT; ++rt)
-        dst[u][rt] = chunk <= last ? frag_load(wp[rt] + (size_t)(s0 + u) * 512) : frag_zero();
+        load16_uncounted(dst[u][rt], chunk <= last ? wp[rt] + (size_t)(s0 + u) * 512 : W);
   };
-  auto compute = [&](int buf, Frag (&src)[US][MID_RT]) {
+  auto compute = [&](int buf, u32x4v (&src)[US][MID_RT]) {
 #pragma unroll
     for (int u = 0; u < US; ++u) {
       const int piece = (wk * US + u) * 4 + g;
@@ -138,9 +156,14 @@ __global__ __launch_bounds__(MID_NT) void gemm_mid_kernel(const bf16_t* __restri
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt)
 #pragma unroll
-        for (int rt = 0; rt < MID_RT; ++rt) acc[rt][mt] = mfma_bf16(src[u][rt], b[mt], acc[rt][mt]);
+        for (int rt = 0; rt < MID_RT; ++rt)
+          acc[rt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, src[u][rt]), b[mt].v,
+                                                                acc[rt][mt], 0, 0, 0);
     }
   };
+  // all but the newest twenty loads (five chunks) have arrived
+#define MID_WAIT_W(R) \
+  asm volatile("s_waitcnt vmcnt(20)" : "+v"(R[0][0]), "+v"(R[0][1]), "+v"(R[1][0]), "+v"(R[1][1])::"memory")
 
 #pragma unroll
   for (int c = 0; c < MID_STAGES - 1; ++c) load_w(c, a[c]);
@@ -148,6 +171,7 @@ __global__ __launch_bounds__(MID_NT) void gemm_mid_kernel(const bf16_t* __restri
 #define MID_STEP(C, CUR, NXT)                 \
   __syncthreads();                            \
   load_w((C) + MID_STAGES - 1, NXT);          \
+  MID_WAIT_W(CUR);                            \
   compute((C) & 1, CUR);                      \
   if ((C) + 1 >= n_chunks) break;
   for (int c = 0;; c += 6) {
@@ -158,6 +182,8 @@ __global__ __launch_bounds__(MID_NT) void gemm_mid_kernel(const bf16_t* __restri
     MID_STEP(c + 4, a[4], a[3])
     MID_STEP(c + 5, a[5], a[4])
   }
+#undef MID_WAIT_W
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // nothing of this wave's is in flight past here
 #undef MID_STEP
 
   // ---- the second wave of a pair hands its sums to the first through shared memory

@@ -100,14 +100,12 @@ class HipOps:
     ACCUM_ROWS = 16         # most rows for which a product adds into the stream itself
     SPLIT_ROWS = 64         # beyond those and up to here it goes in slices of K that the next norm adds; then the library's
     # 65 to MID_ROWS rows: a streaming product of their own for weights with a tiled copy; beyond,
-    # the library's.  Whole engines compared in one process, prompt steps of 65 to 128 tokens: 3.54
-    # against 4.17 ms at the 3B shape, 6.19 against 7.01 at 8B; decode batches of 96: 3.92 against
-    # 5.25 and 6.25 against 7.05.  At the 1B shape the library's products for the two small
-    # weights and for gate/up at 128 rows are as fast or 1 % faster: hence the two limits below.
+    # the library's.  Whole engines compared in one process, prompt steps of 65 to 128 tokens: 3.40
+    # against 4.16 ms at the 3B shape, 5.93 against 7.07 at 8B, 1.62 against 1.66 at 1B; decode
+    # batches of 96: 3.66 against 4.33, 6.10 against 7.08, 1.72 against 1.82.  For the small o
+    # weight of the 1B shape the library's product is as fast (10.2 against 10.4 us): hence the limit.
     MID_ROWS = 128
     MID_MIN_WEIGHT = 3072 * 3072    # elements of a weight from which a product that adds into the stream takes it (in slices of K)
-    MID_SWIGLU_K = 3072             # width from which gate/up takes it at more than MID_SWIGLU_ROWS rows
-    MID_SWIGLU_ROWS = 96
     DECODE_BLOCKS = 768     # blocks of the decode attention grid beyond which sequences are not split further
     DECODE_BLOCKS_AHEAD = 512   # the same where a wave would get DECODE_AHEAD_PAGES pages or more and the sequences
     DECODE_AHEAD_PAGES = 6      # fill such a grid: two blocks a compute unit, at which the kernel overlaps a wave's pages
@@ -448,8 +446,7 @@ class HipOps:
                 raise KernelError("linear_swiglu: a normed record needs the activation dtype")
             x = self._materialise(x, dtype)
             return self.linear_swiglu(x, w, dtype)
-        if (self._mid_ok(x, w, m, k) and inter % 16 == 0 and dtype == torch.bfloat16
-                and (m <= self.MID_SWIGLU_ROWS or k >= self.MID_SWIGLU_K)):
+        if self._mid_ok(x, w, m, k) and inter % 16 == 0 and dtype == torch.bfloat16:
             self._weight(self._plain(w), "linear weight")
             return self._mid(x, w, torch.empty((m, inter), dtype=torch.bfloat16, device=self.device),
                              self._EPI_SWIGLU)
