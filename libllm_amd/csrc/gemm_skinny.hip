@@ -143,7 +143,11 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
     }
   };
   const int wstep = (ldw == 0) ? 512 : 32;       // elements between a lane's fragments of consecutive steps
-  Frag a[3][G][2][RT];
+  // Stages of W in registers: fragments are asked for ST - 1 chunks ahead.  Up to 32 rows of X one
+  // chunk ahead is 2 to 3 % of a decode step faster than two (fewer registers, and the compiler
+  // makes a wave wait for all its loads at every chunk anyway); from 33 rows on it is a third slower.
+  constexpr int ST = (MT <= 2) ? 2 : 3;
+  Frag a[ST][G][2][RT];
   auto load_w = [&](int chunk, Frag (&dst)[G][2][RT]) {
 #pragma unroll
     for (int gi = 0; gi < G; ++gi)
@@ -171,10 +175,10 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
       }
   };
 
-  // W fragments are fetched two chunks ahead (three register stages in rotation), X one chunk
+  // W fragments are fetched ST - 1 chunks ahead (the register stages in rotation), X one chunk
   load_x(0);
   load_w(0, a[0]);
-  if (1 < n_chunks) load_w(1, a[1]);
+  if (ST == 3 && 1 < n_chunks) load_w(1, a[1]);
 
   // What the epilogue needs from memory beside the sums is asked for now, behind the first loads:
   // a thread finishes at most one group of four outputs per round (ITEMS <= NT), and which one is
@@ -246,14 +250,21 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   store_x();                                    \
   __syncthreads();                              \
   if ((C) + 1 < n_chunks) load_x((C) + 1);      \
-  if ((C) + 2 < n_chunks) load_w((C) + 2, NXT); \
+  if ((C) + ST - 1 < n_chunks) load_w((C) + ST - 1, NXT); \
   compute(CUR);                                 \
   __syncthreads();                              \
   if ((C) + 1 >= n_chunks) break;
-  for (int c = 0;; c += 3) {
-    SK_STEP(c, a[0], a[2])
-    SK_STEP(c + 1, a[1], a[0])
-    SK_STEP(c + 2, a[2], a[1])
+  if constexpr (ST == 3) {
+    for (int c = 0;; c += 3) {
+      SK_STEP(c, a[0], a[2])
+      SK_STEP(c + 1, a[1], a[0])
+      SK_STEP(c + 2, a[ST - 1], a[1])
+    }
+  } else {
+    for (int c = 0;; c += 2) {
+      SK_STEP(c, a[0], a[1])
+      SK_STEP(c + 1, a[1], a[0])
+    }
   }
 #undef SK_STEP
 
