@@ -143,10 +143,10 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
     }
   };
   const int wstep = (ldw == 0) ? 512 : 32;       // elements between a lane's fragments of consecutive steps
-  // Stages of W in registers: fragments are asked for ST - 1 chunks ahead.  Up to 32 rows of X one
-  // chunk ahead is 2 to 3 % of a decode step faster than two (fewer registers, and the compiler
-  // makes a wave wait for all its loads at every chunk anyway); from 33 rows on it is a third slower.
-  constexpr int ST = (MT <= 2) ? 2 : 3;
+  // Stages of W in registers: fragments are asked for ST - 1 chunks ahead.  Up to 48 rows of X one
+  // chunk ahead is up to 3 % of a decode step faster than two (fewer registers, and the compiler
+  // makes a wave wait for all its loads at every chunk anyway); from 49 rows on it is a third slower.
+  constexpr int ST = (MT <= 3) ? 2 : 3;
   Frag a[ST][G][2][RT];
   auto load_w = [&](int chunk, Frag (&dst)[G][2][RT]) {
 #pragma unroll
