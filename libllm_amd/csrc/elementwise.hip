@@ -80,12 +80,21 @@ __global__ __launch_bounds__(NT) void add_rmsnorm_reg_kernel(float* __restrict__
     v[j] = in ? *reinterpret_cast<const float4*>(x + i) : make_float4(0.f, 0.f, 0.f, 0.f);
     wv[j] = in ? *reinterpret_cast<const float4*>(w + i) : make_float4(0.f, 0.f, 0.f, 0.f);
     if (d && in) {
-      for (int q = 0; q < n_delta; ++q) {                  // several deltas are added in this order
-        const float4 dv = Conv4<TD>::load(d + q * delta_stride + i);
-        v[j].x += dv.x;
-        v[j].y += dv.y;
-        v[j].z += dv.z;
-        v[j].w += dv.w;
+      // several deltas are added in this order; eight are asked for before the first is added, so
+      // that a row waits for memory once and not once a delta
+      for (int q0 = 0; q0 < n_delta; q0 += 8) {
+        float4 dv[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (q0 + u < n_delta) dv[u] = Conv4<TD>::load(d + (size_t)(q0 + u) * delta_stride + i);
+#pragma unroll
+        for (int u = 0; u < 8; ++u)
+          if (q0 + u < n_delta) {
+            v[j].x += dv[u].x;
+            v[j].y += dv[u].y;
+            v[j].z += dv[u].z;
+            v[j].w += dv[u].w;
+          }
       }
       *reinterpret_cast<float4*>(x + i) = v[j];
     }
