@@ -2,21 +2,19 @@
 // many rows for a block to stage all of them per 16 rows of W, as the product for few rows does.
 // bfloat16 inputs, float32 accumulation on the matrix cores.
 //
-// A block of 4 waves owns 64 rows of W over all of K or one slice of it: two pairs of waves with
-// two tiles of 16 rows each (what a wave reads of X from shared memory serves both tiles; that
-// traffic is what bounds this kernel), the first wave of a pair taking the first two steps (of
-// 32 elements) of every chunk of 128, the second the other two.  W is the copy tiled for the
-// matrix cores (llm_pack_weight): a wave's fragment of a step is 1 KiB in a row, and goes from
-// global memory straight to registers, five chunks ahead.  The rows of X go through shared
-// memory, a chunk at a time, in two buffers filled in turns (one barrier a chunk), and four
-// more waves do nothing but that: a wave's loads complete in the order they were asked for, so a
-// wave that waited for the rows of the next chunk would wait for every fragment of W asked for
-// before them (with every wave doing both, a chunk took 1.9 us instead of 1.5).  The four waves
-// that compute read the rows as B operands, so
-// lane l ends with
-// C[m = 16 mt + l % 16][n = 4 (l / 16) + e] for the 16 rows n of a tile of W.  The two waves of a
-// pair add their sums through shared memory, first wave first: a row's bits do not depend on the
-// other rows.
+// A block owns 64 rows of W over all of K or one slice of it.  Four of its eight waves compute:
+// two pairs of waves with two tiles of 16 rows each (what a wave reads of X from shared memory
+// serves both tiles), the first wave of a pair taking the first two steps (of 32 elements) of
+// every chunk of 128, the second the other two.  W is the copy tiled for the matrix cores
+// (llm_pack_weight): a wave's fragment of a step is 1 KiB in a row, and goes from global memory
+// straight to registers, five chunks ahead.  The rows of X go through shared memory, a chunk at a
+// time, in two buffers filled in turns (one barrier a chunk), and the other four waves do nothing
+// but that: a wave's loads complete in the order they were asked for, so a wave that waited for
+// the rows of the next chunk would wait for every fragment of W asked for before them (with
+// every wave doing both, a chunk took 1.9 us instead of 1.5).  The waves that compute read the
+// rows as B operands, so lane l ends with C[m = 16 mt + l % 16][n = 4 (l / 16) + e] for the 16
+// rows n of a tile of W.  The two waves of a pair add their sums through shared memory, first
+// wave first: a row's bits do not depend on the other rows.
 //
 // Epilogues: plain store as bfloat16; with slices of K (grid height > 1), float32 matrices
 // [slice, M, N] that the caller adds in order; or SwiGLU over a stacked [gate; up] weight
@@ -37,7 +35,10 @@
 // wait for all of its loads once a chunk (it does not count loads across the loop's branches),
 // which puts a trip to memory into every chunk.  The compiler does not see these, so every wave
 // issues the same number per chunk, also past the end (there from one line that all lanes share),
-// and waits by count.
+// and waits by count.  A register such a load fills must not be read, copied or spilled before
+// the wait that covers it: the waits name those registers as operands, and no form of the kernel
+// may spill (the build prints none; the tests compare every form with float64 and bit for bit
+// across row counts).
 typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void load16_uncounted(u32x4v& dst, const void* p) {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(dst) : "v"(p) : "memory");
