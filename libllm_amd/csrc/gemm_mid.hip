@@ -37,8 +37,8 @@
 // issues the same number per chunk, also past the end (there from one line that all lanes share),
 // and waits by count.  A register such a load fills must not be read, copied or spilled before
 // the wait that covers it: the waits name those registers as operands, and no form of the kernel
-// may spill (the build prints none; the tests compare every form with float64 and bit for bit
-// across row counts).
+// may spill (a test compiles this file and checks that; others compare every form with float64,
+// and bit for bit across row counts).
 typedef uint32_t u32x4v __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ void load16_uncounted(u32x4v& dst, const void* p) {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(dst) : "v"(p) : "memory");
