@@ -31,13 +31,16 @@ class Engine:
     # batch sizes the decode graphs are captured for; a step runs in the smallest that holds it, its
     # spare rows pointing at the sink.  With powers of two alone a batch of 40 paid for 64 rows
     # (2.73 ms a step at the 1B shape against 2.43 in a graph of 48).
-    GRAPH_BATCHES = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64, 96, 128)
+    GRAPH_BATCHES = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64, 80, 96, 112, 128)
     GRAPH_MIN_CTX = 1024
     # Steps that bring whole prompts are captured too, padded to one of these numbers of rows and
     # of sequences (one sequence is always spare: it takes the padding rows, in the sink slot).  A
     # shape is captured when it comes the second time, so that a lone prompt does not pay for it.
     # Queued from the host a prompt of up to some hundred tokens waits for the host, not the device.
-    PROMPT_ROWS = (16, 32, 64, 128, 192, 256, 384, 512, 768, 1024, 1536, 2048)
+    # Up to 128 rows the steps are 16 apart, as the products' forms are: a prompt of 70 tokens in
+    # a graph of 80 or 96 rows takes 1.47 ms where one of 128 rows takes 1.58 (1B shape; 5.34
+    # against 5.85 at 8B).
+    PROMPT_ROWS = (16, 32, 48, 64, 80, 96, 112, 128, 192, 256, 384, 512, 768, 1024, 1536, 2048)
     PROMPT_SEQS = (2, 3, 5, 9, 17)
     PROMPT_SEEN = 2
     PROMPT_GRAPHS = 24      # prompt graphs kept; the one unused for longest goes first (each holds its activations)
