@@ -7,7 +7,9 @@
 // serves both tiles), the first wave of a pair taking the first two steps (of 32 elements) of
 // every chunk of 128, the second the other two.  W is the copy tiled for the matrix cores
 // (llm_pack_weight): a wave's fragment of a step is 1 KiB in a row, and goes from global memory
-// straight to registers, five chunks ahead.  The rows of X go through shared memory, a chunk at a
+// straight to registers, three chunks ahead (four register stages: with six and five chunks
+// ahead the kernel needs 164 registers instead of 128, one block instead of two fits a compute
+// unit, and it is 3 to 7 % slower).  The rows of X go through shared memory, a chunk at a
 // time, in two buffers filled in turns (one barrier a chunk), and the other four waves do nothing
 // but that: a wave's loads complete in the order they were asked for, so a wave that waited for
 // the rows of the next chunk would wait for every fragment of W asked for before them (with
@@ -26,7 +28,7 @@
 #define MID_EPI_SWIGLU 1
 #define MID_CK 128          // elements of K per chunk
 #define MID_STEPS 4         // steps of 32 per chunk
-#define MID_STAGES 6        // chunks of W in registers
+#define MID_STAGES 4        // chunks of W in registers
 #define MID_WK 2            // waves that share a tile of W, splitting each chunk's steps
 #define MID_NT 512          // threads of a block: four waves that compute, four that stage X
 #define MID_RT 2            // tiles of W a wave owns
@@ -45,7 +47,7 @@ __device__ __forceinline__ void load16_uncounted(u32x4v& dst, const void* p) {
 }
 
 template <int MT, int EPI, typename OutT>
-__global__ __launch_bounds__(MID_NT) void gemm_mid_kernel(const bf16_t* __restrict__ X,
+__global__ __launch_bounds__(MID_NT, 2) void gemm_mid_kernel(const bf16_t* __restrict__ X,
                                                              const bf16_t* __restrict__ W,
                                                              OutT* __restrict__ C, int M, int N, int K,
                                                              int ldx, int w_steps, int n_out) {
@@ -135,7 +137,7 @@ __global__ __launch_bounds__(MID_NT) void gemm_mid_kernel(const bf16_t* __restri
     return;
   }
 
-  static_assert(US == 2 && MID_RT == 2 && MID_STAGES == 6, "the waits below name four registers and count twenty loads");
+  static_assert(US == 2 && MID_RT == 2 && MID_STAGES == 4, "the waits below name four registers and count twelve loads");
   u32x4v a[MID_STAGES][US][MID_RT];
   const int last = n_chunks - 1;
   auto load_w = [&](int chunk, u32x4v (&dst)[US][MID_RT]) {
@@ -162,9 +164,9 @@ __global__ __launch_bounds__(MID_NT) void gemm_mid_kernel(const bf16_t* __restri
                                                                 acc[rt][mt], 0, 0, 0);
     }
   };
-  // all but the newest twenty loads (five chunks) have arrived
+  // all but the newest twelve loads (three chunks) have arrived
 #define MID_WAIT_W(R) \
-  asm volatile("s_waitcnt vmcnt(20)" : "+v"(R[0][0]), "+v"(R[0][1]), "+v"(R[1][0]), "+v"(R[1][1])::"memory")
+  asm volatile("s_waitcnt vmcnt(12)" : "+v"(R[0][0]), "+v"(R[0][1]), "+v"(R[1][0]), "+v"(R[1][1])::"memory")
 
 #pragma unroll
   for (int c = 0; c < MID_STAGES - 1; ++c) load_w(c, a[c]);
@@ -175,13 +177,11 @@ __global__ __launch_bounds__(MID_NT) void gemm_mid_kernel(const bf16_t* __restri
   MID_WAIT_W(CUR);                            \
   compute((C) & 1, CUR);                      \
   if ((C) + 1 >= n_chunks) break;
-  for (int c = 0;; c += 6) {
-    MID_STEP(c, a[0], a[5])
+  for (int c = 0;; c += 4) {
+    MID_STEP(c, a[0], a[3])
     MID_STEP(c + 1, a[1], a[0])
     MID_STEP(c + 2, a[2], a[1])
     MID_STEP(c + 3, a[3], a[2])
-    MID_STEP(c + 4, a[4], a[3])
-    MID_STEP(c + 5, a[5], a[4])
   }
 #undef MID_WAIT_W
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");       // nothing of this wave's is in flight past here

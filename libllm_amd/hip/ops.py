@@ -100,9 +100,9 @@ class HipOps:
     ACCUM_ROWS = 16         # most rows for which a product adds into the stream itself
     SPLIT_ROWS = 64         # beyond those and up to here it goes in slices of K that the next norm adds; then the library's
     # 65 to MID_ROWS rows: a streaming product of their own for weights with a tiled copy; beyond,
-    # the library's.  Whole engines compared in one process, prompt steps of 65 to 128 tokens: 3.40
-    # against 4.16 ms at the 3B shape, 5.93 against 7.07 at 8B, 1.62 against 1.66 at 1B; decode
-    # batches of 96: 3.66 against 4.33, 6.10 against 7.08, 1.72 against 1.82.  For the small o
+    # the library's.  Whole engines compared in one process, prompt steps of 128 tokens: 3.27
+    # against 4.18 ms at the 3B shape, 5.57 against 7.07 at 8B, 1.62 against 1.66 at 1B; decode
+    # batches of 96: 3.56 against 4.34, 5.84 against 7.10, 1.72 against 1.82.  For the small o
     # weight of the 1B shape the library's product is as fast (10.2 against 10.4 us): hence the limit.
     MID_ROWS = 128
     MID_MIN_WEIGHT = 3072 * 3072    # elements of a weight from which a product that adds into the stream takes it (in slices of K)
