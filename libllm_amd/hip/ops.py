@@ -105,6 +105,7 @@ class HipOps:
     # batches of 96: 3.56 against 4.34, 5.84 against 7.10, 1.72 against 1.82.  For the small o
     # weight of the 1B shape the library's product is as fast (10.2 against 10.4 us): hence the limit.
     MID_ROWS = 128
+    MID_BLOCKS = 256                # blocks that its slices of K aim at (128 and 512 lose 8 to 10 % of a prompt step of 128 tokens at the 3B and 8B shapes: fewer blocks, or more matrices for the norm to add)
     MID_MIN_WEIGHT = 3072 * 3072    # elements of a weight from which a product that adds into the stream takes it (in slices of K)
     DECODE_BLOCKS = 768     # blocks of the decode attention grid beyond which sequences are not split further
     DECODE_BLOCKS_AHEAD = 512   # the same where a wave would get DECODE_AHEAD_PAGES pages or more and the sequences
@@ -308,12 +309,10 @@ class HipOps:
                 and x.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1 and x.stride(0) >= k
                 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and k % 128 == 0)
 
-    @staticmethod
-    def _k_split_mid(n, k):
+    def _k_split_mid(self, n, k):
         """Slices of K for a product of 65 to 128 rows whose result the next norm adds: enough for
-        about a block a compute unit at 64 weight rows a block, each at least 256 long and a
-        multiple of 128."""
-        ks = max(1, min(16, 256 // max(1, -(-n // 64))))
+        about MID_BLOCKS blocks at 64 weight rows a block, each at least 256 long and a multiple of 128."""
+        ks = max(1, min(16, self.MID_BLOCKS // max(1, -(-n // 64))))
         while ks > 1 and (k % (ks * 128) or k // ks < 256):
             ks -= 1
         return ks
