@@ -57,6 +57,23 @@ def test_greedy_generation_through_the_entry_point(model_b, dtype):
     assert model.engine.cache.slots.n_free == model.engine.cache.slots.n_slots
 
 
+def test_greedy_generation_of_a_wide_batch(model_b):
+    """Seventy requests at once, in 32-bit: their prompts in one step, then decode steps of 70 rows
+    (a captured graph of 80 rows, ten of them pointing at the sink), as the plain implementation
+    generates each request alone."""
+    from libllm_amd import Device, Model
+    path, cfg, weights = model_b
+    rng = np.random.default_rng(9)
+    prompts = [rng.integers(10, cfg.vocab, size=int(n)).tolist() for n in rng.integers(1, 12, size=70)]
+    model = Model(path, Device.AUTO, dtype="float32", max_tokens=70 * 64, max_batch=70)
+    got = model.generate(prompts, max_new_tokens=5, temperature=0.0)
+    assert [k[0] for k in model.engine._graphs] == [80]
+    for p, g in zip(prompts[::7], got[::7]):
+        assert g == sampling.generate(cfg, weights, p, 5)
+    model.engine.cache.check()
+    assert model.engine.cache.slots.n_free == model.engine.cache.slots.n_slots
+
+
 def test_sampled_generation_and_stop_tokens(model_b):
     from libllm_amd import Model
     path, cfg, weights = model_b
