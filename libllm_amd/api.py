@@ -111,10 +111,11 @@ class Completion:
 class Model:
     def __init__(self, config_file: str, device: Union[Device, str] = Device.AUTO, dtype: str = "bfloat16",
                  max_tokens: int = 8192, max_batch: int = 64, ops=None, use_graphs: bool = True,
-                 random_weights: bool = False, seed: int = 0) -> None:
+                 random_weights: bool = False, seed: int = 0, keep_float32: bool = False) -> None:
         """``config_file``: the model folder, or the config.json inside it.  ``device``: a Device
         or one of "auto", "cuda", "hip", "cpu".  With ``random_weights`` only config.json is read
-        and every tensor is drawn from ``seed``."""
+        and every tensor is drawn from ``seed``.  ``keep_float32``: in bfloat16 mode, matrices
+        that the file stores in 32-bit stay float32 instead of becoming bfloat16."""
         if int(parse_device(device)) == int(Device.CPU):
             raise ConfigError("this library has no CPU path; use Device.AUTO or Device.GPU")
         model_dir = os.path.dirname(config_file) if os.path.isfile(config_file) else config_file
@@ -124,7 +125,7 @@ class Model:
                                         max_tokens=max_tokens, ops=ops, use_graphs=use_graphs)
         else:
             self.engine = load_engine(model_dir, dtype=dtype, max_tokens=max_tokens, ops=ops,
-                                      use_graphs=use_graphs)
+                                      use_graphs=use_graphs, keep_float32=keep_float32)
         self.config = self.engine.config
         spec = self.engine.model.spec
         self._sampler = Sampler(self.engine.ops, spec.vocab)
@@ -190,8 +191,10 @@ class Model:
         return self._generator.generate(prompts, params, max_new_tokens, stop_tokens, on_token)
 
     def step(self, entries: Sequence[StepEntry]):
-        """One call of the step function; float32 logits ``[wanted, vocab]`` on the device."""
-        return self.engine.step(list(entries))
+        """One call of the step function; float32 logits ``[wanted, vocab]`` on the device, in a
+        tensor of the caller's own (None if nothing is wanted)."""
+        logits = self.engine.step(list(entries))
+        return None if logits is None else logits.clone()
 
     def end(self, requests) -> None:
         self.engine.end(requests)

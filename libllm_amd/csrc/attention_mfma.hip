@@ -615,19 +615,21 @@ __global__ void attn_decode_combine_kernel(const float* __restrict__ part_o,
   if (live) out[((size_t)b * n_heads + h) * hd + d] = f32_to_bf16(o / l);
 }
 
-// The same for any number of partials: block (dims, 8 groups); group g merges partials g, g+8, ...
-// as they come (a running maximum), then the 8 groups are merged through shared memory.
+// The same for any number of partials: block (dims, G groups); group g merges partials g, g+G, ...
+// as they come (a running maximum), then the G groups are merged through shared memory.  G is 8
+// for heads of up to 128 dims and 4 beyond, so that the block stays within 1,024 threads.
+template <int G>
 __global__ void attn_decode_combine_loop_kernel(const float* __restrict__ part_o,
                                                 const float* __restrict__ part_ml,
                                                 bf16_t* __restrict__ out, int n_heads, int hd,
                                                 int n_blk) {
-  __shared__ float s_m[8], s_l[8], s_o[8][256];
+  __shared__ float s_m[G], s_l[G], s_o[G][256];
   const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x, grp = threadIdx.y;
   const size_t idx0 = ((size_t)b * n_heads + h) * n_blk;
   const bool live = d < hd;
   float m = -INFINITY, l = 0.f, o = 0.f;
 #pragma unroll 4
-  for (int s = grp; s < n_blk; s += 8) {
+  for (int s = grp; s < n_blk; s += G) {
     const float2 ml = *reinterpret_cast<const float2*>(part_ml + (idx0 + s) * 2);
     const float ov = live ? part_o[(idx0 + s) * hd + d] : 0.f;
     if (ml.x > -INFINITY) {
@@ -647,10 +649,10 @@ __global__ void attn_decode_combine_loop_kernel(const float* __restrict__ part_o
   if (grp != 0 || !live) return;
   float mm = s_m[0];
 #pragma unroll
-  for (int g = 1; g < 8; ++g) mm = fmaxf(mm, s_m[g]);
+  for (int g = 1; g < G; ++g) mm = fmaxf(mm, s_m[g]);
   float lt = 0.f, ot = 0.f;
 #pragma unroll
-  for (int g = 0; g < 8; ++g) {
+  for (int g = 0; g < G; ++g) {
     const float w = (s_m[g] > -INFINITY) ? exp2f(s_m[g] - mm) : 0.f;
     lt += s_l[g] * w;
     ot += s_o[g][d] * w;
@@ -767,8 +769,11 @@ extern "C" int llm_attention_decode_bf16(const void* q, int q_stride, const void
         attn_decode_combine_kernel<32><<<cgrid, cthreads, 0, stream>>>(part_o, part_ml,           \
                                                                       (bf16_t*)out, n_heads, hd,  \
                                                                       n_blocks);                  \
+      else if (cthreads <= 128)                                                                   \
+        attn_decode_combine_loop_kernel<8><<<cgrid, dim3(cthreads, 8), 0, stream>>>(              \
+            part_o, part_ml, (bf16_t*)out, n_heads, hd, n_blocks);                                \
       else                                                                                        \
-        attn_decode_combine_loop_kernel<<<cgrid, dim3(cthreads, 8), 0, stream>>>(                 \
+        attn_decode_combine_loop_kernel<4><<<cgrid, dim3(cthreads, 4), 0, stream>>>(              \
             part_o, part_ml, (bf16_t*)out, n_heads, hd, n_blocks);                                \
     }                                                                                             \
     return llm_launch_status();                                                                   \

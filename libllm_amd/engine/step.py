@@ -80,7 +80,11 @@ class Engine:
     def step(self, entries: List[StepEntry], tokens_device: Optional[torch.Tensor] = None
              ) -> Optional[torch.Tensor]:
         """Returns float32 logits ``[wanted, vocab]`` in the order of the entries and of their
-        ``want`` lists, or None if nothing is wanted.
+        ``want`` lists, or None if nothing is wanted.  The tensor may be a view of a captured
+        graph's output buffer: it holds these logits until the next call of ``step``, which may
+        overwrite it (on the same stream, so work already queued on it, such as sampling, still
+        reads this step's values).  A caller that keeps logits across steps copies them;
+        ``Model.step`` does.
 
         With ``tokens_device`` (int32 on the device, one per entry, for instance what the sampler
         just wrote) every entry brings exactly one token and that tensor holds it: the ids in the
@@ -198,9 +202,10 @@ class Engine:
             return None
         rows = next(r for r in self.PROMPT_ROWS if r >= m)
         seqs = next(q for q in self.PROMPT_SEQS if q >= b + 1)
-        # the spare sequence may take all rows but one: its positions must lie within a table row;
-        # the wanted rows must fit the places the graph has for them
-        if rows > self.cache.pages_per_seq * PAGE or wanted > seqs:
+        # the spare sequence may take all rows but one, at positions 0..: they must lie within a
+        # row of the page table and within the position encoding's tables (the position limit
+        # need not be a multiple of a page); the wanted rows must fit the places the graph has
+        if rows > min(self.cache.pages_per_seq * PAGE, self.cache.max_position) or wanted > seqs:
             return None
         key = (rows, seqs)
         graph = self._prompt_graphs.pop(key, None)

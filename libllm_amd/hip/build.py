@@ -7,7 +7,9 @@ the library cannot be loaded or built, KernelError says why.
 """
 import ctypes
 import hashlib
+import json
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -30,6 +32,16 @@ LIB_NAME = "libllm_amd_hip.so"
 OPTIONAL_FLAGS = ["-mllvm", "-amdgpu-mfma-vgpr-form=1"]    # left out for a compiler that does not know the switch
 FLAGS = ["--offload-arch=" + ARCH, "-O3", "-fPIC", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"] + OPTIONAL_FLAGS
+# Every source is compiled with the compiler's report of what each kernel uses.  It is read for
+# the kernels that are only right if the compiler spills none of their registers (they fill
+# registers by load instructions that the compiler does not see and wait for them by count: a
+# register saved to memory before its load arrived would be saved with its old contents).  What
+# is found goes into a file beside the library, and the host switches such a kernel off if any
+# of its forms spills: the property belongs to the build that runs, whichever flags it took.
+REPORT_FLAGS = ["-Rpass-analysis=kernel-resource-usage"]
+NO_SPILL_KERNELS = {"gemm_mid.hip": "gemm_mid_kernel"}     # source -> name that its kernels' symbols contain
+INFO_NAME = "libllm_amd_hip.so.json"
+_FORMAT = "build-info-1"                                   # part of the hash: a build without the file is not current
 
 _lib: Optional[ctypes.CDLL] = None
 
@@ -45,8 +57,24 @@ def source_hash() -> str:
         h.update(os.path.basename(path).encode())
         with open(path, "rb") as f:
             h.update(f.read())
-    h.update(" ".join(FLAGS).encode())
+    h.update(" ".join(FLAGS + REPORT_FLAGS + [_FORMAT]).encode())
     return h.hexdigest()[:20]
+
+
+def spills_in_report(report: str, name_part: str):
+    """From the compiler's resource report: (number of kernels whose symbol contains
+    ``name_part``, the symbols among them that spill a vector or scalar register or use scratch
+    memory).  A report that does not give a kernel's spills counts that kernel as spilling."""
+    kernels, bad = 0, []
+    for block in report.split("Function Name: ")[1:]:
+        name = block.split()[0]
+        if name_part not in name:
+            continue
+        kernels += 1
+        found = {key: re.search(key + r"[^:\n]*: (\d+)", block) for key in ("VGPRs Spill", "SGPRs Spill", "ScratchSize")}
+        if any(m is None or int(m.group(1)) != 0 for m in found.values()):
+            bad.append(name)
+    return kernels, bad
 
 
 def _say(msg: str) -> None:
@@ -81,7 +109,7 @@ def _writable(d: str) -> bool:
 
 def _current(d: str, want: str) -> bool:
     so, stamp = os.path.join(d, LIB_NAME), os.path.join(d, LIB_NAME + ".hash")
-    if not (os.path.isfile(so) and os.path.isfile(stamp)):
+    if not (os.path.isfile(so) and os.path.isfile(stamp) and os.path.isfile(os.path.join(d, INFO_NAME))):
         return False
     with open(stamp, "r") as f:
         return f.read().strip() == want
@@ -108,20 +136,31 @@ def build(force: bool = True, verbose: bool = True) -> str:
     if verbose:
         _say("compiling %d HIP sources for %s into %s" % (len(srcs), ARCH, target))
 
+    info = {"hash": want, "optional_flags": True, "no_spill": {}}
+
     def compile_one(src):
-        obj = os.path.join(objdir, os.path.basename(src)[:-4] + ".o")
-        cmd = [hipcc] + FLAGS + ["-I", CSRC, "-c", src, "-o", obj]
+        base = os.path.basename(src)
+        obj = os.path.join(objdir, base[:-4] + ".o")
+        cmd = [hipcc] + FLAGS + REPORT_FLAGS + ["-I", CSRC, "-c", src, "-o", obj]
         proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         if proc.returncode != 0 and OPTIONAL_FLAGS[-1].split("=")[0].lstrip("-") in proc.stdout:
             if verbose:
                 _say("  this hipcc does not know %s: compiling %s without it (the attention kernels "
-                     "run somewhat slower)" % (OPTIONAL_FLAGS[-1], os.path.basename(src)))
-            cmd = [hipcc] + FLAGS[:-len(OPTIONAL_FLAGS)] + ["-I", CSRC, "-c", src, "-o", obj]
+                     "run somewhat slower)" % (OPTIONAL_FLAGS[-1], base))
+            info["optional_flags"] = False
+            cmd = [hipcc] + FLAGS[:-len(OPTIONAL_FLAGS)] + REPORT_FLAGS + ["-I", CSRC, "-c", src, "-o", obj]
             proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
         if proc.returncode != 0:
-            raise KernelError("hipcc failed on %s:\n%s" % (os.path.basename(src), proc.stdout[-4000:]))
+            raise KernelError("hipcc failed on %s:\n%s" % (base, proc.stdout[-4000:]))
+        if base in NO_SPILL_KERNELS:
+            kernels, bad = spills_in_report(proc.stdout, NO_SPILL_KERNELS[base])
+            info["no_spill"][base] = {"kernels": kernels, "spilling": bad}
+            if verbose and (bad or not kernels):
+                _say("  %s: %s; the host will not use these kernels"
+                     % (base, "%d of %d forms spill registers" % (len(bad), kernels) if kernels
+                        else "the compiler's report names no kernel"))
         if verbose:
-            _say("  compiled %s (%.0f s since start)" % (os.path.basename(src), time.time() - t0))
+            _say("  compiled %s (%.0f s since start)" % (base, time.time() - t0))
         return obj
 
     with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
@@ -132,11 +171,27 @@ def build(force: bool = True, verbose: bool = True) -> str:
     if proc.returncode != 0:
         raise KernelError("linking the kernel library failed:\n%s" % proc.stdout[-4000:])
     os.replace(tmp_so, os.path.join(target, LIB_NAME))
+    with open(os.path.join(target, INFO_NAME), "w") as f:
+        json.dump(info, f, indent=1)
     with open(os.path.join(target, LIB_NAME + ".hash"), "w") as f:
         f.write(want)
     if verbose:
         _say("built %s in %.0f s" % (LIB_NAME, time.time() - t0))
     return os.path.join(target, LIB_NAME)
+
+
+def info(path: Optional[str] = None) -> dict:
+    """What the build that made the library at ``path`` (default: the one ``load`` takes) found."""
+    path = path or build(force=False)
+    with open(os.path.join(os.path.dirname(path), INFO_NAME), "r") as f:
+        return json.load(f)
+
+
+def trusted(source: str, path: Optional[str] = None) -> bool:
+    """Whether the kernels of ``source`` (a key of NO_SPILL_KERNELS) may run: the build found
+    them, and none of their forms spills."""
+    found = info(path).get("no_spill", {}).get(source)
+    return bool(found) and found["kernels"] > 0 and not found["spilling"]
 
 
 CAPI_NAME = "libllm.so"

@@ -140,6 +140,10 @@ class HipOps:
         self.pack_weights = True        # keep a tiled copy of every weight for the skinny product
         self.fast_gemm = True           # the skinny product for few rows (else the library's for every product)
         self.mid_gemm = True            # the product for 65 to 128 rows (else the library's)
+        if not build.trusted("gemm_mid.hip"):
+            # its loads are invisible to the compiler: with a spilled register it would be wrong
+            self.mid_gemm = False
+            build._say("the product for 65 to 128 rows spills registers in this build: the library's runs instead")
         self.fold_norms = True          # up to ACCUM_ROWS rows, a norm between two products gets no kernel of its own
         self.prompt_tiles = 0           # tiles of rows a wave of prompt attention takes (1 or 2; 0: by the number of blocks)
 

@@ -31,15 +31,19 @@ def default_ops():
 
 
 def load_engine(model_dir: str, dtype="bfloat16", max_tokens: int = 8192, ops=None,
-                max_slots: Optional[int] = None, use_graphs: bool = True) -> Engine:
+                max_slots: Optional[int] = None, use_graphs: bool = True,
+                keep_float32: bool = False) -> Engine:
     """Reads config.json, chooses the architecture by its ``model_type``, loads the tensors by
-    name and returns an engine whose cache holds ``max_tokens`` tokens."""
+    name and returns an engine whose cache holds ``max_tokens`` tokens.  ``keep_float32``: in
+    bfloat16 mode a matrix that the file stores in 32-bit stays float32 (true 32-bit products
+    for it) instead of becoming bfloat16."""
     config = config_from_dir(model_dir)
     tdtype = parse_dtype(dtype)
     spec = config.to_spec()
     model = DecoderModel(spec)
     ops = ops if ops is not None else default_ops()
-    tensors = load_tensors(model_dir, model.declared(), spec.optional_tensors, tdtype, ops.device)
+    tensors = load_tensors(model_dir, model.declared(), spec.optional_tensors, tdtype, ops.device,
+                           keep_float32)
     model.bind(tensors, ops, tdtype)
     engine = Engine(model, ops, tdtype, max_tokens, max_slots=max_slots, use_graphs=use_graphs)
     engine.config = config
@@ -47,10 +51,12 @@ def load_engine(model_dir: str, dtype="bfloat16", max_tokens: int = 8192, ops=No
 
 
 def random_engine(config, seed: int = 0, dtype="bfloat16", max_tokens: int = 8192, ops=None,
-                  max_slots: Optional[int] = None, use_graphs: bool = True, std: float = 0.02) -> Engine:
+                  max_slots: Optional[int] = None, use_graphs: bool = True, std: float = 0.02,
+                  stored: torch.dtype = torch.bfloat16) -> Engine:
     """The random-weights mode without a file: every tensor the model declares is drawn on the
     device from ``seed`` (matrices normal with ``std``, norm scales 1) and bound as a loaded file
-    would be.  ``config`` is a typed configuration."""
+    would be that stores ``stored`` (float32: full significands for the 32-bit path).  ``config``
+    is a typed configuration."""
     tdtype = parse_dtype(dtype)
     spec = config.to_spec()
     model = DecoderModel(spec)
@@ -58,7 +64,7 @@ def random_engine(config, seed: int = 0, dtype="bfloat16", max_tokens: int = 819
     declared = model.declared()
     tensors = {}
     for name in sorted(declared):
-        t = random_tensors({name: declared[name]}, seed, std=std, dtype=torch.bfloat16,
+        t = random_tensors({name: declared[name]}, seed, std=std, dtype=stored,
                            device=ops.device)[name]
         tensors[name] = place(t, declared[name], tdtype, ops.device)
     model.bind(tensors, ops, tdtype)

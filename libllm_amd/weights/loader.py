@@ -4,9 +4,14 @@ The reference asks its tensor dictionary for each name with the expected shape a
 first mismatch (src/libllm/var_builder.cc:113-125, src/flint/tensor.cc:228-272).  Here the model
 first declares every tensor it needs; the file is compared with the declaration as a whole.
 
-Storage on the device: a matrix stays in bfloat16 (half precision files are converted), a tensor
-stored in 32-bit stays in 32-bit, integer tables become int32, small per-channel vectors are held
-in float32; with dtype float32 every floating tensor is widened to 32-bit.
+Storage on the device: with dtype bfloat16 every matrix becomes bfloat16, whatever float type the
+file stores (the reference casts every float tensor to its device's float type,
+src/libllm/var_builder.cc:113-125), so that every product runs on the matrix cores and a 32-bit
+file costs no more memory than a 16-bit one; small per-channel vectors (norm scales, biases) are
+held in float32, which is how a vector stored in 32-bit stays so; integer tables become int32.
+With ``keep_float32`` a matrix stored in 32-bit or wider stays float32 in bfloat16 mode too, and
+its products then run in true 32-bit.  With dtype float32 every floating tensor is widened to
+32-bit and nothing is rounded on the way.
 """
 import fnmatch
 from typing import Dict, Iterable
@@ -63,31 +68,33 @@ def check_tensors(entries: Dict[str, TensorEntry], expected: Dict[str, WeightDec
     raise err
 
 
-def device_dtype(decl: WeightDecl, stored: torch.dtype, model_dtype: torch.dtype) -> torch.dtype:
+def device_dtype(decl: WeightDecl, stored: torch.dtype, model_dtype: torch.dtype,
+                 keep_float32: bool = False) -> torch.dtype:
     if decl.role == "table":
         return torch.int32
     if decl.role == "vector" or model_dtype == torch.float32:
         return torch.float32
-    if stored in (torch.float32, torch.float64):
-        return torch.float32               # a tensor stored in 32-bit stays so
+    if keep_float32 and stored in (torch.float32, torch.float64):
+        return torch.float32
     return torch.bfloat16
 
 
-def place(t: torch.Tensor, decl: WeightDecl, model_dtype: torch.dtype, device) -> torch.Tensor:
-    target = device_dtype(decl, t.dtype, model_dtype)
+def place(t: torch.Tensor, decl: WeightDecl, model_dtype: torch.dtype, device,
+          keep_float32: bool = False) -> torch.Tensor:
+    target = device_dtype(decl, t.dtype, model_dtype, keep_float32)
     if decl.role == "table" and t.numel() and (int(t.max()) > 2**31 - 1 or int(t.min()) < -2**31):
         raise WeightError("an integer table holds values outside the int32 range")
     return t.to(device=device, dtype=target, copy=True).contiguous()
 
 
 def load_tensors(model_dir: str, expected: Dict[str, WeightDecl], optional: Iterable[str],
-                 model_dtype: torch.dtype, device) -> Dict[str, torch.Tensor]:
+                 model_dtype: torch.dtype, device, keep_float32: bool = False) -> Dict[str, torch.Tensor]:
     entries = open_model_files(model_dir)
     check_tensors(entries, expected, optional)
     out = {}
     for name, decl in expected.items():
         e = entries[name]
-        out[name] = place(e.file.tensor(name), decl, model_dtype, device)
+        out[name] = place(e.file.tensor(name), decl, model_dtype, device, keep_float32)
     for f in {e.file for e in entries.values()}:
         f.close()
     return out

@@ -6,16 +6,30 @@ from libllm_amd.parts import CacheNeed, KVView, StepContext
 
 PAGE = 64
 
-# Bounds on max|out - ref| / mean|ref| (the reference's metric, src/libllm/llama_test.cc:109-130).
+# Bounds on max|out - ref| / mean|ref| (the reference's metric, src/libllm/llama_test.cc:109-130)
+# and, per position, on the relative L2 error of the logits row.
+#
 # float32: only the order of additions differs from the float64 oracle.
 TOL_F32 = 1e-4
-# bfloat16 keeps 8 bits of mantissa where the reference's half keeps 11, so its own bound for half
-# (0.02, src/libllm/llama_test.cc:49) scales by 2^3.
-TOL_BF16 = 0.16
-# Per position, the relative L2 error of the logits row.  A bfloat16 rounding is 2^-9 relative and
-# a logit has passed some tens of them, so a row is off by about one percent; a lost key, a wrong
-# page or a position off by one moves the affected rows by far more.
 ROW_F32 = 2e-5
+#
+# bfloat16, against the plain implementation: the bound is a formula, not a constant.  The plain
+# implementation runs a second time with every tensor that an engine stores between two operators
+# rounded to bfloat16 (``plain.llama.logits_all(..., store=to_bfloat16)``): an engine that computes
+# every sum exactly and stores in bfloat16.  Its distance from the exact logits, in the same two
+# metrics, is what bfloat16 costs for these weights and these tokens; it grows with the spread of
+# the weights times the root of the width (peaked softmax, large SiLU arguments) and differs from
+# position to position.  A correct engine rounds at slightly other places (probabilities, the
+# products that are added into the stream, a norm's scale before or after the rounding), so its
+# error is another draw of the same size: measured ratios of engine error to this model's error
+# are 0.95 to 1.5 (kernels emulated on the CPU) and up to 1.6 (GPU, the traces of the tests).
+# The bound is BF16_MARGIN times the model's error of the same request.
+BF16_MARGIN = 2.0
+# bfloat16 without such a model (one engine against another, toy parts with references of their
+# own): constants for the tiny configurations, widths up to 192 at a spread of 0.08.  bfloat16 keeps
+# 8 bits of significand where the reference's half keeps 11, so its bound for half (0.02,
+# src/libllm/llama_test.cc:49) scales by 2^3; a row has passed some tens of roundings of 2^-9.
+TOL_BF16 = 0.16
 ROW_BF16 = 0.05
 
 
@@ -40,10 +54,35 @@ def row_tol_for(dtype):
     return ROW_F32 if dtype in ("float32", torch.float32) else ROW_BF16
 
 
-def assert_logits_close(out, ref, dtype, what=""):
+def bounds(dtype, ref=None, rounded=None):
+    """(bound on the max metric, bound on the row metric).  ``rounded``: the plain
+    implementation's logits for the same tokens with stored tensors rounded to bfloat16."""
+    if dtype in ("float32", torch.float32) or rounded is None:
+        return tol_for(dtype), row_tol_for(dtype)
+    return BF16_MARGIN * rel_err(rounded, ref), BF16_MARGIN * row_err(rounded, ref)
+
+
+def assert_logits_close(out, ref, dtype, what="", rounded=None):
     e, r = rel_err(out, ref), row_err(out, ref)
-    assert e < tol_for(dtype) and r < row_tol_for(dtype), "%s: max error %.3g, row error %.3g" % (what, e, r)
+    tol, row_tol = bounds(dtype, ref, rounded)
+    assert e < tol and r < row_tol, "%s: max error %.3g (bound %.3g), row error %.3g (bound %.3g)" % (
+        what, e, tol, r, row_tol)
     return e, r
+
+
+def assert_clear_argmax_agrees(out, ref, row_tol, what=""):
+    """The predicted token matches wherever the oracle leaves no doubt
+    (src/libllm/llama_test.cc:182-187 asks it everywhere, of a half-precision engine against a
+    float32 one): at positions where the oracle's first logit leads its second by more than eight
+    times the error that ``row_tol`` allows an element (row_tol * |row| / sqrt(vocab))."""
+    ref = np.asarray(ref, dtype=np.float64)
+    top2 = np.sort(ref, axis=-1)[:, -2:]
+    sigma = row_tol * np.linalg.norm(ref, axis=-1) / np.sqrt(ref.shape[-1])
+    clear = (top2[:, 1] - top2[:, 0]) > 8.0 * sigma
+    got, want = np.asarray(out).argmax(-1), ref.argmax(-1)
+    assert (got[clear] == want[clear]).all(), "%s: arg-max differs at positions %s" % (
+        what, np.nonzero(clear & (got != want))[0][:8].tolist())
+    return int(clear.sum())
 
 
 def make_ctx(ops, dtype, seqs):

@@ -166,52 +166,62 @@ def fused_qkv(weights, prefix):
     return w, b
 
 
-def attention_block(cfg, weights, layer, x, positions):
-    """x [T, H] normed input -> [T, H]  (src/libllm/llama.cc:178-225)."""
+def exact(x):
+    """The default of ``store``: nothing is rounded."""
+    return x
+
+
+def attention_block(cfg, weights, layer, x, positions, store=exact):
+    """x [T, H] normed input -> [T, H]  (src/libllm/llama.cc:178-225).  ``store`` is applied
+    wherever the reference keeps a tensor in its device float type between two operators (its
+    operators return tensors of that type, src/flint/functional.cc:205-207): the model of an
+    engine that computes exactly and stores in reduced precision, used to size error bounds."""
     p = "model.layers.%d.self_attn." % layer
     t = x.shape[0]
     wqkv, bqkv = fused_qkv(weights, p)
-    qkv = linear(x, wqkv, bqkv)
+    qkv = store(linear(x, wqkv, bqkv))
     qd, kd = cfg.n_heads * cfg.head_dim, cfg.n_kv * cfg.head_dim
     q = qkv[:, :qd].reshape(t, cfg.n_heads, cfg.head_dim)
     k = qkv[:, qd:qd + kd].reshape(t, cfg.n_kv, cfg.head_dim)
     v = qkv[:, qd + kd:qd + 2 * kd].reshape(t, cfg.n_kv, cfg.head_dim)
     cos, sin = rope_table(positions, rope_inv_freq(cfg.head_dim, cfg.theta, cfg.scaling))
-    q = apply_rope(q, cos, sin)
-    k = apply_rope(k, cos, sin)
+    q = store(apply_rope(q, cos, sin))
+    k = store(apply_rope(k, cos, sin))
     o = attention(q.transpose(1, 0, 2), k.transpose(1, 0, 2), v.transpose(1, 0, 2), True)
-    o = o.transpose(1, 0, 2).reshape(t, qd)
-    return linear(o, weights[p + "o_proj.weight"])
+    o = store(o.transpose(1, 0, 2).reshape(t, qd))
+    return store(linear(o, weights[p + "o_proj.weight"]))
 
 
-def mlp(cfg, weights, layer, x):
+def mlp(cfg, weights, layer, x, store=exact):
     """down(swiglu(gate_up(x))), gate rows first (src/libllm/llama.cc:92-98,
     tools/llama_exporter.py:73-78)."""
     p = "model.layers.%d.mlp." % layer
     wgu = np.concatenate([weights[p + "gate_proj.weight"], weights[p + "up_proj.weight"]], axis=0)
-    return linear(swiglu(linear(x, wgu)), weights[p + "down_proj.weight"])
+    h = store(swiglu(store(linear(x, wgu))))
+    return store(linear(h, weights[p + "down_proj.weight"]))
 
 
-def decode_layer(cfg, weights, layer, x, positions):
-    """Pre-norm residual block (src/libllm/llama.cc:251-267)."""
+def decode_layer(cfg, weights, layer, x, positions, store=exact):
+    """Pre-norm residual block (src/libllm/llama.cc:251-267).  The running sum itself is not
+    passed through ``store``: the bounds are for engines that keep it in 32-bit."""
     p = "model.layers.%d." % layer
     residual = x
-    h = rms_norm(x, weights[p + "input_layernorm.weight"], cfg.eps)
-    h = attention_block(cfg, weights, layer, h, positions)
+    h = store(rms_norm(x, weights[p + "input_layernorm.weight"], cfg.eps))
+    h = attention_block(cfg, weights, layer, h, positions, store)
     x = h + residual
     residual = x
-    h = rms_norm(x, weights[p + "post_attention_layernorm.weight"], cfg.eps)
-    h = mlp(cfg, weights, layer, h)
+    h = store(rms_norm(x, weights[p + "post_attention_layernorm.weight"], cfg.eps))
+    h = mlp(cfg, weights, layer, h, store)
     return h + residual
 
 
-def hidden_states(cfg, weights, ids, position_offset=0):
+def hidden_states(cfg, weights, ids, position_offset=0, store=exact):
     """Embedding, layers, final norm (src/libllm/llama.cc:294-303)."""
     x = embedding(weights["model.embed_tokens.weight"], ids)
     positions = np.arange(len(ids)) + position_offset
     for layer in range(cfg.n_layers):
-        x = decode_layer(cfg, weights, layer, x, positions)
-    return rms_norm(x, weights["model.norm.weight"], cfg.eps)
+        x = decode_layer(cfg, weights, layer, x, positions, store)
+    return store(rms_norm(x, weights["model.norm.weight"], cfg.eps))
 
 
 def lm_head(cfg, weights, h):
@@ -220,7 +230,15 @@ def lm_head(cfg, weights, h):
     return linear(h, w)
 
 
-def logits_all(cfg, weights, ids, position_offset=0):
+def logits_all(cfg, weights, ids, position_offset=0, store=exact):
     """Logits at every position of one whole sequence: [T, V]
     (the forwardAll of src/libllm/llama_test.cc:92-97)."""
-    return lm_head(cfg, weights, hidden_states(cfg, weights, ids, position_offset))
+    return lm_head(cfg, weights, hidden_states(cfg, weights, ids, position_offset, store))
+
+
+def to_bfloat16(x):
+    """Rounds to the nearest value with 8 bits of significand, ties to even: what storing a
+    float32 result as bfloat16 does (the upper 16 bits of the float32 pattern)."""
+    bits = np.ascontiguousarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    bits = ((bits + 0x7FFF + ((bits >> 16) & 1)) >> 16) << 16
+    return bits.astype(np.uint32).view(np.float32).astype(np.float64).reshape(np.shape(x))

@@ -836,6 +836,30 @@ def test_attention_decode_over_many_pages(ops, ctx_len, far):
     assert max_err(out, ref) < BF16_2ULP
 
 
+def test_a_build_whose_product_for_65_to_128_rows_spills_does_not_use_it(monkeypatch):
+    """The build's record decides (see test_build.py): with a spill on record the host sends
+    steps of 65 to 128 rows to the library's product."""
+    from libllm_amd.hip import HipOps, build
+    assert HipOps().mid_gemm
+    monkeypatch.setattr(build, "trusted", lambda source, path=None: False)
+    other = HipOps()
+    assert not other.mid_gemm
+    x, w = rnd((100, 256), torch.bfloat16, 1).cuda(), rnd((3200, 256), torch.bfloat16, 2).cuda()
+    assert not other._mid_ok(x, other.prepare_weight(w), 100, 256)
+
+
+@pytest.mark.parametrize("hd", [160, 192, 256])
+@pytest.mark.parametrize("ctx_len,far", [(600, 3), (2100, 1999), (9000, 77)])
+def test_attention_decode_of_wide_heads_over_many_pages(ops, hd, ctx_len, far):
+    """Heads wider than 128: the decode kernel's form of two waves a block, and each form of the
+    merge (up to 8 partials, up to 32, and the loop, whose block must stay within 1,024 threads:
+    four groups of 192 or 256 threads, not eight).  One far key dominates."""
+    out, ref = run_attention(ops, torch.bfloat16, 4, 2, hd, [(0, ctx_len, 1)], seed=hd, boost=(far, 12.0))
+    assert max_err(out, ref) < BF16_2ULP
+    out, ref = run_attention(ops, torch.bfloat16, 2, 1, hd, [(1, ctx_len - 70, 1), (0, ctx_len, 1)], seed=hd + 1)
+    assert max_err(out, ref) < BF16_2ULP
+
+
 @pytest.mark.parametrize("hd", [64, 128])
 @pytest.mark.parametrize("blocks", [1, 3, 4096])
 def test_attention_decode_pages_of_a_wave(ops, monkeypatch, hd, blocks):

@@ -11,9 +11,10 @@ import sys
 
 import numpy as np
 import pytest
+import torch
 
 import traces
-from helpers import assert_logits_close
+from helpers import assert_clear_argmax_agrees, assert_logits_close, bounds
 from plain import files, llama
 from tiny import TINY_A, TINY_B, TINY_C, make_model
 
@@ -44,10 +45,12 @@ def make_requests(cfg, lengths, seed):
 _oracle_cache = {}
 
 
-def oracle(name, cfg, weights, toks):
-    key = (name, tuple(toks))
+def oracle(name, cfg, weights, toks, rounded=False):
+    """The plain implementation's logits at every position; ``rounded``: with stored tensors
+    rounded to bfloat16 (the model of bfloat16's cost that the bounds are sized by)."""
+    key = (name, tuple(toks), rounded)
     if key not in _oracle_cache:
-        _oracle_cache[key] = llama.logits_all(cfg, weights, toks)
+        _oracle_cache[key] = llama.logits_all(cfg, weights, toks, store=llama.to_bfloat16 if rounded else llama.exact)
     return _oracle_cache[key]
 
 
@@ -69,19 +72,21 @@ WORST = {}
 
 
 def check(name, cfg, weights, requests, got, dtype):
-    worst = WORST.get(dtype, 0.0)
+    """Every position of every request against the plain implementation: both metrics within
+    their bounds (helpers.bounds), and the arg-max wherever the oracle's margin is clear."""
+    worst = WORST.get(dtype, (0.0, 0.0))
     for rid, toks in requests.items():
         ref = oracle(name, cfg, weights, toks)
+        rounded = oracle(name, cfg, weights, toks, rounded=True) if dtype == "bfloat16" else None
         assert sorted(got[rid]) == list(range(len(toks))), "positions of %s" % rid
         out = np.stack([got[rid][p] for p in range(len(toks))])
-        err, row = assert_logits_close(out, ref, dtype, "%s %s %s" % (name, dtype, rid))
-        worst = max(worst, row)
-        # arg-max agrees wherever the oracle's margin exceeds the error (src/libllm/llama_test.cc:182-187)
-        top2 = np.sort(ref, axis=-1)[:, -2:]
-        clear = (top2[:, 1] - top2[:, 0]) > 2 * np.abs(out - ref).max(axis=-1)
-        assert (out.argmax(-1)[clear] == ref.argmax(-1)[clear]).all()
+        what = "%s %s %s" % (name, dtype, rid)
+        err, row = assert_logits_close(out, ref, dtype, what, rounded)
+        tol, row_tol = bounds(dtype, ref, rounded)
+        assert_clear_argmax_agrees(out, ref, row_tol, what)
+        worst = (max(worst[0], err / tol), max(worst[1], row / row_tol))
     WORST[dtype] = worst
-    print("worst row error so far (%s): %.3g" % (dtype, worst))
+    print("largest fraction of a bound used so far (%s): max metric %.2f, row metric %.2f" % ((dtype,) + worst))
     return worst
 
 
@@ -152,6 +157,57 @@ def test_first_tokens(models, tmp_path, dtype):
         check(name, cfg, weights, requests, traces.collect(steps, str(out_dir), cfg.vocab), dtype)
 
 
+def _is_matrix(name, arr):
+    return arr.ndim == 2
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("name,stored", [("A", "float32"), ("B", "float32"), ("C", "float16")])
+def test_files_of_other_float_types(tmp_path, name, stored, dtype):
+    """Model files that store float32 (full significands, jittered norm scales) or float16.  The
+    32-bit engine must keep every bit of them: a path that rounded a weight, a norm scale or a bias
+    to bfloat16 between the file and a kernel would be a thousand times beyond the 32-bit bound.
+    The bfloat16 engine must turn every matrix into bfloat16 at load, as the reference casts every
+    float tensor to its device's type (src/libllm/var_builder.cc:113-125), keep the vectors in
+    32-bit, and run the matrix-core products: it is compared with the plain implementation on
+    matrices rounded the same way."""
+    from libllm_amd.hip.ops import PreparedWeight
+    path = make_model(tmp_path, CONFIGS[name], seed=23, name=name + stored, stored=stored)
+    cfg_json, weights = files.read_model_dir(path)
+    cfg = llama.PlainConfig(cfg_json)
+    assert any(np.any(w != llama.to_bfloat16(w)) for w in weights.values())     # the file needs more than bfloat16
+    if dtype == "bfloat16":
+        weights = {n: llama.to_bfloat16(w) if _is_matrix(n, w) else w for n, w in weights.items()}
+    requests = make_requests(cfg, [70, 9, 100, 33, 1], seed=31)
+    steps = traces.batches([requests], {r: min(8, len(t) - 1) for r, t in requests.items()})
+    engine = run_replay(path, dtype, steps, tmp_path / dtype)
+    tag = name + stored + dtype
+    check(tag, cfg, weights, requests, traces.collect(steps, str(tmp_path / dtype), cfg.vocab), dtype)
+    for block in engine.model.blocks:
+        for lin in (block.mixer.qkv, block.mixer.out, block.feed_forward.gate_up, block.feed_forward.down):
+            if dtype == "bfloat16":
+                assert isinstance(lin.prepared, PreparedWeight) and lin.weight.dtype == torch.bfloat16
+            else:
+                assert lin.weight.dtype == torch.float32
+        assert all(n.weight.dtype == torch.float32 for n in block.norms)
+
+
+def test_matrices_kept_in_32_bit_on_request(tmp_path):
+    """``keep_float32``: in bfloat16 mode the matrices of a float32 file stay float32 and their
+    products run in true 32-bit; activations and the cache are bfloat16 all the same."""
+    from libllm_amd.engine.trace import replay
+    from libllm_amd.runtime import load_engine
+    path = make_model(tmp_path, CONFIGS["A"], seed=24, name="kept", stored="float32")
+    cfg_json, weights = files.read_model_dir(path)
+    cfg = llama.PlainConfig(cfg_json)
+    requests = make_requests(cfg, [40, 7, 66], seed=32)
+    steps = traces.batches([requests], {r: 4 for r in requests})
+    engine = load_engine(path, dtype="bfloat16", max_tokens=traces.max_tokens_needed(steps), keep_float32=True)
+    assert engine.model.blocks[0].mixer.qkv.weight.dtype == torch.float32
+    replay(engine, traces.lines(steps), str(tmp_path / "out"), log=io.StringIO())
+    check("kept", cfg, weights, requests, traces.collect(steps, str(tmp_path / "out"), cfg.vocab), "bfloat16")
+
+
 @pytest.fixture(scope="module")
 def long_models(tmp_path_factory):
     """The tiny configurations with position limits beyond a thousand, so that one request of a
@@ -208,11 +264,12 @@ def random_trace(rng, cfg):
     return steps, requests
 
 
-@pytest.mark.parametrize("case", range(12))
+@pytest.mark.parametrize("case", range(66))
 def test_random_traces(long_models, tmp_path, case):
     """Drawn batches, cuts and cache sizes (see random_trace) in both dtypes, with and without
-    captured graphs, every position of every request against the plain implementation."""
-    name, dtype, use_graphs = "ABC"[case % 3], DTYPES[(case // 3) % 2], case < 9
+    captured graphs (every fourth group of six without), every position of every request against
+    the plain implementation."""
+    name, dtype, use_graphs = "ABC"[case % 3], DTYPES[(case // 3) % 2], (case // 6) % 4 != 3
     path, cfg, weights = long_models[name]
     rng = np.random.default_rng(1000 + case)
     steps, requests = random_trace(rng, cfg)
@@ -274,6 +331,24 @@ ODD = {
     "one layer, one head": dict(num_hidden_layers=1, hidden_size=16, num_attention_heads=1, num_key_value_heads=1,
                                 intermediate_size=8, vocab_size=9),
     "feed-forward of one, vocabulary 70001": dict(intermediate_size=1, vocab_size=70001),
+    "width 72, a multiple of 8 only": dict(hidden_size=72, num_attention_heads=3, num_key_value_heads=1, head_dim=32,
+                                          intermediate_size=88, vocab_size=33),
+    "width 66, a multiple of 2 only": dict(hidden_size=66, intermediate_size=90, vocab_size=77),
+    "head size 96": dict(hidden_size=96, num_attention_heads=3, num_key_value_heads=3, head_dim=96),
+    "head size 8": dict(hidden_size=32, num_attention_heads=4, num_key_value_heads=2, head_dim=8),
+    "a group of 8 heads": dict(hidden_size=128, num_attention_heads=16, num_key_value_heads=2),
+    # Widths that are multiples of 8 and not of 32 or 16: the skinny product's last step of K is
+    # short, the SwiGLU epilogue is not taken, the library's products run at 65 rows and more.  At
+    # the tests' spread of 0.08 a row of 2,056 columns gives products of spread 3.6: the softmax
+    # is sharply peaked and bfloat16 costs six times what it costs the tiny configurations (the
+    # plain implementation with stored tensors rounded to bfloat16 is 0.078 off in the row metric
+    # and 0.32 in the max metric, where Tiny A is 0.012 and 0.05 off).  The bounds follow that.
+    "width 2056, feed-forward 8200": dict(hidden_size=2056, num_attention_heads=8, num_key_value_heads=4, head_dim=64,
+                                          intermediate_size=8200, vocab_size=500),
+    # the same at a spread of 0.02 (products of spread 0.9): bfloat16 costs what it costs Tiny A,
+    # and the bounds are as tight as there
+    "width 2056, feed-forward 8200, spread 0.02": dict(hidden_size=2056, num_attention_heads=8, num_key_value_heads=4,
+                                                       head_dim=64, intermediate_size=8200, vocab_size=500, spread=0.02),
 }
 
 
@@ -282,7 +357,7 @@ def test_odd_sizes_end_to_end(tmp_path, what):
     """Sizes that a configuration may have and no released model has, through the whole engine in
     both dtypes: a batch of up to 18 unequal prompts, then six tokens each."""
     cfg_dict = dict(TINY_A, max_position_embeddings=512, **ODD[what])
-    path = make_model(tmp_path, cfg_dict, seed=len(what), name="odd")
+    path = make_model(tmp_path, cfg_dict, seed=len(what), name="odd", std=cfg_dict.pop("spread", 0.08))
     cfg_json, weights = files.read_model_dir(path)
     cfg = llama.PlainConfig(cfg_json)
     lengths = [70, 9, 131, 20, 1, 64, 33, 200, 5, 17, 90, 40, 3, 66, 128, 12, 7, 100]
@@ -360,9 +435,9 @@ def test_norms_between_products_get_no_kernel(models, name):
     assert calls["folded"] == prompt + 4 * 2
     assert_logits_close(a, b.astype(np.float64), "bfloat16", "folded norms against norm kernels")
     for i, (rid, toks) in enumerate(requests.items()):
-        ref = oracle(name, cfg, weights, toks)
-        for step in range(4):                                   # step s fed token -(4 - s): logits at that position
-            assert_logits_close(a[step, i][None], ref[len(toks) - 4 + step][None], "bfloat16", "%s step %d" % (rid, step))
+        ref, rounded = oracle(name, cfg, weights, toks), oracle(name, cfg, weights, toks, rounded=True)
+        rows = slice(len(toks) - 4, len(toks))                  # step s fed token -(4 - s): logits at that position
+        assert_logits_close(a[:, i], ref[rows], "bfloat16", rid, rounded[rows])
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -418,7 +493,7 @@ def test_prompt_steps_through_graphs(models, name, dtype):
                 assert torch_equal(a, b), "round %d step %d" % (rnd, k)
             for j, e in enumerate(entries):
                 upto = (lengths[e.request] if k == 1 else lengths[e.request] + k - 1)
-                want = oracle(name, cfg, weights, toks[e.request][:upto])[-1]
+                want = oracle(name, cfg, weights, toks[e.request])[upto - 1]
                 assert_logits_close(a[j].cpu().numpy()[None], want[None], dtype, "round %d step %d" % (rnd, k))
         eng.end(list(toks)); ref.end(list(toks))
     assert eng._prompt_graphs and not ref._prompt_graphs

@@ -16,9 +16,9 @@ from plain import files
 from tiny import TINY_A, TINY_B, TINY_C, make_model
 
 
-def load(path, cfg, dtype):
+def load(path, cfg, dtype, keep_float32=False):
     model = DecoderModel(config_from_dict(cfg).to_spec())
-    return load_tensors(path, model.declared(), model.spec.optional_tensors, dtype, "cpu")
+    return load_tensors(path, model.declared(), model.spec.optional_tensors, dtype, "cpu", keep_float32)
 
 
 def rewrite(path, change):
@@ -53,13 +53,24 @@ def test_storage_dtypes(tmp_path):
     t32 = load(path, TINY_A, torch.float32)
     assert all(v.dtype == torch.float32 for v in t32.values())
     assert torch.equal(t32["model.embed_tokens.weight"], t["model.embed_tokens.weight"].float())
-    # a matrix stored in 32-bit stays so; one stored in half precision becomes bfloat16
+    # in bfloat16 mode every matrix becomes bfloat16, rounded to nearest, whatever the file stores
+    # (src/libllm/var_builder.cc:113-125); in float32 mode nothing is rounded; with keep_float32
+    # a matrix stored in 32-bit stays so
+    wide = t32["model.layers.0.mlp.down_proj.weight"] + 1e-4
     rewrite(path, lambda ts: ts.update({
-        "model.layers.0.mlp.down_proj.weight": ts["model.layers.0.mlp.down_proj.weight"].float() + 1e-4,
-        "model.layers.1.mlp.down_proj.weight": ts["model.layers.1.mlp.down_proj.weight"].half()}))
+        "model.layers.0.mlp.down_proj.weight": wide,
+        "model.layers.1.mlp.down_proj.weight": ts["model.layers.1.mlp.down_proj.weight"].half(),
+        "model.norm.weight": ts["model.norm.weight"].float() + 1e-4}))
     t = load(path, TINY_A, torch.bfloat16)
-    assert t["model.layers.0.mlp.down_proj.weight"].dtype == torch.float32
+    assert t["model.layers.0.mlp.down_proj.weight"].dtype == torch.bfloat16
+    assert torch.equal(t["model.layers.0.mlp.down_proj.weight"], wide.to(torch.bfloat16))
     assert t["model.layers.1.mlp.down_proj.weight"].dtype == torch.bfloat16
+    assert t["model.norm.weight"].dtype == torch.float32                 # a vector stored in 32-bit keeps its bits
+    assert float((t["model.norm.weight"] - 1.0).abs().min()) > 0
+    assert torch.equal(load(path, TINY_A, torch.float32)["model.layers.0.mlp.down_proj.weight"], wide)
+    kept = load(path, TINY_A, torch.bfloat16, keep_float32=True)
+    assert torch.equal(kept["model.layers.0.mlp.down_proj.weight"], wide)
+    assert kept["model.layers.1.mlp.down_proj.weight"].dtype == torch.bfloat16
 
 
 def test_one_error_lists_everything(tmp_path):

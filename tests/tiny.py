@@ -31,12 +31,15 @@ TINY_C = {
 }
 
 
-def make_model(tmpdir, cfg_dict, seed=0, std=0.08, norm_std=0.2, name="model"):
+def make_model(tmpdir, cfg_dict, seed=0, std=0.08, norm_std=0.2, name="model", stored="bfloat16"):
     """Writes a model folder through the library's random-weights mode.  The spread of the
     weights is wider than the usual 0.02 so that attention is far from uniform, and norm scales
-    are jittered so that a missing scale shows."""
+    are jittered so that a missing scale shows.  ``stored``: the float type the file holds
+    ("float32": full significands, which no 16-bit type can carry)."""
+    import torch
     from libllm_amd.config import config_from_dict
     from libllm_amd.weights import write_random_model
     path = os.path.join(str(tmpdir), name)
-    write_random_model(path, config_from_dict(cfg_dict), seed=seed, std=std, norm_std=norm_std)
+    write_random_model(path, config_from_dict(cfg_dict), seed=seed, std=std, norm_std=norm_std,
+                       dtype=getattr(torch, stored))
     return path
