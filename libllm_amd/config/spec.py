@@ -44,10 +44,14 @@ class EmbeddingSpec:
 
 @dataclass
 class HeadSpec:
+    """The output layer.  ``kind`` names the registered class that turns the normalised wanted
+    rows into logits ("linear": a bare matrix product); one with a bias, a scale or a cap on the
+    logits is another kind with a record of its own that extends this one."""
     vocab: int
     width: int
     tensor: str                         # tensor name of the output matrix (the table's, if tied)
     tied: bool = False
+    kind: str = "linear"
 
 
 @dataclass

@@ -670,19 +670,6 @@ extern "C" int llm_attention_mfma_supported(int hd) {
   return 0;
 }
 
-static int compute_units() {
-  static int units = 0;                     // of the current device, asked once
-  if (units == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) == hipSuccess &&
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-      units = n;
-    else
-      units = 256;
-  }
-  return units;
-}
-
 static bool attn_args_ok(const void* q, int q_stride, const void* k, const void* v, int n_heads,
                          int n_kv, int hd, int window) {
   if (n_heads <= 0 || n_kv <= 0 || n_heads % n_kv || window < 0) return false;
@@ -743,7 +730,7 @@ extern "C" int llm_attention_decode_bf16(const void* q, int q_stride, const void
   const float scale_log2 = scale * 1.4426950408889634f;
   dim3 grid(n_blocks, n_kv, n_seqs);
   // pages overlapped within a wave where all blocks are resident at two a compute unit
-  const bool ahead = hd <= 128 && (long long)n_blocks * n_kv * n_seqs <= 2LL * compute_units();
+  const bool ahead = hd <= 128 && (long long)n_blocks * n_kv * n_seqs <= 2LL * llm_compute_units();
 #define CASE(D)                                                                                   \
   if (hd == D) {                                                                                  \
     constexpr int WAVES = (D > 128) ? 2 : 4;                                                      \

@@ -97,3 +97,17 @@ __device__ __forceinline__ float block_max(float v, float* scratch) {
 static inline int llm_launch_status() {
   return hipGetLastError() == hipSuccess ? LLM_OK : LLM_ERR_LAUNCH;
 }
+
+// Compute units of the current device, asked once (launchers weigh their grids against it).
+static inline int llm_compute_units() {
+  static int units = 0;
+  if (units == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+      units = n;
+    else
+      units = 256;
+  }
+  return units;
+}

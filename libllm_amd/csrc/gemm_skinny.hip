@@ -447,16 +447,20 @@ static int launch_skinny(const SkinnyArgs& a) {
 
 template <int MT, int EPI, typename OutT>
 static int pick_rows(const SkinnyArgs& a) {
+  const int units = llm_compute_units();
   if constexpr (EPI == SK_EPI_SWIGLU) {
-    // four tiles a block pay from 33 rows of X on; at 17 to 32 rows two are 2 % of a decode step
-    // faster (whole engines compared in one process, 1B and 8B shapes)
-    if (a.n_out >= 8192 && MT >= 3) return launch_skinny<MT, 4, 1, 1, EPI, OutT>(a);
+    // four tiles a block (32 output columns) where that still leaves a block for every compute
+    // unit; they pay from 33 rows of X on; at 17 to 32 rows two are 2 % of a decode step faster
+    // (whole engines compared in one process; feed-forwards of 8,192 and 14,336 on 256 units)
+    if (a.n_out >= 32 * units && MT >= 3) return launch_skinny<MT, 4, 1, 1, EPI, OutT>(a);
     return launch_skinny<MT, 2, 1, 1, EPI, OutT>(a);
   } else {
     // slices of K: 64 rows of W a block, so that a slice of X is staged for as many as possible
     if (a.k_split > 1) return launch_skinny<MT, 2, 2, 1, EPI, OutT>(a);
-    if (a.N >= 8192) return launch_skinny<MT, 2, 2, 1, EPI, OutT>(a);
-    if (a.N >= 6144) return launch_skinny<MT, 2, 1, 1, EPI, OutT>(a);
+    // else as many rows of W a block (64, 32, 16) as leave blocks for half of the compute units,
+    // for three quarters, or whatever there is (measured at 8,192, 6,144 and fewer rows on 256 units)
+    if (a.N >= 32 * units) return launch_skinny<MT, 2, 2, 1, EPI, OutT>(a);
+    if (a.N >= 24 * units) return launch_skinny<MT, 2, 1, 1, EPI, OutT>(a);
     return launch_skinny<MT, 1, 1, 1, EPI, OutT>(a);
   }
 }
@@ -467,11 +471,11 @@ static int pick_shape(const SkinnyArgs& a) {
   const int mt = (a.M + 15) / 16;
   switch (mt) {
     case 1:
-      // few rows of W (so few blocks): more of each row in flight per wave.  Whole engines compared
-      // in one process: 1 to 1.5 % of a decode step at the 1B shape, nothing lost at 3B and 8B;
-      // for the 6,144 rows of the 8B shape's q|k|v product it costs 2.5 %.
+      // no more tiles of W than compute units (so a block a unit at most): more of each row in
+      // flight per wave.  Whole engines compared in one process on 256 units: 1 to 1.5 % of a decode
+      // step with weights of 2,048 and 3,072 rows, nothing lost at 4,096; at 6,144 rows it costs 2.5 %.
       if constexpr (RT == 1) {
-        if (a.N <= 4096) return launch_skinny<1, RT, 1, 4, EPI, OutT>(a);
+        if (a.N <= 16 * llm_compute_units()) return launch_skinny<1, RT, 1, 4, EPI, OutT>(a);
       }
       // gate/up has more blocks than the chip has compute units: with the narrow chunk a block
       // needs few enough registers for two of them to share a unit, and the tail of one overlaps

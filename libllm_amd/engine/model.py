@@ -10,8 +10,8 @@ import torch
 
 from ..config.spec import ModelSpec, validate_schedule
 from ..errors import ConfigError
-from ..parts import (Stream, StepContext, WeightDecl, build_block, build_feed_forward, build_mixer,
-                     build_norm)
+from ..parts import (Stream, StepContext, WeightDecl, build_block, build_feed_forward, build_head,
+                     build_mixer, build_norm)
 
 
 def _build_layers(spec: ModelSpec):
@@ -43,8 +43,8 @@ class DecoderModel:
         self.spec = spec
         self.blocks = _build_layers(spec)
         self.final_norm = build_norm(spec.final_norm)
+        self.head = build_head(spec.head)
         self.embed_table: Optional[torch.Tensor] = None
-        self.head_weight: Optional[torch.Tensor] = None
         self._decls = None
 
     # ---- weights
@@ -84,10 +84,7 @@ class DecoderModel:
                 if id(part) not in parts:
                     part.bind({}, ops, dtype)
         self.embed_table = tensors[s.embedding.tensor]
-        self.head_weight = self.embed_table if s.head.tied else tensors[s.head.tensor]
-        self.head_prepared = self.head_weight
-        if hasattr(ops, "prepare_weight"):
-            self.head_prepared = ops.prepare_weight(self.head_weight)
+        self.head.bind(self.embed_table if s.head.tied else tensors[s.head.tensor], ops, dtype)
 
     # ---- what the cache has to hold
     def cache_needs(self):
@@ -110,7 +107,7 @@ class DecoderModel:
             for part in [block.mixer, block.feed_forward] + list(block.norms):
                 if not getattr(part, "graph_safe", False):
                     return False
-        return getattr(self.final_norm, "graph_safe", False)
+        return getattr(self.final_norm, "graph_safe", False) and getattr(self.head, "graph_safe", False)
 
     # ---- one step over packed rows
     def forward(self, ctx: StepContext, want_rows: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
@@ -128,8 +125,8 @@ class DecoderModel:
         ctx.norm_after_block = None
         if want_rows is None or want_rows.numel() == 0:
             return None
-        h = self.final_norm.add_norm(ctx, stream, rows=want_rows, lazy=True)
-        return ctx.ops.linear(h, self.head_prepared, None, torch.float32)
+        h = self.final_norm.add_norm(ctx, stream, rows=want_rows, lazy=getattr(self.head, "takes_normed", False))
+        return self.head.forward(ctx, h)
 
 
 def declared_weights(spec: ModelSpec) -> Dict[str, WeightDecl]:

@@ -105,11 +105,14 @@ class HipOps:
     # batches of 96: 3.56 against 4.34, 5.84 against 7.10, 1.72 against 1.82.  For the small o
     # weight of the 1B shape the library's product is as fast (10.2 against 10.4 us): hence the limit.
     MID_ROWS = 128
-    MID_BLOCKS = 256                # blocks that its slices of K aim at (128 and 512 lose 8 to 10 % of a prompt step of 128 tokens at the 3B and 8B shapes: fewer blocks, or more matrices for the norm to add)
-    MID_MIN_WEIGHT = 3072 * 3072    # elements of a weight from which a product that adds into the stream takes it (in slices of K)
-    DECODE_BLOCKS = 768     # blocks of the decode attention grid beyond which sequences are not split further
-    DECODE_BLOCKS_AHEAD = 512   # the same where a wave would get DECODE_AHEAD_PAGES pages or more and the sequences
-    DECODE_AHEAD_PAGES = 6      # fill such a grid: two blocks a compute unit, at which the kernel overlaps a wave's pages
+    # Launch sizes below are in blocks per compute unit; ``__init__`` multiplies them by the
+    # device's number of units (the figures in the comments were measured on 256 units).
+    MID_BLOCKS_PER_UNIT = 1.0       # blocks that the slices of K of the product for 65 to 128 rows aim at (half and twice as many lose 8 to 10 % of a prompt step of 128 tokens at the 3B and 8B shapes: fewer blocks, or more matrices for the norm to add)
+    MID_FILL = 0.75                 # it takes a product that adds into the stream only if slices of at least MID_MIN_SLICE elements of K give it blocks for this share of the units (a 2,048 x 2,048 weight gets 128 blocks: the library's product is as fast, 10.2 against 10.4 us; 3,072 x 3,072 gets 192 and gains)
+    MID_MIN_SLICE = 512
+    DECODE_BLOCKS_PER_UNIT = 3      # blocks of the decode attention grid beyond which sequences are not split further
+    DECODE_BLOCKS_AHEAD_PER_UNIT = 2    # the same where a wave would get DECODE_AHEAD_PAGES pages or more and the sequences
+    DECODE_AHEAD_PAGES = 6              # fill such a grid: two blocks a compute unit, at which the kernel overlaps a wave's pages
     # New rows of the step's longest sequence from which a wave of prompt attention takes two
     # tiles of rows: heads up to 64 wide, up to 128 (wider ones never: one wave a unit would be
     # left).  A block's walk over the pages of its rows is what a short prompt waits for, and two
@@ -135,6 +138,10 @@ class HipOps:
             fn.argtypes = argtypes
             fn.restype = _i
         torch.backends.cuda.matmul.allow_tf32 = False
+        self.units = torch.cuda.get_device_properties(self.device).multi_processor_count
+        self.MID_BLOCKS = max(1, int(self.MID_BLOCKS_PER_UNIT * self.units))
+        self.DECODE_BLOCKS = self.DECODE_BLOCKS_PER_UNIT * self.units
+        self.DECODE_BLOCKS_AHEAD = self.DECODE_BLOCKS_AHEAD_PER_UNIT * self.units
         # switches for tests and measurements; the product runs with all three on
         self.fast_attention = True      # bfloat16 attention on the matrix cores (else the plain kernel, as for float32)
         self.pack_weights = True        # keep a tiled copy of every weight for the skinny product
@@ -315,9 +322,10 @@ class HipOps:
 
     def _k_split_mid(self, n, k):
         """Slices of K for a product of 65 to 128 rows whose result the next norm adds: enough for
-        about MID_BLOCKS blocks at 64 weight rows a block, each at least 256 long and a multiple of 128."""
+        about MID_BLOCKS blocks at 64 weight rows a block, each at least MID_MIN_SLICE long and a
+        multiple of 128."""
         ks = max(1, min(16, self.MID_BLOCKS // max(1, -(-n // 64))))
-        while ks > 1 and (k % (ks * 128) or k // ks < 256):
+        while ks > 1 and (k % (ks * 128) or k // ks < self.MID_MIN_SLICE):
             ks -= 1
         return ks
 
@@ -402,9 +410,8 @@ class HipOps:
         if self._mid_ok(x, w, m, k) and bias is None and out_dtype != torch.float32:
             # (without slices of K, for a product that does not add into the stream, it has too few
             # blocks for the q|k|v weights and loses to the library: 16.7 against 13.0 us at 128 rows)
-            if residual is not None and n * k >= self.MID_MIN_WEIGHT:
+            if residual is not None and (ks := self._k_split_mid(n, k)) * -(-n // 64) >= self.MID_FILL * self.units:
                 # K in slices for enough blocks; the norm kernel that follows adds them, in order
-                ks = self._k_split_mid(n, k)
                 return self._mid(x, w, torch.empty((ks, m, n), dtype=torch.float32, device=self.device),
                                  self._EPI_NONE, ks)
         w = self._plain(w)

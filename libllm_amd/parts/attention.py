@@ -89,15 +89,23 @@ class Attention(Mixer):
         if s.qkv_bias:
             bias = torch.cat([tensors[n + ".bias"] for n in (s.q_name, s.k_name, s.v_name)]).contiguous()
         w = torch.cat(parts, dim=0)                      # q rows, then k, then v
-        # kernels that rotate inside the projection want the two dims of a pair side by side:
-        # reorder the output rows of q and k (and the bias) once; scores do not change, since
-        # queries and keys are reordered alike
-        self.adjacent = bool(getattr(ops, "prefers_adjacent_pairs", False)) and self.position.rot_dim > 0
-        if self.adjacent:
-            order = self._pair_order(w.device)
-            w = w[order]
-            if bias is not None:
-                bias = bias[order].contiguous()
+        # A position encoding pairs dims (j, j + rot_dim/2) ("half", the default) or neighbours
+        # (2j, 2j+1) ("interleaved").  Kernels that rotate inside the projection want the two dims
+        # of a pair side by side: for "half" the output rows of q and k (and the bias) are
+        # reordered once; scores do not change, since queries and keys are reordered alike.
+        pairing = getattr(self.position, "pairing", "half")
+        rotates = self.position.rot_dim > 0
+        if pairing == "interleaved" and rotates:
+            if not getattr(ops, "prefers_adjacent_pairs", False):
+                raise ConfigError("these kernels rotate the halves of a head only (pairing 'interleaved')")
+            self.adjacent = True
+        else:
+            self.adjacent = bool(getattr(ops, "prefers_adjacent_pairs", False)) and rotates
+            if self.adjacent:
+                order = self._pair_order(w.device)
+                w = w[order]
+                if bias is not None:
+                    bias = bias[order].contiguous()
         self.qkv.bind(w, ops=ops)
         self.q_only.bind(self.qkv.weight[:self.q_dim], ops=ops, like=self.qkv.prepared)    # the same storage
         self.bias = bias                                 # added inside the rotation kernel
@@ -127,7 +135,8 @@ class Attention(Mixer):
         else:
             qkv = proj(ctx, x)
             ctx.ops.rope_kv_write(qkv, self.bias, s.n_heads, s.n_kv_heads, s.head_dim, self.cos,
-                                  self.sin, self.position.rot_dim, ctx, kv, entry.writes)
+                                  self.sin, self.position.rot_dim, ctx, kv, entry.writes,
+                                  **({"adjacent": True} if self.adjacent else {}))
         o = ctx.ops.attention(qkv, s.n_heads, s.n_kv_heads, s.head_dim, ctx, kv,
                               self.scale, s.window)
         return self.out(ctx, o, residual=residual)

@@ -16,6 +16,7 @@ _FEED_FORWARDS: Dict[str, Callable] = {}
 _NORMS: Dict[str, Callable] = {}
 _POSITIONS: Dict[str, Callable] = {}
 _BLOCKS: Dict[str, Callable] = {}
+_HEADS: Dict[str, Callable] = {}
 
 
 def _register(table, what):
@@ -42,9 +43,11 @@ register_feed_forward = _register(_FEED_FORWARDS, "feed-forward")
 register_norm = _register(_NORMS, "norm")
 register_position = _register(_POSITIONS, "position encoding")
 register_block = _register(_BLOCKS, "block")
+register_head = _register(_HEADS, "output layer")
 
 build_mixer = _build(_MIXERS, "mixer")
 build_feed_forward = _build(_FEED_FORWARDS, "feed-forward")
 build_norm = _build(_NORMS, "norm")
 build_position = _build(_POSITIONS, "position encoding")
 build_block = _build(_BLOCKS, "block")
+build_head = _build(_HEADS, "output layer")

@@ -23,7 +23,7 @@ class RotarySpec(PartSpec):
     theta: float = 10000.0
     max_position: int = 0
     scaling: Optional[Dict] = None     # {"rope_type": "llama3", "factor": ..., ...} or None
-    pairing: str = "half"              # dims (j, j + rot_dim/2) rotate together
+    pairing: str = "half"              # "half": dims (j, j + rot_dim/2) rotate together; "interleaved": (2j, 2j + 1)
 
 
 @dataclass
@@ -69,12 +69,13 @@ class RotaryPosition:
     def __init__(self, spec: RotarySpec):
         if spec.rot_dim <= 0 or spec.rot_dim % 2:
             raise ConfigError("rotary dimension must be positive and even, got %d" % spec.rot_dim)
-        if spec.pairing != "half":
-            raise ConfigError("unsupported rotary pairing %r" % (spec.pairing,))
+        if spec.pairing not in ("half", "interleaved"):
+            raise ConfigError("unsupported rotary pairing %r (half or interleaved)" % (spec.pairing,))
         if spec.max_position <= 0:
             raise ConfigError("rotary position encoding needs max_position > 0")
         self.spec = spec
         self.rot_dim = spec.rot_dim
+        self.pairing = spec.pairing
         self._tables = {}
 
     def inv_freq(self) -> torch.Tensor:

@@ -15,16 +15,20 @@ ROW_F32 = 2e-5
 #
 # bfloat16, against the plain implementation: the bound is a formula, not a constant.  The plain
 # implementation runs a second time with every tensor that an engine stores between two operators
-# rounded to bfloat16 (``plain.llama.logits_all(..., store=to_bfloat16)``): an engine that computes
-# every sum exactly and stores in bfloat16.  Its distance from the exact logits, in the same two
-# metrics, is what bfloat16 costs for these weights and these tokens; it grows with the spread of
-# the weights times the root of the width (peaked softmax, large SiLU arguments) and differs from
-# position to position.  A correct engine rounds at slightly other places (probabilities, the
-# products that are added into the stream, a norm's scale before or after the rounding), so its
-# error is another draw of the same size: measured ratios of engine error to this model's error
-# are 0.95 to 1.5 (kernels emulated on the CPU) and up to 1.6 (GPU, the traces of the tests).
-# The bound is BF16_MARGIN times the model's error of the same request.
-BF16_MARGIN = 2.0
+# rounded to bfloat16, and the probabilities as they enter the second product of attention
+# (``plain.llama.logits_all(..., store=to_bfloat16)``): an engine that computes every sum exactly
+# and stores in bfloat16.  Its distance from the exact logits, in the same two metrics, is what
+# bfloat16 costs for these weights and these tokens; it grows with the spread of the weights times
+# the root of the width (peaked softmax, large SiLU arguments) and differs from position to
+# position.  A correct engine rounds at slightly other places (a product that is added into the
+# stream, a norm's scale before or after the rounding, q|k|v before and after the rotation), so its
+# error is another draw of about the same size, and both metrics are maxima over the rows of a
+# request, which spreads their quotient.  Measured, engine error over this model's error, per
+# request: kernels emulated on the CPU 0.95 to 1.5; on the GPU over the 1,596 bfloat16 requests of
+# 132 drawn traces the median is 1.02, 99 in 100 lie below 1.5, the largest is 1.63 in the row
+# metric and 1.96 in the max metric (the configuration with a bias on q|k|v lies highest).  The
+# bound is BF16_MARGIN times the model's error of the same request.
+BF16_MARGIN = 2.5
 # bfloat16 without such a model (one engine against another, toy parts with references of their
 # own): constants for the tiny configurations, widths up to 192 at a spread of 0.08.  bfloat16 keeps
 # 8 bits of significand where the reference's half keeps 11, so its bound for half (0.02,

@@ -137,11 +137,14 @@ def expand_kv_heads(x, n_heads):
     return np.repeat(x, group, axis=0)
 
 
-def attention(q, k, v, causal):
+def attention(q, k, v, causal, store=None):
     """q [n_heads, Lq, hd], k, v [n_kv, Lk, hd] -> [n_heads, Lq, hd].
     Scores (q*s)(k*s)^T with s = sqrt(1/sqrt(hd)); the causal mask of size Lk is sliced to its
     last Lq rows (bottom-right aligned) and skipped for a single query
-    (src/flint/operators.cc:100-127)."""
+    (src/flint/operators.cc:100-127).  ``store`` (see attention_block) is applied to the
+    probabilities, which are the left operand of the second product in the storage type; not to
+    the scores, which the reference also stores between its operators but which an engine with
+    one attention kernel keeps in 32-bit."""
     n_heads, lq, hd = q.shape
     n_kv, lk, _ = k.shape
     assert n_heads % n_kv == 0
@@ -152,7 +155,8 @@ def attention(q, k, v, causal):
     scores = (q * s) @ np.swapaxes(k * s, -1, -2)
     if causal and lq > 1:
         scores = scores + causal_mask(lk)[lk - lq:lk][None]
-    return softmax(scores) @ v
+    p = softmax(scores)
+    return (p if store is None else store(p)) @ v
 
 
 # --------------------------------------------------------------------------- blocks
@@ -187,7 +191,7 @@ def attention_block(cfg, weights, layer, x, positions, store=exact):
     cos, sin = rope_table(positions, rope_inv_freq(cfg.head_dim, cfg.theta, cfg.scaling))
     q = store(apply_rope(q, cos, sin))
     k = store(apply_rope(k, cos, sin))
-    o = attention(q.transpose(1, 0, 2), k.transpose(1, 0, 2), v.transpose(1, 0, 2), True)
+    o = attention(q.transpose(1, 0, 2), k.transpose(1, 0, 2), v.transpose(1, 0, 2), True, store)
     o = store(o.transpose(1, 0, 2).reshape(t, qd))
     return store(linear(o, weights[p + "o_proj.weight"]))
 

@@ -7,7 +7,7 @@ from libllm_amd import ConfigError
 from libllm_amd.config import (LlamaConfig, ScheduleEntry, architectures, config_from_dict,
                                config_from_dir, register_architecture, validate_schedule)
 from libllm_amd.engine import DecoderModel
-from tiny import TINY_A, TINY_B, TINY_C
+from tiny import LLAMA3_MIDDLE_BAND, TINY_A, TINY_B, TINY_C
 
 
 def test_every_key_is_read():
@@ -60,6 +60,18 @@ def test_errors_name_the_key(change, word):
     with pytest.raises(ConfigError) as e:
         DecoderModel(config_from_dict(d).to_spec()).blocks[0].mixer.position.inv_freq()
     assert word in str(e.value)
+
+
+@pytest.mark.parametrize("params,want", LLAMA3_MIDDLE_BAND)
+def test_llama3_middle_band_values(params, want):
+    """The engine's frequency table at the pairs of the middle band, against numbers worked out
+    apart from it (see tiny.LLAMA3_MIDDLE_BAND)."""
+    from libllm_amd.parts.rope import scaled_inv_freq
+    factor, low, high, orig, theta, hd = params
+    got = scaled_inv_freq(hd, theta, {"rope_type": "llama3", "factor": factor, "low_freq_factor": low,
+                                      "high_freq_factor": high, "original_max_position_embeddings": orig})
+    for j, value in want.items():
+        assert abs(float(got[j]) / value - 1.0) < 1e-12, (j, float(got[j]), value)
 
 
 def test_config_from_dir(tmp_path):

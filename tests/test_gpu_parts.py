@@ -216,6 +216,80 @@ def test_toy_routed_feed_forward_and_position_encoding(ops, dtype):
     engine.cache.check()
 
 
+def _halves_from_neighbours(w, n_heads, hd, rot):
+    """Rows of a q or k projection (or bias) reordered so that the dims an interleaved encoding
+    rotates together, (2j, 2j+1), become the pair (j, j + rot/2) of the rotate-half form."""
+    head = np.arange(hd)
+    head[:rot // 2], head[rot // 2:rot] = np.arange(0, rot, 2), np.arange(1, rot, 2)
+    order = (np.arange(n_heads)[:, None] * hd + head[None, :]).reshape(-1)
+    return w[order]
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("base", [TINY_A, dict(TINY_B, attention_bias=True)])
+def test_interleaved_rotary_pairing(ops, dtype, base):
+    """A position encoding that rotates neighbouring dims (2j, 2j+1) instead of the halves of a
+    head: chosen in the model's record, no other change.  The plain implementation rotates halves;
+    it is given the q and k projections with their rows reordered accordingly, which leaves every
+    score unchanged.  Whole prompts, cut prompts and single tokens."""
+    cfg = llama.PlainConfig(base)
+    spec = config_from_dict(base).to_spec()
+    for layer in spec.layers:
+        layer.mixer.position.pairing = "interleaved"
+    model = DecoderModel(spec)
+    t = random_tensors(model.declared(), 31, std=0.1, norm_std=0.2)
+    model.bind({k: v.to("cuda", torch.float32 if (dtype == torch.float32 or v.dim() == 1) else dtype)
+                for k, v in t.items()}, ops, dtype)
+    assert all(b.mixer.adjacent for b in model.blocks)
+    engine = Engine(model, ops, dtype, max_tokens=512)
+    w = {k: v.double().numpy() for k, v in t.items()}
+    for name in list(w):
+        for proj, heads in (("q_proj", cfg.n_heads), ("k_proj", cfg.n_kv)):
+            if "." + proj + "." in name:
+                w[name] = _halves_from_neighbours(w[name], heads, cfg.head_dim, cfg.head_dim)
+    rng = np.random.default_rng(6)
+    reqs = {"a": rng.integers(0, cfg.vocab, size=90).tolist(), "b": rng.integers(0, cfg.vocab, size=17).tolist()}
+    steps = traces.batches([reqs], {"a": 20, "b": 5})
+    got = {}
+    for s in steps:
+        out = engine.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        row = 0
+        for e in s["entries"]:
+            for _ in e["want"]:
+                got.setdefault(e["id"], []).append(out[row].double().cpu().numpy())
+                row += 1
+        engine.end(s["end"])
+    for rid, toks in reqs.items():
+        assert_logits_close(np.stack(got[rid]), llama.logits_all(cfg, w, toks), dtype, rid)
+    # and it is not the rotate-half form under another name: the unpermuted weights give other logits
+    plain_half = llama.logits_all(cfg, {k: v.double().numpy() for k, v in t.items()}, reqs["a"])
+    assert rel_err(np.stack(got["a"]), plain_half) > 0.5
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_output_layer(ops, dtype):
+    """An output layer of another kind (capped logits), defined in tests/toy.py and chosen in the
+    model's record; it runs inside captured graphs like the built-in one."""
+    cfg = llama.PlainConfig(TINY_A)
+    spec = config_from_dict(TINY_A).to_spec()
+    spec.head = toy.CappedHeadSpec(spec.head.vocab, spec.head.width, spec.head.tensor, spec.head.tied,
+                                   kind="capped", cap=2.0)
+    model = DecoderModel(spec)
+    t = random_tensors(model.declared(), 33, std=0.1, norm_std=0.2)
+    model.bind({k: v.to("cuda", torch.float32 if (dtype == torch.float32 or v.dim() == 1) else dtype)
+                for k, v in t.items()}, ops, dtype)
+    engine = Engine(model, ops, dtype, max_tokens=256)
+    assert engine.use_graphs
+    w = {k: v.double().numpy() for k, v in t.items()}
+    ids = np.random.default_rng(9).integers(0, 256, size=40).tolist()
+    ref = 2.0 * np.tanh(llama.logits_all(cfg, w, ids) / 2.0)
+    assert np.abs(ref).max() > 1.5                                   # the cap bites
+    out = [engine.step([StepEntry("a", ids[:30], list(range(30)))]).double().cpu().numpy()]
+    out += [engine.step([StepEntry("a", [x], [0])]).double().cpu().numpy() for x in ids[30:]]
+    assert engine._graphs
+    assert_logits_close(np.concatenate(out), ref, dtype, "capped")
+
+
 @pytest.mark.parametrize("dtype", DTYPES)
 def test_schedule_and_mixed_layers_on_the_gpu(ops, dtype):
     """A layer run twice, a run that reads another run's keys, and a layer with a window and

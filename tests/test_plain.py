@@ -9,7 +9,7 @@ import pytest
 from scipy.special import softmax as scipy_softmax
 
 from plain import llama, sampling
-from tiny import TINY_A, TINY_B
+from tiny import LLAMA3_MIDDLE_BAND, TINY_A, TINY_B
 
 
 def rng(seed=0):
@@ -131,6 +131,16 @@ def test_llama3_frequency_bands():
             assert abs(_scaled_single(freq, sc) / freq - want) < 1e-6
     one = dict(sc, factor=1.0)
     assert np.allclose(llama.rope_inv_freq(hd, cfg["rope_theta"], one), plain)
+
+
+@pytest.mark.parametrize("params,want", LLAMA3_MIDDLE_BAND)
+def test_llama3_middle_band_values(params, want):
+    factor, low, high, orig, theta, hd = params
+    sc = {"rope_type": "llama3", "factor": factor, "low_freq_factor": low, "high_freq_factor": high,
+          "original_max_position_embeddings": orig}
+    got = llama.rope_inv_freq(hd, theta, sc)
+    for j, value in want.items():
+        assert abs(got[j] / value - 1.0) < 1e-12, (j, got[j], value)
 
 
 def _scaled_single(freq, sc):

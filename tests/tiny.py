@@ -31,6 +31,23 @@ TINY_C = {
 }
 
 
+# The middle band at the parameters of the released 1B and 3B models (factor 32, original window
+# 8,192, base 500,000, head size 64) and of Tiny B, worked out apart from the code under test with
+# 50 decimal digits: pair j has frequency f = base^(-2j/hd) and wavelength 2 pi / f; with
+# s = (window / wavelength - low) / (high - low), linear in the quotient of the frequencies, the
+# scaled frequency is (1 - s) f / factor + s f.  A blend that is linear in the wavelength instead
+# keeps the bands, their bounds and the continuity at both edges, and gives 42 % to 158 % more at
+# these pairs.  Parity with the table that the reference's exporter stores
+# (tools/llama_exporter.py:54-62 takes it from an external rotary module) is not pinned by any file
+# of the reference: these numbers hold the published rule.
+LLAMA3_MIDDLE_BAND = [
+    ((32.0, 1.0, 4.0, 8192, 500000.0, 64), {14: 0.003211445994752591, 15: 0.0012905479282092638,
+                                           16: 0.0004295567965593682, 17: 9.708287802627673e-05,
+                                           18: 1.9461638184831125e-05}),
+    ((8.0, 1.0, 4.0, 64, 500000.0, 32), {1: 0.44036660267178046, 2: 0.0794030091792082, 3: 0.010674637535720701}),
+]
+
+
 def make_model(tmpdir, cfg_dict, seed=0, std=0.08, norm_std=0.2, name="model", stored="bfloat16"):
     """Writes a model folder through the library's random-weights mode.  The spread of the
     weights is wider than the usual 0.02 so that attention is far from uniform, and norm scales

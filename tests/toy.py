@@ -196,3 +196,31 @@ def toys_oracle(cfg, weights, ids, step=0.05):
     x = x + y
     out = llama.lm_head(cfg, weights, llama.rms_norm(x, weights["model.norm.weight"], cfg.eps))
     return out, margin[:, -1] - margin[:, -2]
+
+
+# ---------------------------------------------------------------------------------------------
+# An output layer of another kind: logits capped smoothly, cap * tanh(h W^T / cap).
+from libllm_amd.config.spec import HeadSpec  # noqa: E402
+from libllm_amd.parts import register_head  # noqa: E402
+from libllm_amd.parts.linear import Linear  # noqa: E402
+
+
+@dataclass
+class CappedHeadSpec(HeadSpec):
+    cap: float = 30.0
+
+
+@register_head("capped")
+class CappedHead:
+    graph_safe = True
+    takes_normed = True
+
+    def __init__(self, spec: CappedHeadSpec):
+        self.cap = float(spec.cap)
+        self.linear = Linear(spec.width, spec.vocab)
+
+    def bind(self, weight, ops, dtype):
+        self.linear.bind(weight, ops=ops)
+
+    def forward(self, ctx, h):
+        return self.cap * torch.tanh(self.linear(ctx, h, out_dtype=torch.float32) / self.cap)
