@@ -5,10 +5,13 @@ decoding at batch 1 and 64.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
 
-A step is one decode step of the engine that generation uses: the step function over the cache
-(as a captured graph), arg-max sampling on the device and the sampled tokens fed back.  The
-sequences are first filled by real prompt steps so that the timed steps end at the context length.
-One JSON line is printed; everything else goes to standard error.
+A step is one decode step inside the generation loop (``Generator.stream``, the loop that serves
+requests): the step function over the cache as a captured graph, arg-max sampling on the device,
+the sampled tokens fed back, the loop's own bookkeeping.  The prompts go through the loop's prompt
+steps, sized so that the timed steps end at the context length.  Beside the published peaks the
+line gives what this GPU reaches in kernels of this library that only read memory or only issue
+matrix instructions (``peak_measured``).  One JSON line is printed; everything else goes to
+standard error.
 
 The reference's own tool reports prompt and decoding speed of one sequence
 (src/libllm/benchmark_main.cc:52-86); it publishes no numbers, so ``vs_baseline`` is null.
@@ -78,49 +81,32 @@ def prefill_flops(cfg, t):
     return linear + attention + head
 
 
-def fill(engine, torch, names, length, vocab, seed, chunk_tokens=16384):
-    """Brings every named sequence to ``length`` cached tokens through prompt steps."""
-    from libllm_amd.engine import StepEntry
-    g = torch.Generator().manual_seed(seed)
-    per_step = max(1, chunk_tokens // max(length, 1))
-    for i in range(0, len(names), per_step):
-        group = names[i:i + per_step]
-        entries = [StepEntry(n, torch.randint(0, vocab, (length,), generator=g).tolist(), [])
-                   for n in group]
-        engine.step(entries)
-    torch.cuda.synchronize()
-
-
-def decode_steps(engine, sampler, params, torch, names, tokens, n):
-    """``n`` decode steps as the generation loop runs them: a step is queued with the tokens the
-    sampler left on the device, and the host reads each step's tokens while the next one runs."""
-    from libllm_amd.engine import StepEntry
-    streams = list(range(len(names)))
-    logits = engine.step([StepEntry(r, [t], [0]) for r, t in zip(names, tokens)])
-    pending = sampler.sample_device(logits, params, streams, [0] * len(names))
-    placeholders = [StepEntry(r, [0], [0]) for r in names]
-    for k in range(1, n):
-        logits = engine.step(placeholders, tokens_device=pending.device)
-        ahead = sampler.sample_device(logits, params, streams, [k] * len(names))
-        pending.tokens()                                   # the host sees every token, one step late
-        pending = ahead
-    return pending.tokens()
-
-
-def time_decode(engine, sampler, params, torch, batch, context, steps, warmup, vocab, tag):
-    names = [(tag, i) for i in range(batch)]
-    start = context - steps - warmup
+def time_decode(gen, params, torch, batch, context, steps, warmup, vocab):
+    """Seconds that ``steps`` decode steps of ``batch`` sequences take inside the generation loop
+    (``Generator.stream``: the loop that serves requests, with its bookkeeping, the next step
+    queued while the host reads the last one's tokens), the last of them at ``context`` tokens.
+    The prompts are random tokens and go through the loop's own prompt steps; ``warmup`` decode
+    steps run before the clock starts.  The clock is read after a device-wide wait on both sides."""
+    start = context - steps - warmup - 1
     if start < 1:
         raise SystemExit("context %d is too short for %d steps" % (context, steps + warmup))
-    fill(engine, torch, names, start, vocab, seed=batch)
-    tokens = [(11 * i + 5) % vocab for i in range(batch)]
-    tokens = decode_steps(engine, sampler, params, torch, names, tokens, warmup)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    decode_steps(engine, sampler, params, torch, names, tokens, steps)
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    engine.end(names)
+    g = torch.Generator().manual_seed(batch)
+    prompts = [torch.randint(0, vocab, (start,), generator=g).tolist() for _ in range(batch)]
+    stream = gen.stream(prompts, params, max_new_tokens=warmup + steps + 4, stop_tokens=())
+    seen, t0, dt = 0, None, None
+    # When the tokens of decode step s have come, step s + 1 is queued already: the wait at the
+    # first mark ends with step warmup + 1, the wait at the second with step warmup + steps + 1.
+    first_mark, second_mark = (warmup + 1) * batch, (warmup + steps + 1) * batch
+    for _ in stream:
+        seen += 1
+        if seen == first_mark:
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+        elif seen == second_mark:
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            break
+    stream.close()                                         # ends the requests, gives their slots back
     return dt
 
 
@@ -222,7 +208,9 @@ def main() -> int:
     if args.workload:
         return run_workload(args, torch)
 
+    from libllm_amd.cache import PAGE
     from libllm_amd.config import config_from_dict
+    from libllm_amd.engine import Generator
     from libllm_amd.runtime import random_engine
     from libllm_amd.sampling import Sampler, SamplingParams
 
@@ -240,16 +228,19 @@ def main() -> int:
     log("building %d layers of %d with random weights, cache for %d tokens" %
         (args.layers, layers_full, max_tokens))
     engine = random_engine(cfg, seed=0, dtype=args.dtype, max_tokens=max_tokens)
-    sampler = Sampler(engine.ops, cfg.vocab_size)
+    gen = Generator(engine, Sampler(engine.ops, cfg.vocab_size), (), cfg.max_position_embeddings,
+                    engine.cache.n_pages, PAGE, max_batch=biggest)
     params = SamplingParams(temperature=0.0)
     vocab = cfg.vocab_size
+    peaks = engine.ops.measured_peaks()
+    log("measured on this GPU: read %.0f GB/s, copy %.0f GB/s, bf16 matrix cores %.0f TFLOP/s, fp32 %.1f TFLOP/s"
+        % (peaks["read_GBs"], peaks["copy_GBs"], peaks["bf16_TFs"], peaks["fp32_TFs"]))
 
     pre_s = time_prefill(engine, torch, args.prefill, vocab, reps=3)
     pf = prefill_flops(cfg, args.prefill)
     log("prefill of %d tokens: %.2f ms" % (args.prefill, pre_s * 1e3))
 
-    dt = time_decode(engine, sampler, params, torch, args.batch, args.context, args.steps, args.warmup,
-                     vocab, "main")
+    dt = time_decode(gen, params, torch, args.batch, args.context, args.steps, args.warmup, vocab)
     ms = dt / args.steps * 1e3
     value = args.batch * args.steps / dt
     log("decode at batch %d: %.3f ms a step, %.0f tokens/s" % (args.batch, ms, value))
@@ -257,11 +248,11 @@ def main() -> int:
     step_bytes = weight_bytes(cfg, itemsize) + args.batch * mean_ctx * kv_bytes_per_token(cfg, itemsize)
     achieved = step_bytes / (dt / args.steps) / 1e9
 
+    flops_measured = (peaks["bf16_TFs"] if short == "bf16" else peaks["fp32_TFs"]) * 1e12
     points = {}
     if not args.no_points:
         for b in (1, 64):
-            dtb = time_decode(engine, sampler, params, torch, b, args.context, args.steps, args.warmup,
-                              vocab, "b%d" % b)
+            dtb = time_decode(gen, params, torch, b, args.context, args.steps, args.warmup, vocab)
             points["decode_b%d" % b] = round(b * args.steps / dtb, 1)
             log("decode at batch %d: %.3f ms a step, %.0f tokens/s" % (b, dtb / args.steps * 1e3, b * args.steps / dtb))
 
@@ -281,9 +272,13 @@ def main() -> int:
             "prefill_tokens": args.prefill, "sampling": "greedy", "parallelism": "single GPU",
         },
         "prefill": {"value": round(args.prefill / pre_s, 1), "tokens": args.prefill,
-                    "ms": round(pre_s * 1e3, 3), "frac": round(pf / pre_s / DENSE_FLOPS[short], 4)},
+                    "ms": round(pre_s * 1e3, 3), "frac": round(pf / pre_s / DENSE_FLOPS[short], 4),
+                    "peak_measured": round(flops_measured / 1e12, 1), "unit_measured": "TFLOP/s",
+                    "frac_measured": round(pf / pre_s / flops_measured, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_BYTES_PER_S / 1e9,
-                     "unit": "GB/s", "frac": round(achieved / (HBM_BYTES_PER_S / 1e9), 4)},
+                     "unit": "GB/s", "frac": round(achieved / (HBM_BYTES_PER_S / 1e9), 4),
+                     "peak_measured": round(peaks["read_GBs"], 1),
+                     "frac_measured": round(achieved / peaks["read_GBs"], 4)},
         "points": points,
     }
     print(json.dumps(out), flush=True)

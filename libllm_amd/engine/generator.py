@@ -9,6 +9,8 @@ leave the batch and give their slot back, and batches follow one another until a
 from dataclasses import dataclass, field
 from typing import Callable, Iterable, List, Optional, Sequence
 
+import torch
+
 from ..errors import RequestError
 from ..sampling import Sampler, SamplingParams
 from .step import StepEntry
@@ -40,6 +42,30 @@ def plan_batches(prompt_lens: Sequence[int], max_new_tokens: int, max_batch: int
     if cur:
         batches.append(cur)
     return batches
+
+
+def plan_prompt_steps(prompt_lens: Sequence[int], max_rows: int) -> List[List[tuple]]:
+    """Cuts the prompts of a batch into steps of at most ``max_rows`` rows, which bounds the
+    activations a step needs: a list of steps, each a list of (sequence, first token, end).  The
+    sequences come in their order; a prompt that does not fit what is left of a step goes on in
+    the next one (a step's entries then hold parts of different prompts, which the step function
+    takes as they are).  Prompts that fit together make one step."""
+    if max_rows <= 0:
+        raise RequestError("the rows of a prompt step must be positive")
+    steps, cur, room = [], [], max_rows
+    for i, n in enumerate(prompt_lens):
+        start = 0
+        while start < n:
+            take = min(n - start, room)
+            cur.append((i, start, start + take))
+            start += take
+            room -= take
+            if room == 0:
+                steps.append(cur)
+                cur, room = [], max_rows
+    if cur:
+        steps.append(cur)
+    return steps
 
 
 @dataclass
@@ -85,7 +111,10 @@ class Generator:
     ``sample(logits, params, streams, counters)``."""
 
     def __init__(self, engine, sampler, stop_tokens: Iterable[int], max_position: int,
-                 page_budget: int, page: int, max_batch: int = 64):
+                 page_budget: int, page: int, max_batch: int = 64, max_prompt_rows: int = 16384):
+        """``max_prompt_rows``: the most rows one prompt step brings; a batch whose prompts hold
+        more starts with several steps (see ``plan_prompt_steps``)."""
+        self.max_prompt_rows = max_prompt_rows
         self.engine = engine
         self.sampler = sampler
         self.stop_tokens = set(stop_tokens)
@@ -134,9 +163,7 @@ class Generator:
         ahead = (getattr(self.sampler, "samples_ahead", False)
                  and getattr(self.engine, "takes_device_tokens", False))
         try:
-            entries = [StepEntry(name[st.index], list(prompts[st.index]), [st.prompt_len - 1])
-                       for st in live]
-            logits = self.engine.step(entries)
+            logits = self._prompt_steps(live, prompts, name)
             pending = self._draw(logits, params, live, 0, ahead)
             while True:
                 queued = None
@@ -174,6 +201,24 @@ class Generator:
             held = [name[st.index] for st in live if self._holds(name[st.index])]
             if held:
                 self.engine.end(held)
+
+    def _prompt_steps(self, live, prompts, name):
+        """The prompts of a batch through the step function; returns the logits of every
+        sequence's last prompt token, in the order of ``live``."""
+        plan = plan_prompt_steps([st.prompt_len for st in live], self.max_prompt_rows)
+        rows = []
+        for step in plan:
+            entries = []
+            for i, start, end in step:
+                st = live[i]
+                entries.append(StepEntry(name[st.index], list(prompts[st.index][start:end]),
+                                         [end - start - 1] if end == st.prompt_len else []))
+            logits = self.engine.step(entries)
+            if len(plan) == 1:
+                return logits
+            if logits is not None:
+                rows.append(logits.clone())        # the next step may overwrite what it returned
+        return torch.cat(rows, dim=0)
 
     def _draw(self, logits, params, seqs, lead, ahead):
         """Samples one token for each sequence; ``lead`` counts tokens that are drawn but not yet

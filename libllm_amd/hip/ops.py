@@ -56,6 +56,11 @@ _SIGNATURES = {
     "llm_sample": [_vp, _vp, _i, _i, _f, _i, _f, _u64, _vp, _vp, _vp, _vp, _vp, _vp],
     "llm_sample_parts": [_i],
     "llm_sample_k_part": [_i, _i],
+    "llm_peak_sink_words": [],
+    "llm_peak_read": [_vp, ctypes.c_size_t, _vp, _vp],
+    "llm_peak_copy": [_vp, _vp, ctypes.c_size_t, _vp],
+    "llm_peak_mfma_bf16": [_vp, _i, ctypes.POINTER(ctypes.c_double), _vp],
+    "llm_peak_fma_f32": [_vp, _i, ctypes.POINTER(ctypes.c_double), _vp],
 }
 
 
@@ -631,6 +636,38 @@ class HipOps:
             kv.block_table.data_ptr(), kv.block_table.shape[1], 64, ctx.tok_pos.data_ptr(),
             ctx.tok_seq.data_ptr(), ctx.seq_slot.data_ptr(), out.data_ptr(), m, n_heads, n_kv, hd,
             float(scale), int(window), self._stream()), "attention")
+        return out
+
+    def measured_peaks(self, nbytes: int = 2 << 30, reps: int = 5):
+        """What this GPU reaches at most, by kernels of this library timed with events (the best of
+        ``reps`` runs after one to warm up): {"read_GBs": a read of ``nbytes``, "copy_GBs": a copy
+        of them (bytes read plus bytes written), "bf16_TFs": a loop of matrix-core instructions on
+        registers, "fp32_TFs": a loop of float32 multiply-adds}."""
+        src = torch.empty(nbytes, dtype=torch.uint8, device=self.device).fill_(1)
+        dst = torch.empty_like(src)
+        sink = torch.empty(self.lib.llm_peak_sink_words(), dtype=torch.int32, device=self.device)
+        flops = ctypes.c_double(0.0)
+
+        def best(launch):
+            times = []
+            for r in range(reps + 1):
+                t0, t1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                t0.record()
+                self._check(launch(), "peak measurement")
+                t1.record()
+                t1.synchronize()
+                if r:
+                    times.append(t0.elapsed_time(t1) * 1e-3)
+            return min(times)
+        out = {}
+        t = best(lambda: self.lib.llm_peak_read(src.data_ptr(), nbytes, sink.data_ptr(), self._stream()))
+        out["read_GBs"] = nbytes / t / 1e9
+        t = best(lambda: self.lib.llm_peak_copy(src.data_ptr(), dst.data_ptr(), nbytes, self._stream()))
+        out["copy_GBs"] = 2 * nbytes / t / 1e9
+        t = best(lambda: self.lib.llm_peak_mfma_bf16(sink.data_ptr(), 20000, ctypes.byref(flops), self._stream()))
+        out["bf16_TFs"] = flops.value / t / 1e12
+        t = best(lambda: self.lib.llm_peak_fma_f32(sink.data_ptr(), 20000, ctypes.byref(flops), self._stream()))
+        out["fp32_TFs"] = flops.value / t / 1e12
         return out
 
     def argmax(self, logits):

@@ -4,7 +4,7 @@ import pytest
 import torch
 
 from libllm_amd import RequestError
-from libllm_amd.engine import Generator, SequenceState, plan_batches
+from libllm_amd.engine import Generator, SequenceState, plan_batches, plan_prompt_steps
 from libllm_amd.sampling import Sampler, SamplingParams
 
 
@@ -22,6 +22,8 @@ class ScriptedEngine:
         for e in entries:
             i = e.request[2]
             self.live.add(e.request)
+            if not e.want:                  # a part of a prompt: nothing comes back for it
+                continue
             n = self.cursor.get(i, 0)
             out.append(self.scripts[i][n])
             self.cursor[i] = n + 1
@@ -193,3 +195,26 @@ def test_queued_ahead_respects_the_position_limit():
     gen = Generator(eng, smp, (99,), 5, 1000, 64)           # prompt 3 + 2 tokens reach the limit
     assert gen.generate([[1, 2, 3]], SamplingParams(0.0), max_new_tokens=10) == [[5, 6]]
     assert [s[0][1] for s in eng.steps] == [[1, 2, 3], [5]]  # no step beyond the limit
+
+
+def test_prompt_steps_are_bounded():
+    """The prompts of a batch come in steps of at most ``max_prompt_rows`` rows: prompts that fit
+    together share a step, a long one is cut, and the last token's logits are wanted where a
+    prompt ends.  The tokens that follow are the same as with one big step."""
+    assert plan_prompt_steps([3, 2, 4], 100) == [[(0, 0, 3), (1, 0, 2), (2, 0, 4)]]
+    assert plan_prompt_steps([3, 2, 4], 4) == [[(0, 0, 3), (1, 0, 1)], [(1, 1, 2), (2, 0, 3)], [(2, 3, 4)]]
+    assert plan_prompt_steps([9], 4) == [[(0, 0, 4)], [(0, 4, 8)], [(0, 8, 9)]]
+    with pytest.raises(RequestError):
+        plan_prompt_steps([1], 0)
+    scripts = {0: [5, 6, 99], 1: [7, 99], 2: [8, 9, 99]}
+    prompts = [[1, 2, 3], [4, 5], [6, 7, 8, 9]]
+    eng, smp, gen = make(scripts)
+    gen.max_prompt_rows = 4
+    out = gen.generate(prompts, SamplingParams(0.0), max_new_tokens=8)
+    assert out == [[5, 6], [7], [8, 9]]
+    assert eng.steps[0] == [(0, [1, 2, 3], [2]), (1, [4], [])]
+    assert eng.steps[1] == [(1, [5], [0]), (2, [6, 7, 8], [])]
+    assert eng.steps[2] == [(2, [9], [0])]
+    assert eng.steps[3] == [(0, [5], [0]), (1, [7], [0]), (2, [8], [0])]
+    assert smp.calls[0] == ([0, 1, 2], [0, 0, 0])
+    assert sorted(eng.ended) == [0, 1, 2] and not eng.live
