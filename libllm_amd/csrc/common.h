@@ -9,6 +9,7 @@
 #define LLM_OK 0
 #define LLM_ERR_ARG 1        // an argument the kernel refuses (size, dtype, alignment)
 #define LLM_ERR_LAUNCH 2     // the runtime refused the launch
+#define LLM_ERR_TOO_LARGE 3  // the operands exceed a fixed buffer of an entry point that allocates nothing
 
 typedef uint16_t bf16_t;     // bfloat16 as raw bits: the upper half of an IEEE float
 

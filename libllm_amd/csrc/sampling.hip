@@ -6,7 +6,10 @@
 // r = u * sum(kept), first candidate whose running sum exceeds r.  With top_k == 0 nothing is cut
 // and the draw walks the vocabulary in index order.  u comes from a counter hash of
 // (seed, stream, counter).
+#include <mutex>
+
 #include "common.h"
+#include "no_alloc.h"
 
 __device__ __forceinline__ uint32_t order_key(float x) {
   const uint32_t u = __float_as_uint(x);
@@ -105,6 +108,53 @@ extern "C" int llm_argmax(const float* logits, int* out, float* part_val, int* p
   if (hipGetLastError() != hipSuccess) return LLM_ERR_LAUNCH;
   argmax_final_kernel<64><<<R, 64, 0, stream>>>(part_val, part_idx, parts, out);
   return llm_launch_status();
+}
+
+// The same without scratch arrays from the caller (see no_alloc.h): the partial results live in a
+// file-scope device array.  In host code the array's name stands for the symbol, not for device
+// memory: its address on a device comes from hipGetSymbolAddress, once per device, and only that
+// pointer goes to kernels.
+static __device__ __align__(256) unsigned char argmax_static_scratch[LLM_ARGMAX_STATIC_BYTES];
+
+#define LLM_MAX_DEVICES 64
+static void* argmax_static_ptr[LLM_MAX_DEVICES];      // per device: each GPU has its own copy of the array
+static std::mutex argmax_static_lock;
+
+// The array's address on the current device; null if the runtime refuses.
+static void* argmax_static_address() {
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= LLM_MAX_DEVICES) return nullptr;
+  std::lock_guard<std::mutex> guard(argmax_static_lock);
+  if (argmax_static_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    if (hipGetSymbolAddress(&p, HIP_SYMBOL(argmax_static_scratch)) != hipSuccess) {
+      (void)hipGetLastError();
+      return nullptr;
+    }
+    argmax_static_ptr[dev] = p;
+  }
+  return argmax_static_ptr[dev];
+}
+
+extern "C" int llm_argmax_static_init(void) {
+  return argmax_static_address() != nullptr ? LLM_OK : LLM_ERR_LAUNCH;
+}
+
+extern "C" int llm_argmax_static_max_rows(int V) {
+  if (V <= 0) return 0;
+  const int rows = LLM_ARGMAX_STATIC_ENTRIES / llm_argmax_parts(V);
+  return rows > 65535 ? 65535 : rows;
+}
+
+extern "C" int llm_argmax_static(const float* logits, int* out, int R, int V, hipStream_t stream) {
+  if (R <= 0) return LLM_OK;
+  if (V <= 0 || !logits || !out) return LLM_ERR_ARG;
+  if (R > llm_argmax_static_max_rows(V)) return LLM_ERR_TOO_LARGE;
+  void* base = argmax_static_address();
+  if (base == nullptr) return LLM_ERR_LAUNCH;
+  float* part_val = (float*)base;
+  int* part_idx = (int*)((unsigned char*)base + (size_t)LLM_ARGMAX_STATIC_ENTRIES * sizeof(float));
+  return llm_argmax(logits, out, part_val, part_idx, R, V, stream);
 }
 
 // ---------------------------------------------------------------------------------- sampling

@@ -167,7 +167,9 @@ class HipOps:
     def _check(status: int, what: str):
         if status != 0:
             raise KernelError("%s: %s" % (what, {1: "the kernel refuses these operands",
-                                                 2: "the launch failed"}.get(status, "error %d" % status)))
+                                                 2: "the launch failed",
+                                                 3: "the operands exceed the fixed buffer of this entry point"
+                                                 }.get(status, "error %d" % status)))
 
     def _weight(self, w: torch.Tensor, what: str):
         """A weight matrix: on the device, rows contiguous; rows may lie further apart than
