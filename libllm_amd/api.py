@@ -111,21 +111,25 @@ class Completion:
 class Model:
     def __init__(self, config_file: str, device: Union[Device, str] = Device.AUTO, dtype: str = "bfloat16",
                  max_tokens: int = 8192, max_batch: int = 64, ops=None, use_graphs: bool = True,
-                 random_weights: bool = False, seed: int = 0, keep_float32: bool = False) -> None:
+                 random_weights: bool = False, seed: int = 0, keep_float32: bool = False,
+                 tiled_weights: bool = True) -> None:
         """``config_file``: the model folder, or the config.json inside it.  ``device``: a Device
         or one of "auto", "cuda", "hip", "cpu".  With ``random_weights`` only config.json is read
         and every tensor is drawn from ``seed``.  ``keep_float32``: in bfloat16 mode, matrices
-        that the file stores in 32-bit stay float32 instead of becoming bfloat16."""
+        that the file stores in 32-bit stay float32 instead of becoming bfloat16.
+        ``tiled_weights=False``: the matrices are held once, not twice (see ``load_engine``)."""
         if int(parse_device(device)) == int(Device.CPU):
             raise ConfigError("this library has no CPU path; use Device.AUTO or Device.GPU")
         model_dir = os.path.dirname(config_file) if os.path.isfile(config_file) else config_file
         self.model_dir = model_dir
         if random_weights:
             self.engine = random_engine(config_from_dir(model_dir), seed=seed, dtype=dtype,
-                                        max_tokens=max_tokens, ops=ops, use_graphs=use_graphs)
+                                        max_tokens=max_tokens, ops=ops, use_graphs=use_graphs,
+                                        tiled_weights=tiled_weights)
         else:
             self.engine = load_engine(model_dir, dtype=dtype, max_tokens=max_tokens, ops=ops,
-                                      use_graphs=use_graphs, keep_float32=keep_float32)
+                                      use_graphs=use_graphs, keep_float32=keep_float32,
+                                      tiled_weights=tiled_weights)
         self.config = self.engine.config
         spec = self.engine.model.spec
         self._sampler = Sampler(self.engine.ops, spec.vocab)

@@ -156,6 +156,10 @@ def benchmark_main(argv) -> int:
         model.end(["bench"])
     print("prefill@%d  %.1f tokens/s" % (args.l, args.l / prefill))
     print("decode@%d   %.1f tokens/s" % (args.l, args.n / decode))
+    ops = model.engine.ops
+    if getattr(ops, "timing", False):                       # LIBLLM_AMD_TIME=1: where the time went
+        for name, calls, ms in ops.timing_report():
+            print("  %-14s %6d calls %10.3f ms" % (name, calls, ms))
     return 0
 
 

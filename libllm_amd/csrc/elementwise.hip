@@ -198,8 +198,12 @@ extern "C" int llm_silu_mul(const void* gu, void* out, int dtype, int M, int I, 
   if (I <= 0 || M > 65535 * 32) return LLM_ERR_ARG;
   if (dtype == LLM_DTYPE_BF16 && I % 8 == 0 && ((((uintptr_t)gu) | ((uintptr_t)out)) & 15) == 0) {
     const size_t total_vec = (size_t)M * (I / 8);
-    size_t blocks = (total_vec + 511) / 512;                      // two vectors a thread
-    if (blocks > 65536) blocks = 65536;
+    size_t blocks = (total_vec + 511) / 512;                      // two vectors a thread and round
+    // no more than three blocks a compute unit, each going round several times: what the grid
+    // touches at one moment then lies closer together in memory, and a long array streams a
+    // sixth faster than with a block for every 512 vectors (6.4 against 5.4 TB/s when only read)
+    const size_t cap = (size_t)llm_compute_units() * 3;
+    if (blocks > cap) blocks = cap;
     if (blocks == 0) blocks = 1;
     silu_mul_vec_kernel<<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total_vec);
     return llm_launch_status();

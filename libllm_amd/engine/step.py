@@ -54,7 +54,8 @@ class Engine:
         self.vocab = model.spec.vocab
         self.cache = SequenceCache(model.cache_needs(), model.state_needs(), max_tokens,
                                    model.spec.max_position, dtype, self.device, max_slots)
-        self.use_graphs = bool(use_graphs) and ops.supports_graphs and model.graph_safe()
+        self.use_graphs = (bool(use_graphs) and ops.supports_graphs and model.graph_safe()
+                           and not getattr(ops, "timing", False))
         self._graphs: Dict[tuple, "_DecodeGraph"] = {}     # (batch bucket, context bucket) -> graph
         self._prompt_graphs: Dict[tuple, "_PromptGraph"] = {}   # (rows, sequences) -> graph
         self._prompt_seen: Dict[tuple, int] = {}

@@ -8,6 +8,7 @@ for them as well, src/flint/cuda/gemm_cublas.cc:160-197); every other operation 
 """
 import ctypes
 import gc
+import os
 from typing import List, Optional
 
 import numpy as np
@@ -57,8 +58,8 @@ _SIGNATURES = {
     "llm_sample_parts": [_i],
     "llm_sample_k_part": [_i, _i],
     "llm_peak_sink_words": [],
-    "llm_peak_read": [_vp, ctypes.c_size_t, _vp, _vp],
-    "llm_peak_copy": [_vp, _vp, ctypes.c_size_t, _vp],
+    "llm_peak_read": [_vp, ctypes.c_size_t, _vp, _i, _vp],
+    "llm_peak_copy": [_vp, _vp, ctypes.c_size_t, _i, _vp],
     "llm_peak_mfma_bf16": [_vp, _i, ctypes.POINTER(ctypes.c_double), _vp],
     "llm_peak_fma_f32": [_vp, _i, ctypes.POINTER(ctypes.c_double), _vp],
 }
@@ -158,6 +159,50 @@ class HipOps:
             build._say("the product for 65 to 128 rows spills registers in this build: the library's runs instead")
         self.fold_norms = True          # up to ACCUM_ROWS rows, a norm between two products gets no kernel of its own
         self.prompt_tiles = 0           # tiles of rows a wave of prompt attention takes (1 or 2; 0: by the number of blocks)
+        self.timing = False
+        if os.environ.get("LIBLLM_AMD_TIME", "") not in ("", "0"):
+            self.start_timing()
+
+    # ---- time per operation, behind a switch
+    _TIMED = ("embed", "add_rmsnorm", "linear", "linear_swiglu", "silu_mul", "qkv_rope", "rope_kv_write",
+              "attention", "argmax", "sample")
+
+    def start_timing(self) -> None:
+        """From now on every operation is bracketed by two events on its stream, and
+        ``timing_report`` says where the time went (the reference has LOG_TIME around blocks and a
+        build that waits after every kernel, src/lutil/log.h:39-42, src/flint/cuda/common.h:50-54).
+        Also switched on by the environment variable LIBLLM_AMD_TIME=1.  Engines built on these
+        operations then queue every step kernel by kernel: a captured graph would hide the
+        operations from the clock."""
+        if self.timing:
+            return
+        self.timing, self._timed, self._depth = True, {}, 0
+        for name in self._TIMED:
+            setattr(self, name, self._timed_call(name, getattr(self, name)))
+
+    def _timed_call(self, name, fn):
+        def call(*args, **kwargs):
+            if self._depth or torch.cuda.is_current_stream_capturing():
+                return fn(*args, **kwargs)                 # an operation inside another counts once
+            start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            self._depth += 1
+            try:
+                start.record()
+                out = fn(*args, **kwargs)
+                end.record()
+            finally:
+                self._depth -= 1
+            self._timed.setdefault(name, []).append((start, end))
+            return out
+        return call
+
+    def timing_report(self, reset: bool = True):
+        """[(operation, calls, milliseconds)] since the last report, the longest first."""
+        torch.cuda.synchronize(self.device)
+        rows = [(name, len(ev), sum(a.elapsed_time(b) for a, b in ev)) for name, ev in self._timed.items()]
+        if reset:
+            self._timed = {}
+        return sorted(rows, key=lambda r: -r[2])
 
     # ---- helpers
     def _stream(self):
@@ -642,9 +687,10 @@ class HipOps:
 
     def measured_peaks(self, nbytes: int = 2 << 30, reps: int = 5):
         """What this GPU reaches at most, by kernels of this library timed with events (the best of
-        ``reps`` runs after one to warm up): {"read_GBs": a read of ``nbytes``, "copy_GBs": a copy
-        of them (bytes read plus bytes written), "bf16_TFs": a loop of matrix-core instructions on
-        registers, "fp32_TFs": a loop of float32 multiply-adds}."""
+        ``reps`` runs after one to warm up, and for the memory kernels the best of several grid
+        sizes): {"read_GBs": a read of ``nbytes``, "copy_GBs": a copy of them (bytes read plus
+        bytes written), "bf16_TFs": a loop of matrix-core instructions on registers, "fp32_TFs": a
+        loop of float32 multiply-adds in the vector units}."""
         src = torch.empty(nbytes, dtype=torch.uint8, device=self.device).fill_(1)
         dst = torch.empty_like(src)
         sink = torch.empty(self.lib.llm_peak_sink_words(), dtype=torch.int32, device=self.device)
@@ -662,9 +708,12 @@ class HipOps:
                     times.append(t0.elapsed_time(t1) * 1e-3)
             return min(times)
         out = {}
-        t = best(lambda: self.lib.llm_peak_read(src.data_ptr(), nbytes, sink.data_ptr(), self._stream()))
+        grids = (2, 3, 4, 6, 16)        # blocks for every two compute units
+        t = min(best(lambda g=g: self.lib.llm_peak_read(src.data_ptr(), nbytes, sink.data_ptr(), g, self._stream()))
+                for g in grids)
         out["read_GBs"] = nbytes / t / 1e9
-        t = best(lambda: self.lib.llm_peak_copy(src.data_ptr(), dst.data_ptr(), nbytes, self._stream()))
+        t = min(best(lambda g=g: self.lib.llm_peak_copy(src.data_ptr(), dst.data_ptr(), nbytes, g, self._stream()))
+                for g in grids)
         out["copy_GBs"] = 2 * nbytes / t / 1e9
         t = best(lambda: self.lib.llm_peak_mfma_bf16(sink.data_ptr(), 20000, ctypes.byref(flops), self._stream()))
         out["bf16_TFs"] = flops.value / t / 1e12

@@ -188,3 +188,38 @@ def test_smoke_entry():
     sys.path.insert(0, ROOT)
     import __graft_entry__
     __graft_entry__.smoke()
+
+
+def test_time_per_operation_behind_a_switch(tmp_path):
+    """With timing switched on every operation is clocked by events, steps are queued kernel by
+    kernel (no graphs), and the tokens are the same as without."""
+    from libllm_amd import Model
+    from libllm_amd.hip import HipOps
+    path = make_model(tmp_path, TINY_B, seed=12)
+    prompts = [[5, 6, 7, 8, 9], [11, 12]]
+    plain = Model(path, dtype="bfloat16", max_tokens=512).generate(prompts, max_new_tokens=6, temperature=0.0, stop_tokens=())
+    ops = HipOps()
+    ops.start_timing()
+    timed = Model(path, dtype="bfloat16", max_tokens=512, ops=ops)
+    assert not timed.engine.use_graphs
+    assert timed.generate(prompts, max_new_tokens=6, temperature=0.0, stop_tokens=()) == plain
+    report = dict((name, (calls, ms)) for name, calls, ms in ops.timing_report())
+    layers = TINY_B["num_hidden_layers"]
+    assert report["attention"][0] == 6 * layers and report["argmax"][0] == 6 and report["embed"][0] == 6
+    assert all(ms > 0 for _, ms in report.values())
+    assert ops.timing_report() == []
+
+
+def test_weights_held_once(tmp_path):
+    """``tiled_weights=False`` keeps no second copy of the matrices; the products then read the
+    matrices as loaded and give the same tokens."""
+    import torch
+    from libllm_amd import Model
+    path = make_model(tmp_path, TINY_B, seed=13)
+    prompts = [[5, 6, 7, 8, 9] * 15, [11, 12]]                      # 75 and 2 tokens: a prompt step of 77 rows
+    twice = Model(path, dtype="bfloat16", max_tokens=512)
+    once = Model(path, dtype="bfloat16", max_tokens=512, tiled_weights=False)
+    assert isinstance(once.engine.model.blocks[0].mixer.out.prepared, torch.Tensor)
+    assert not isinstance(twice.engine.model.blocks[0].mixer.out.prepared, torch.Tensor)
+    a = twice.generate(prompts, max_new_tokens=6, temperature=0.0, stop_tokens=())
+    assert once.generate(prompts, max_new_tokens=6, temperature=0.0, stop_tokens=()) == a

@@ -317,6 +317,65 @@ def test_layers_of_the_measured_shapes(tmp_path, shape):
             check(shape, cfg, weights, checked, traces.collect(steps, str(out_dir), cfg.vocab), dtype)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_a_prompt_of_thousands_of_rows(tmp_path, dtype):
+    """A prompt of 3,700 tokens in one step (beyond the captured prompt graphs; in bfloat16 the
+    form of prompt attention in which a wave takes two tiles of rows), then a second request in a
+    batch with its last tokens one by one across a page border, every position against the plain
+    implementation."""
+    cfg_dict = dict(TINY_A, max_position_embeddings=4096)
+    path = make_model(tmp_path, cfg_dict, seed=41, name="long")
+    cfg_json, weights = files.read_model_dir(path)
+    cfg = llama.PlainConfig(cfg_json)
+    requests = make_requests(cfg, [3700, 3650], seed=42)
+    steps = traces.whole({"r0": requests["r0"]}) + traces.batches([{"r1": requests["r1"]}], {"r1": 20})
+    for i, s in enumerate(steps):
+        s["step"] = i
+    out_dir = tmp_path / dtype
+    run_replay(path, dtype, steps, out_dir)
+    check("long", cfg, weights, requests, traces.collect(steps, str(out_dir), cfg.vocab), dtype)
+
+
+def test_the_1b_shape_whole_in_32_bit_and_bfloat16():
+    """All 16 layers of the measured 1B shape with its vocabulary of 128,256, random weights drawn
+    on the device, in true 32-bit and in bfloat16: an unequal batch of three prompts (247 rows: the
+    library's products in bfloat16), then four tokens each, the logits at the wanted places
+    against the plain implementation run on the same weights."""
+    import bench
+    from libllm_amd.config import config_from_dict
+    from libllm_amd.engine import StepEntry
+    from libllm_amd.runtime import random_engine
+    from libllm_amd.weights import random_tensors
+    config = config_from_dict(dict(bench.FULL, max_position_embeddings=4096))
+    cfg = llama.PlainConfig(config.to_dict())
+    rng = np.random.default_rng(77)
+    toks = {i: rng.integers(0, cfg.vocab, size=n + 4).tolist() for i, n in enumerate((200, 40, 7))}
+    weights, ref, rounded = None, {}, {}
+    for dtype in DTYPES:
+        engine = random_engine(config, seed=3, dtype=dtype, max_tokens=1024)
+        if weights is None:
+            # the random-weights mode draws every tensor from (seed, name): the same draw here
+            declared = engine.model.declared()
+            weights = {name: random_tensors({name: declared[name]}, 3, std=0.02, dtype=torch.bfloat16,
+                                            device="cuda")[name].double().cpu().numpy() for name in declared}
+            for i, t in toks.items():
+                rows = list(range(len(t) - 5, len(t)))
+                ref[i] = llama.lm_head(cfg, weights, llama.hidden_states(cfg, weights, t)[rows])
+                rounded[i] = llama.lm_head(cfg, weights, llama.hidden_states(cfg, weights, t, store=llama.to_bfloat16)[rows])
+        got = {i: [] for i in toks}
+        out = engine.step([StepEntry(i, t[:-4], [len(t) - 5]) for i, t in toks.items()])
+        for j, i in enumerate(toks):
+            got[i].append(out[j].double().cpu().numpy())
+        for k in range(4):
+            out = engine.step([StepEntry(i, [t[len(t) - 4 + k]], [0]) for i, t in toks.items()])
+            for j, i in enumerate(toks):
+                got[i].append(out[j].double().cpu().numpy())
+        for i in toks:
+            assert_logits_close(np.stack(got[i]), ref[i], dtype, "1b %s request %d" % (dtype, i),
+                                rounded[i] if dtype == "bfloat16" else None)
+        del engine
+
+
 ODD = {
     "width 100, feed-forward 150, vocabulary 101": dict(hidden_size=100, num_attention_heads=5, num_key_value_heads=5,
                                                         intermediate_size=150, vocab_size=101),
