@@ -102,31 +102,66 @@ class DecoderModel:
         return needs
 
     def graph_safe(self) -> bool:
-        """True if no part reads host-side step data, so a step can be captured and replayed."""
-        for block in self.blocks:
-            for part in [block.mixer, block.feed_forward] + list(block.norms):
-                if not getattr(part, "graph_safe", False):
-                    return False
-        return getattr(self.final_norm, "graph_safe", False) and getattr(self.head, "graph_safe", False)
+        """True if no part reads host-side step data, so a whole step can be captured."""
+        return all(safe for safe, _ in self.stretches()) and len(self.stretches()) == 1
 
-    # ---- one step over packed rows
+    # ---- one step over packed rows, in units: the embedding, every run of the schedule, the output
+    def n_units(self) -> int:
+        return len(self.spec.schedule) + 2
+
+    def unit_is_graph_safe(self, unit: int) -> bool:
+        """Whether a unit reads nothing from the host while it runs (so it can be captured)."""
+        n = len(self.spec.schedule)
+        if unit == 0:
+            return True
+        if unit == n + 1:
+            return getattr(self.final_norm, "graph_safe", False) and getattr(self.head, "graph_safe", False)
+        block = self.blocks[self.spec.schedule[unit - 1].layer]
+        return all(getattr(part, "graph_safe", False)
+                   for part in [block.mixer, block.feed_forward] + list(block.norms))
+
+    def stretches(self):
+        """The units of a step cut into runs of neighbours that are all graph-safe or all not:
+        [(safe, [units])].  A model whose parts all are gives one stretch."""
+        out = []
+        for unit in range(self.n_units()):
+            safe = self.unit_is_graph_safe(unit)
+            if out and out[-1][0] == safe:
+                out[-1][1].append(unit)
+            else:
+                out.append((safe, [unit]))
+        return out
+
+    def run_unit(self, unit: int, ctx: StepContext, stream: Optional[Stream], want_rows):
+        """Runs one unit.  Unit 0 returns the stream it has made from the tokens; the last unit
+        returns float32 logits (None if no row is wanted); the others return None."""
+        s = self.spec
+        n = len(s.schedule)
+        if unit == 0:
+            return Stream(ctx.ops.embed(self.embed_table, ctx.tokens, s.embedding.scale))
+        if unit == n + 1:
+            ctx.norm_after_block = None
+            if want_rows is None or want_rows.numel() == 0:
+                return None
+            h = self.final_norm.add_norm(ctx, stream, rows=want_rows,
+                                         lazy=getattr(self.head, "takes_normed", False))
+            return self.head.forward(ctx, h)
+        i = unit - 1
+        entry = s.schedule[i]
+        # the block is told which norm reads the stream after it, so that its last product
+        # may prepare that norm (the final norm gathers rows and is left alone)
+        nxt = s.schedule[i + 1] if i + 1 < n else None
+        ctx.norm_after_block = self.blocks[nxt.layer].entry_norm() if nxt is not None else None
+        self.blocks[entry.layer].forward(ctx, stream, entry)
+        return None
+
     def forward(self, ctx: StepContext, want_rows: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
         """Runs every token of the step through the schedule; returns float32 logits
         ``[len(want_rows), vocab]`` (None if no row is wanted)."""
-        s = self.spec
-        res = ctx.ops.embed(self.embed_table, ctx.tokens, s.embedding.scale)
-        stream = Stream(res)
-        for i, entry in enumerate(s.schedule):
-            # the block is told which norm reads the stream after it, so that its last product
-            # may prepare that norm (the final norm gathers rows and is left alone)
-            nxt = s.schedule[i + 1] if i + 1 < len(s.schedule) else None
-            ctx.norm_after_block = self.blocks[nxt.layer].entry_norm() if nxt is not None else None
-            self.blocks[entry.layer].forward(ctx, stream, entry)
-        ctx.norm_after_block = None
-        if want_rows is None or want_rows.numel() == 0:
-            return None
-        h = self.final_norm.add_norm(ctx, stream, rows=want_rows, lazy=getattr(self.head, "takes_normed", False))
-        return self.head.forward(ctx, h)
+        stream = self.run_unit(0, ctx, None, want_rows)
+        for unit in range(1, self.n_units() - 1):
+            self.run_unit(unit, ctx, stream, want_rows)
+        return self.run_unit(self.n_units() - 1, ctx, stream, want_rows)
 
 
 def declared_weights(spec: ModelSpec) -> Dict[str, WeightDecl]:

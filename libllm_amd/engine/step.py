@@ -54,8 +54,9 @@ class Engine:
         self.vocab = model.spec.vocab
         self.cache = SequenceCache(model.cache_needs(), model.state_needs(), max_tokens,
                                    model.spec.max_position, dtype, self.device, max_slots)
-        self.use_graphs = (bool(use_graphs) and ops.supports_graphs and model.graph_safe()
-                           and not getattr(ops, "timing", False))
+        # a part that reads the step's host-side data cannot be captured; the stretches of the
+        # schedule around it still are (see _CapturedForward)
+        self.use_graphs = bool(use_graphs) and ops.supports_graphs and not getattr(ops, "timing", False)
         self._graphs: Dict[tuple, "_DecodeGraph"] = {}     # (batch bucket, context bucket) -> graph
         self._prompt_graphs: Dict[tuple, "_PromptGraph"] = {}   # (rows, sequences) -> graph
         self._prompt_seen: Dict[tuple, int] = {}
@@ -238,6 +239,75 @@ class Engine:
         return graph.run([e.tokens[0] for e in entries], slots, pos0, tokens_device)
 
 
+class _CapturedForward:
+    """``model.forward`` over fixed device buffers, ready to be run again and again: the stretches
+    of units whose parts read nothing from the host are captured HIP graphs, the units between
+    them (a part with ``graph_safe = False``) run from the host each time, on the same stream.
+
+    What passes from one stretch to the next is the residual stream: its 32-bit sum, which the
+    parts change in place, and the rows still to be added.  A captured stretch leaves them at
+    fixed addresses; what a host-run unit returns lies somewhere new each time and is copied to
+    a buffer that the next captured stretch was captured with (a prepared norm that such a unit
+    may leave is dropped: the next norm then works from the sum itself).  The state of the stream
+    object at every border is kept from set-up, since a replayed graph runs no Python."""
+
+    def __init__(self, model, ops, ctx, want_rows):
+        self.model, self.ctx, self.want_rows = model, ctx, want_rows
+        self.pieces = []                 # (graph or None, units, border state after the piece)
+        self.stream = None
+        self.logits = None
+        last = model.n_units() - 1
+        for safe, units in model.stretches():
+            before = self.pieces[-1][2] if self.pieces else None
+            if safe:
+                # (the capture runs its body twice, once to warm up: each run starts from the
+                # stream as the piece before left it)
+                graph = ops.capture(lambda units=units, before=before: self._run(units, before))
+                graph.replay()           # its results are real for the host-run unit that may follow
+                self.pieces.append((graph, units, self._border()))
+            else:
+                self._run(units, before)
+                static = None
+                if self.stream.delta is not None:
+                    static = self.stream.delta.clone()
+                self.stream.delta, self.stream.pre = static, None
+                self.pieces.append((None, units, self._border()))
+        self.n_graphs = sum(1 for g, _, _ in self.pieces if g is not None)
+        self.n_host_pieces = len(self.pieces) - self.n_graphs
+        self.last_unit = last
+
+    def _run(self, units, before=None):
+        if before is not None:
+            self.stream.res, self.stream.delta, self.stream.pre = before
+        for unit in units:
+            out = self.model.run_unit(unit, self.ctx, self.stream, self.want_rows)
+            if unit == 0:
+                self.stream = out
+            elif unit == self.model.n_units() - 1:
+                self.logits = out
+
+    def _border(self):
+        return (self.stream.res, self.stream.delta, self.stream.pre)
+
+    def run(self):
+        """Runs the step that the buffers hold; returns the logits (None if no row is wanted)."""
+        before = None
+        for graph, units, border in self.pieces:
+            if graph is not None:
+                graph.replay()
+            else:
+                self._run(units, before)
+                res, delta, _ = border
+                if self.stream.res is not res:
+                    res.copy_(self.stream.res)
+                if (self.stream.delta is None) != (delta is None):
+                    raise RequestError("a part that runs from the host changed what it returns between steps")
+                if delta is not None:
+                    delta.copy_(self.stream.delta)
+            before = border
+        return self.logits
+
+
 class _DecodeGraph:
     """One captured decode step for a batch of exactly ``bucket`` rows whose sequences hold at
     most ``max_ctx`` tokens after the step.  Rows beyond the live sequences point at the cache's
@@ -275,16 +345,16 @@ class _DecodeGraph:
         engine._attach_cache(ctx)
         self.ctx = ctx
         self._fill([0] * b, [engine.cache.sink_slot] * b, [0] * b)
-        self.logits = None
-        self.graph = ops.capture(self._body)
-
-    def _body(self):
-        self.logits = self.model.forward(self.ctx, self.want_rows)
+        self.forward = _CapturedForward(self.model, ops, ctx, self.want_rows)
 
     def _fill(self, tokens, slots, pos0):
         b = self.bucket
         n = len(tokens)
         sink = self.sink_slot
+        # for the parts that run from the host: the padding rows are sequences in the sink slot
+        self.ctx.seq_lens = [1] * b
+        self.ctx.seq_slot_host = list(slots) + [sink] * (b - n)
+        self.ctx.seq_pos0_host = list(pos0) + [0] * (b - n)
         self.turn = (self.turn + 1) % self.RING
         if self.ring_done[self.turn] is not None:
             self.ring_done[self.turn].synchronize()        # its last upload has been read
@@ -309,8 +379,7 @@ class _DecodeGraph:
         self._fill(tokens, slots, pos0)
         if tokens_device is not None:
             self.static[:len(tokens)].copy_(tokens_device, non_blocking=True)
-        self.graph.replay()
-        return self.logits[:len(tokens)]
+        return self.forward.run()[:len(tokens)]
 
 
 class _PromptGraph:
@@ -348,16 +417,17 @@ class _PromptGraph:
         engine._attach_cache(ctx)
         self.ctx = ctx
         self._fill([], [], [], [], [])
-        self.logits = None
-        self.graph = ops.capture(self._body)
-
-    def _body(self):
-        self.logits = self.model.forward(self.ctx, self.want_rows)
+        self.forward = _CapturedForward(self.model, ops, ctx, self.want_rows)
 
     def _fill(self, tokens, slots, lens, pos0, want):
         t, b = self.rows, self.seqs
         n, m = len(lens), len(tokens)
         sink = self.sink_slot
+        # for the parts that run from the host: the spare sequence holds the rows left over, in
+        # the sink slot, and the sequences after it are empty
+        self.ctx.seq_lens = list(lens) + [t - m] + [0] * (b - n - 1)
+        self.ctx.seq_slot_host = list(slots) + [sink] * (b - n)
+        self.ctx.seq_pos0_host = list(pos0) + [0] * (b - n)
         self.turn = (self.turn + 1) % self.RING
         if self.ring_done[self.turn] is not None:
             self.ring_done[self.turn].synchronize()        # its last upload has been read
@@ -392,5 +462,5 @@ class _PromptGraph:
         want = [int(starts[i]) + int(w) for i, e in enumerate(entries) for w in e.want]
         tokens = np.concatenate([np.asarray(e.tokens, dtype=np.int64) for e in entries])
         self._fill(tokens, slots, lens, pos0, want)
-        self.graph.replay()
-        return self.logits[:len(want)] if want else None
+        logits = self.forward.run()
+        return logits[:len(want)] if want else None

@@ -167,7 +167,11 @@ def test_toy_mixer_registers_builds_and_steps(ops, dtype):
     model.bind({k: v.to("cuda", torch.float32 if (dtype == torch.float32 or v.dim() == 1) else dtype)
                 for k, v in t.items()}, ops, dtype)
     engine = Engine(model, ops, dtype, max_tokens=512)
-    assert not engine.use_graphs and list(engine.cache.state) == [1]
+    engine.PROMPT_SEEN = 1                               # prompt steps through captured graphs from the first
+    # the toy reads the step's sequences on the host: its layer runs from the host, the stretches
+    # of the schedule before and after it are captured graphs all the same
+    assert engine.use_graphs and [safe for safe, _ in model.stretches()] == [True, False, True]
+    assert list(engine.cache.state) == [1]
     w = {k: v.double().numpy() for k, v in t.items()}
     rng = np.random.default_rng(5)
     reqs = {"a": rng.integers(0, 256, size=30).tolist(), "b": rng.integers(0, 256, size=11).tolist()}
@@ -184,7 +188,17 @@ def test_toy_mixer_registers_builds_and_steps(ops, dtype):
     for rid, toks in (("a", reqs["a"]), ("b", reqs["b"]), ("c", reqs["b"])):
         ref = toy.toy_oracle(cfg, w, w["model.layers.1.toy.mix.weight"], toks)
         assert_logits_close(np.stack(got[rid]), ref, dtype, rid)
+    # a prompt of which only the last row is wanted goes through a captured prompt step too
+    d = rng.integers(0, 256, size=25).tolist()
+    rows = [engine.step([StepEntry("d", d[:20], [19])]).double().cpu().numpy()]
+    rows += [engine.step([StepEntry("d", [x], [0])]).double().cpu().numpy() for x in d[20:]]
+    engine.end(["d"])
+    ref = toy.toy_oracle(cfg, w, w["model.layers.1.toy.mix.weight"], d)
+    assert_logits_close(np.concatenate(rows), ref[19:], dtype, "d")
     engine.cache.check()
+    graphs = list(engine._graphs.values()) + list(engine._prompt_graphs.values())
+    assert engine._graphs and engine._prompt_graphs
+    assert all(g.forward.n_graphs == 2 and g.forward.n_host_pieces == 1 for g in graphs)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -199,7 +213,9 @@ def test_toy_routed_feed_forward_and_position_encoding(ops, dtype):
     model.bind({k: v.to("cuda", torch.float32 if (dtype == torch.float32 or v.dim() == 1) else dtype)
                 for k, v in t.items()}, ops, dtype)
     engine = Engine(model, ops, dtype, max_tokens=512)
-    assert not engine.use_graphs                          # the routed part reads on the host
+    # the routed part picks rows on the host's say: its layer runs from the host between two graphs
+    assert engine.use_graphs and [(safe, units) for safe, units in model.stretches()] == [
+        (True, [0, 1]), (False, [2]), (True, [3])]
     w = {k: v.double().numpy() for k, v in t.items()}
     ids = np.random.default_rng(8).integers(0, 256, size=100).tolist()
     ref, margin = toy.toys_oracle(cfg, w, ids)
