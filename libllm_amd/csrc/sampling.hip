@@ -326,7 +326,8 @@ __global__ __launch_bounds__(NT) void sample_final_kernel(const float* __restric
                                                            uint64_t seed,
                                                            const long long* __restrict__ streams,
                                                            const long long* __restrict__ counters,
-                                                           SampleParts in, int* __restrict__ out) {
+                                                           SampleParts in, int* __restrict__ out,
+                                                           int open_ended) {
   __shared__ float fbuf[NT / 64];
   __shared__ unsigned int hist[256], wsum[4];
   __shared__ unsigned long long cand[SP_KMAX];
@@ -456,6 +457,12 @@ __global__ __launch_bounds__(NT) void sample_final_kernel(const float* __restric
       ++n;
       if (kept >= top_p) break;
     }
+    if (open_ended && kept < top_p) {
+      // no limit on the candidates was asked for, and the most probable top_k of them do not
+      // reach top_p: the row is left to sample_nucleus_kernel, which walks the whole vocabulary
+      out[row] = -1;
+      return;
+    }
     const float r = u * kept;
     float run = 0.f;
     int pick = n - 1;
@@ -465,6 +472,156 @@ __global__ __launch_bounds__(NT) void sample_final_kernel(const float* __restric
     }
     out[row] = (int)(0xffffffffu - (uint32_t)(cand[pick] & 0xffffffffull));
   }
+}
+
+
+// Nucleus sampling without a limit on the candidates (top_k == 0, top_p < 1) for the rows that
+// sample_final_kernel has left (out[row] < 0: the SP_KMAX most probable tokens do not reach
+// top_p).  One block a row.  In the order of the draw (probability falling, the lower index first
+// among equals) the kept tokens are the shortest prefix whose probabilities sum to top_p or more,
+// and the drawn token is the first whose running sum exceeds r = u * (sum of the kept).  Both are
+// places where a running sum in that order crosses a mark, and each is found without sorting: by
+// a descent over the 32-bit order key of the logit, 8 bits a pass, over histograms of probability
+// instead of counts, then among the tokens of the last key (equal logits) by index.  Probabilities
+// are counted in units of 2^-40 as integers, so that the sums do not depend on the order in which
+// the threads add them.
+#define NUC_NT 1024
+#define NUC_ONE 1099511627776.0   // 2^40
+
+struct NucleusShared {
+  unsigned long long hist[256];
+  unsigned long long wsum[4];
+  unsigned long long above, pe, kept;
+  uint32_t prefix;
+  int bin, last_bin, pick, n_eq;
+  int ibuf[NUC_NT / 64];
+};
+
+__device__ __forceinline__ unsigned long long nucleus_mass(float x, float inv_temp, float mx, float inv_z) {
+  const float p = expf(x * inv_temp - mx) * inv_z;
+  return (unsigned long long)((double)p * NUC_ONE + 0.5);
+}
+
+// The token at which the running sum, in drawing order, first reaches `target` (strict: first
+// exceeds it).  Leaves its index in sh.pick and the running sum up to and including it in sh.kept.
+__device__ void nucleus_cross(const float* __restrict__ x, int V, float inv_temp, float mx, float inv_z,
+                              unsigned long long target, bool strict, NucleusShared& sh) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  if (tid == 0) { sh.prefix = 0u; sh.above = 0ull; }
+  __syncthreads();
+  for (int pass = 0; pass < 4; ++pass) {
+    const int shift = 24 - 8 * pass;
+    for (int b = tid; b < 256; b += NUC_NT) sh.hist[b] = 0ull;
+    if (tid == 0) { sh.bin = -1; sh.last_bin = -1; }
+    __syncthreads();
+    const uint32_t prefix = sh.prefix;
+    const unsigned long long above = sh.above;
+    // a thread adds up the tokens that follow one another into the same bin before it touches
+    // the histogram: the first passes have few bins, which all threads would crowd
+    int cur = -1;
+    unsigned long long acc = 0ull;
+    for (int i = tid; i < V; i += NUC_NT) {
+      const float v = x[i];
+      const uint32_t key = order_key(v);
+      if (pass != 0 && (key >> (shift + 8)) != prefix) continue;
+      const int b = (int)((key >> shift) & 255u);
+      if (b != cur) {
+        if (acc) atomicAdd(&sh.hist[cur], acc);
+        cur = b;
+        acc = 0ull;
+      }
+      acc += nucleus_mass(v, inv_temp, mx, inv_z);
+    }
+    if (acc) atomicAdd(&sh.hist[cur], acc);
+    __syncthreads();
+    // bins from the top: inclusive running sums by threads 0..255
+    unsigned long long v = 0ull, inc = 0ull;
+    if (tid < 256) {
+      v = sh.hist[255 - tid];
+      inc = v;
+#pragma unroll
+      for (int off = 1; off < 64; off <<= 1) {
+        const unsigned long long o = __shfl_up(inc, off, 64);
+        if (lane >= off) inc += o;
+      }
+      if (lane == 63) sh.wsum[wave] = inc;
+    }
+    __syncthreads();
+    if (tid < 256) {
+      for (int w = 0; w < wave; ++w) inc += sh.wsum[w];
+      const unsigned long long run = above + inc, before = run - v;
+      const bool crossed = strict ? run > target : run >= target;
+      const bool crossed_before = strict ? before > target : before >= target;
+      if (v != 0ull && crossed && !crossed_before) sh.bin = 255 - tid;
+      if (v != 0ull) atomicMax(&sh.last_bin, tid);           // the lowest bin that holds anything
+    }
+    __syncthreads();
+    if (tid == 0) {
+      // rounding may leave the whole sum short of the mark: the last token that has any
+      // probability then ends the walk
+      const int bin = sh.bin >= 0 ? sh.bin : (sh.last_bin >= 0 ? 255 - sh.last_bin : 0);
+      unsigned long long skipped = 0ull;
+      for (int b = 255; b > bin; --b) skipped += sh.hist[b];
+      sh.above = above + skipped;
+      sh.prefix = (prefix << 8) | (uint32_t)bin;
+    }
+    __syncthreads();
+  }
+  // the tokens whose key is the one found have equal logits and so equal probabilities: the
+  // c-th of them by index is the place
+  const uint32_t kth = sh.prefix;
+  const int chunk = (V + NUC_NT - 1) / NUC_NT;
+  const int c0 = min(V, tid * chunk), c1 = min(V, c0 + chunk);
+  int eq_mine = 0;
+  float eq_val = 0.f;
+  for (int i = c0; i < c1; ++i)
+    if (order_key(x[i]) == kth) { ++eq_mine; eq_val = x[i]; }
+  int eq_total;
+  const int eq_inc = block_inclusive_scan<int, NUC_NT>(eq_mine, sh.ibuf, &eq_total);
+  if (eq_mine > 0 && eq_inc == eq_mine) sh.pe = nucleus_mass(eq_val, inv_temp, mx, inv_z);   // the first thread that has one
+  if (tid == 0) { sh.n_eq = eq_total; sh.pick = 0; }
+  __syncthreads();
+  const unsigned long long pe = sh.pe, above = sh.above;
+  long long c = 1;
+  if (pe > 0ull && target >= above) {
+    const unsigned long long gap = target - above;
+    c = strict ? (long long)(gap / pe) + 1 : (long long)((gap + pe - 1) / pe);
+  }
+  if (c < 1) c = 1;
+  if (c > eq_total) c = eq_total;
+  const int rank0 = eq_inc - eq_mine;                        // equals before this thread's chunk
+  if (eq_mine > 0 && c > rank0 && c <= eq_inc) {
+    int rank = rank0;
+    for (int i = c0; i < c1; ++i)
+      if (order_key(x[i]) == kth && ++rank == c) { sh.pick = i; break; }
+    sh.kept = above + (unsigned long long)c * pe;
+  }
+  __syncthreads();
+}
+
+__global__ __launch_bounds__(NUC_NT) void sample_nucleus_kernel(const float* __restrict__ logits, int V,
+                                                               int parts, float inv_temp, float top_p,
+                                                               uint64_t seed,
+                                                               const long long* __restrict__ streams,
+                                                               const long long* __restrict__ counters,
+                                                               SampleParts in, int* __restrict__ out) {
+  __shared__ NucleusShared sh;
+  const int row = blockIdx.x;
+  if (out[row] >= 0) return;                                 // decided among the most probable tokens
+  const float* x = logits + (size_t)row * V;
+  const float* pm = in.part_max + (size_t)row * parts;
+  const float* ps = in.part_sum + (size_t)row * parts;
+  float mx = -INFINITY;
+  for (int p = 0; p < parts; ++p) mx = fmaxf(mx, pm[p]);
+  float Z = 0.f;
+  for (int p = 0; p < parts; ++p) Z += ps[p] * expf(pm[p] - mx);
+  const float inv_z = 1.0f / Z;
+  const double u = (double)counter_uniform(seed, (uint64_t)streams[row], (uint64_t)counters[row]);
+  nucleus_cross(x, V, inv_temp, mx, inv_z, (unsigned long long)((double)top_p * NUC_ONE), false, sh);
+  const unsigned long long kept = sh.kept;
+  __syncthreads();
+  nucleus_cross(x, V, inv_temp, mx, inv_z, (unsigned long long)(u * (double)kept), true, sh);
+  if (threadIdx.x == 0) out[row] = sh.pick;
 }
 
 // Parts a row of V logits is cut into, and candidates kept per part: the scratch arrays hold
@@ -487,9 +644,14 @@ extern "C" int llm_sample(const float* logits, int* out, int R, int V, float tem
                           unsigned long long* cand, hipStream_t stream) {
   if (R <= 0) return LLM_OK;
   if (V <= 0 || R > 65535 || !(temperature > 0.f) || top_k < 0 || top_k > SP_KMAX || top_k > V ||
-      !(top_p > 0.f && top_p <= 1.f) || (top_k == 0 && top_p < 1.f) || !part_max || !part_sum ||
-      (top_k > 0 && !cand))
+      !(top_p > 0.f && top_p <= 1.f) || !part_max || !part_sum)
     return LLM_ERR_ARG;
+  // top_k == 0 with top_p < 1: a nucleus with no limit on the candidates.  The SP_KMAX most
+  // probable tokens are tried first (nearly always they hold the nucleus); a row in which they
+  // do not reach top_p is then done by the kernel that walks the whole vocabulary.
+  const bool open_ended = top_k == 0 && top_p < 1.f;
+  if (open_ended) top_k = V < SP_KMAX ? V : SP_KMAX;
+  if (top_k > 0 && !cand) return LLM_ERR_ARG;
   const int parts = llm_sample_parts(V);
   if (parts > 65535) return LLM_ERR_ARG;
   const int per = (V + parts - 1) / parts;
@@ -499,6 +661,12 @@ extern "C" int llm_sample(const float* logits, int* out, int R, int V, float tem
   sample_part_kernel<<<dim3(parts, R), SP_NT, 0, stream>>>(logits, V, per, inv_temp, k_part, sp);
   if (hipGetLastError() != hipSuccess) return LLM_ERR_LAUNCH;
   sample_final_kernel<1024><<<R, 1024, 0, stream>>>(logits, V, per, parts, inv_temp, top_k, k_part,
-                                                    top_p, (uint64_t)seed, streams, counters, sp, out);
+                                                    top_p, (uint64_t)seed, streams, counters, sp, out,
+                                                    open_ended && top_k < V ? 1 : 0);
+  if (open_ended && top_k < V) {
+    if (hipGetLastError() != hipSuccess) return LLM_ERR_LAUNCH;
+    sample_nucleus_kernel<<<R, NUC_NT, 0, stream>>>(logits, V, parts, inv_temp, top_p, (uint64_t)seed,
+                                                    streams, counters, sp, out);
+  }
   return llm_launch_status();
 }

@@ -742,7 +742,8 @@ class HipOps:
         keys = torch.tensor([streams, counters], dtype=torch.int64).pin_memory().to(self.device, non_blocking=True)
         out = torch.empty((r,), dtype=torch.int32, device=self.device)
         parts = self.lib.llm_sample_parts(v)
-        k_part = self.lib.llm_sample_k_part(v, int(top_k))
+        # (no limit on the candidates and top_p below 1: the kernel first tries the most probable 1,024)
+        k_part = self.lib.llm_sample_k_part(v, int(top_k) if (top_k or top_p >= 1.0) else min(v, 1024))
         part_max = torch.empty((r * parts,), dtype=torch.float32, device=self.device)
         part_sum = torch.empty((r * parts,), dtype=torch.float32, device=self.device)
         cand = torch.empty((max(1, r * parts * k_part),), dtype=torch.int64, device=self.device)

@@ -4,7 +4,8 @@ The reference's order (src/libllm/generator.cc:197-214, 47-113): logits * (1/tem
 the top_k most probable tokens sorted from the largest, the shortest prefix of them whose
 probabilities reach top_p, then one draw in proportion to the probabilities kept.  It has no
 greedy class; top_k == 1 is arg-max (src/flint/cuda/test.cc:385-392).  Here temperature 0 and
-top_k 1 are arg-max (lowest index wins a tie), top_k 0 means no limit, and the uniform number of a
+top_k 1 are arg-max (lowest index wins a tie), top_k 0 means no limit (with top_p below 1 the
+nucleus is then taken over the whole vocabulary), and the uniform number of a
 draw comes from a counter hash of (seed, stream, counter): the same request draws the same tokens
 whatever else is in its batch.
 """
@@ -38,10 +39,7 @@ class SamplingParams:
             return SamplingParams(self.temperature, k, self.top_p, self.seed)
         if k > TOP_K_MAX:
             raise RequestError("top_k above %d is not supported (0 means no limit)" % TOP_K_MAX)
-        if k == 0 and self.top_p < 1.0:
-            if vocab > TOP_K_MAX:
-                raise RequestError("top_p below 1 needs top_k between 1 and %d" % TOP_K_MAX)
-            k = vocab
+        # k == 0 with top_p < 1: the nucleus over the whole vocabulary, however many tokens it takes
         return SamplingParams(self.temperature, k, self.top_p, self.seed)
 
     @property

@@ -127,13 +127,12 @@ def test_sampling_params():
     assert SamplingParams().validate(v) == SamplingParams(1.0, 50, 0.8, 0)   # src/libllm/llm.cc:125-132
     assert SamplingParams(0.0, 50, 0.8).greedy and SamplingParams(1.0, 1, 0.8).greedy
     assert SamplingParams(1.0, 5000, 1.0).validate(v).top_k == 0             # clamped, not an abort
-    assert SamplingParams(1.0, 0, 0.5).validate(v).top_k == v                # the nucleus needs an order
+    assert SamplingParams(1.0, 0, 0.5).validate(v).top_k == 0                # a nucleus with no limit on its size
+    assert SamplingParams(1.0, 0, 0.9).validate(128256) == SamplingParams(1.0, 0, 0.9, 0)
     for bad in (SamplingParams(-1.0), SamplingParams(1.0, -1), SamplingParams(1.0, 5, 0.0),
                 SamplingParams(1.0, 5, 1.5), SamplingParams(1.0, 2000, 0.9)):
         with pytest.raises(RequestError):
             bad.validate(128256)
-    with pytest.raises(RequestError):
-        SamplingParams(1.0, 0, 0.9).validate(128256)
 
     class Ops:
         def argmax(self, logits):

@@ -912,8 +912,6 @@ def test_sampling_matches_plain(ops):
         streams = list(range(100, 124))
         counters = list(range(24))
         k = 0 if top_k >= vocab else top_k
-        if k == 0 and top_p < 1.0:
-            k = vocab
         got = ops.sample(logits.cuda(), temp, k, top_p, 77, streams, counters).tolist()
         bad = 0
         for r in range(24):
@@ -924,6 +922,38 @@ def test_sampling_matches_plain(ops):
                 assert sampling.margin(logits[r].double().numpy(), temp, k, top_p, u) < 1e-5, (vocab, r)
                 bad += 1
         assert bad <= 2
+
+
+@pytest.mark.parametrize("vocab", [5003, 128256])
+def test_nucleus_without_a_limit_on_the_candidates(ops, vocab):
+    """top_k 0 with top_p below 1 (the reference's sampler takes any top_k up to the vocabulary,
+    src/libllm/generator.cc:66-90): the nucleus is the shortest prefix, in falling probability,
+    that reaches top_p, however long.  Rows whose nucleus lies within the most probable 1,024
+    tokens, rows as flat as to need most of the vocabulary (the walk over the whole vocabulary),
+    and a row of few distinct values (equal logits are ranked by index)."""
+    from plain import sampling
+    g = torch.Generator().manual_seed(vocab)
+    peaked = torch.randn((8, vocab), generator=g) * 4.0
+    flat = torch.randn((8, vocab), generator=g) * 0.3
+    stepped = torch.randint(0, 3, (8, vocab), generator=g).float() * 1.5
+    logits = torch.cat([peaked, flat, stepped])
+    rows = logits.shape[0]
+    streams, counters = list(range(50, 50 + rows)), list(range(rows))
+    for top_p, temp in ((0.9, 1.0), (0.5, 0.7), (0.999, 1.5)):
+        got = ops.sample(logits.cuda(), temp, 0, top_p, 99, streams, counters).tolist()
+        bad, long_ones = 0, 0
+        for r in range(rows):
+            row = logits[r].double().numpy()
+            u = sampling.uniform(99, streams[r], counters[r])
+            labels, _ = sampling.candidates(row, temp, 0, top_p)
+            long_ones += len(labels) > 1024
+            want = sampling.sample(row, temp, 0, top_p, u)
+            if got[r] != want:
+                # only a draw within rounding of a boundary of the running sum may differ (with equal
+                # logits a boundary moves the pick to a neighbour of equal probability)
+                assert sampling.margin(row, temp, 0, top_p, u) < 1e-5 and got[r] in labels, (vocab, top_p, r)
+                bad += 1
+        assert bad <= 2 and long_ones >= 8                      # the long walk was taken
 
 
 def test_sampling_seed_and_top1(ops):
