@@ -46,6 +46,12 @@ __device__ __forceinline__ void load16_uncounted(u32x4v& dst, const void* p) {
   asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(dst) : "v"(p) : "memory");
 }
 
+// The same with the non-temporal hint, for the weights, which are read once: they then do not push
+// the rows of X out of the chiplet's cache (1 to 2 % of a decode step at batches of 96 and 128).
+__device__ __forceinline__ void load16_uncounted_stream(u32x4v& dst, const void* p) {
+  asm volatile("global_load_dwordx4 %0, %1, off nt" : "=&v"(dst) : "v"(p) : "memory");
+}
+
 template <int MT, int EPI, typename OutT>
 __global__ __launch_bounds__(MID_NT, 2) void gemm_mid_kernel(const bf16_t* __restrict__ X,
                                                              const bf16_t* __restrict__ W,
@@ -146,7 +152,7 @@ __global__ __launch_bounds__(MID_NT, 2) void gemm_mid_kernel(const bf16_t* __res
     for (int u = 0; u < US; ++u)
 #pragma unroll
       for (int rt = 0; rt < MID_RT; ++rt)
-        load16_uncounted(dst[u][rt], chunk <= last ? wp[rt] + (size_t)(s0 + u) * 512 : W);
+        load16_uncounted_stream(dst[u][rt], chunk <= last ? wp[rt] + (size_t)(s0 + u) * 512 : W);
   };
   auto compute = [&](int buf, u32x4v (&src)[US][MID_RT]) {
 #pragma unroll

@@ -156,7 +156,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
         const int s = chunk * (CK / 32) + gi * 16 + wk * 2 + u;
         const bool in = s < n_steps && (s * 32 + g * 8) < K;
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt) dst[gi][u][rt] = in ? frag_load(wp[rt] + (size_t)s * wstep) : frag_zero();
+        for (int rt = 0; rt < RT; ++rt) dst[gi][u][rt] = in ? frag_load_stream(wp[rt] + (size_t)s * wstep) : frag_zero();
       }
   };
   auto compute = [&](Frag (&src)[G][2][RT]) {
