@@ -23,6 +23,23 @@ __global__ __launch_bounds__(256) void peak_read_kernel(const uint4* __restrict_
   sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = acc;
 }
 
+// The same with the non-temporal hint on every load, as the products stream their weights.
+typedef uint32_t peak_u32x4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void peak_read_stream_kernel(const peak_u32x4* __restrict__ src, size_t n16,
+                                                               uint32_t* __restrict__ sink) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  peak_u32x4 acc = {0u, 0u, 0u, 0u};
+  for (; i + 3 * stride < n16; i += 4 * stride) {
+    const peak_u32x4 a = __builtin_nontemporal_load(src + i), b = __builtin_nontemporal_load(src + i + stride),
+                     c = __builtin_nontemporal_load(src + i + 2 * stride),
+                     d = __builtin_nontemporal_load(src + i + 3 * stride);
+    acc ^= a ^ b ^ c ^ d;
+  }
+  for (; i < n16; i += stride) acc ^= __builtin_nontemporal_load(src + i);
+  sink[(size_t)blockIdx.x * blockDim.x + threadIdx.x] = acc.x ^ acc.y ^ acc.z ^ acc.w;
+}
+
 __global__ __launch_bounds__(256) void peak_copy_kernel(const uint4* __restrict__ src,
                                                         uint4* __restrict__ dst, size_t n16) {
   const size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -81,12 +98,16 @@ extern "C" int llm_peak_sink_words() { return peak_blocks(8) * 256; }
 // half_blocks_per_unit: blocks of 256 threads for every two compute units (1 to 16).  The grid's
 // size decides how far apart in memory the loads of one moment lie, and with it the bandwidth: a
 // block or two a unit reads a sixth faster than eight (6.4 against 5.4 TB/s on an MI355X).
+// streaming: the loads carry the non-temporal hint.
 extern "C" int llm_peak_read(const void* src, size_t bytes, void* sink, int half_blocks_per_unit,
-                             hipStream_t stream) {
+                             int streaming, hipStream_t stream) {
   if (!src || !sink || bytes < 16 || (((uintptr_t)src) & 15) || half_blocks_per_unit < 1 || half_blocks_per_unit > 16)
     return LLM_ERR_ARG;
   const int blocks = (peak_blocks(half_blocks_per_unit) + 1) / 2;
-  peak_read_kernel<<<blocks, 256, 0, stream>>>((const uint4*)src, bytes / 16, (uint32_t*)sink);
+  if (streaming)
+    peak_read_stream_kernel<<<blocks, 256, 0, stream>>>((const peak_u32x4*)src, bytes / 16, (uint32_t*)sink);
+  else
+    peak_read_kernel<<<blocks, 256, 0, stream>>>((const uint4*)src, bytes / 16, (uint32_t*)sink);
   return llm_launch_status();
 }
 

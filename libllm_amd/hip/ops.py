@@ -58,7 +58,7 @@ _SIGNATURES = {
     "llm_sample_parts": [_i],
     "llm_sample_k_part": [_i, _i],
     "llm_peak_sink_words": [],
-    "llm_peak_read": [_vp, ctypes.c_size_t, _vp, _i, _vp],
+    "llm_peak_read": [_vp, ctypes.c_size_t, _vp, _i, _i, _vp],
     "llm_peak_copy": [_vp, _vp, ctypes.c_size_t, _i, _vp],
     "llm_peak_mfma_bf16": [_vp, _i, ctypes.POINTER(ctypes.c_double), _vp],
     "llm_peak_fma_f32": [_vp, _i, ctypes.POINTER(ctypes.c_double), _vp],
@@ -709,8 +709,9 @@ class HipOps:
             return min(times)
         out = {}
         grids = (2, 3, 4, 6, 16)        # blocks for every two compute units
-        t = min(best(lambda g=g: self.lib.llm_peak_read(src.data_ptr(), nbytes, sink.data_ptr(), g, self._stream()))
-                for g in grids)
+        t = min(best(lambda g=g, nt=nt: self.lib.llm_peak_read(src.data_ptr(), nbytes, sink.data_ptr(), g, nt,
+                                                               self._stream()))
+                for g in grids for nt in (0, 1))
         out["read_GBs"] = nbytes / t / 1e9
         t = min(best(lambda g=g: self.lib.llm_peak_copy(src.data_ptr(), dst.data_ptr(), nbytes, g, self._stream()))
                 for g in grids)
