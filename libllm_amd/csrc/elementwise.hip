@@ -29,6 +29,49 @@ extern "C" int llm_embed(const void* table, int table_dtype, const int* ids, flo
   return llm_launch_status();
 }
 
+// The same, and what the RMS norm that reads these rows next needs from them (see the head of
+// gemm_skinny.hip): raw[m, :] = bfloat16(out[m, :] * norm_w) and ssq[m, t], the sum of squares of
+// out[m, 16 t .. 16 t + 15].  H is a multiple of 16; four threads share a tile of 16 columns.
+template <typename T>
+__global__ __launch_bounds__(256) void embed_norm_kernel(const T* __restrict__ table, const int* __restrict__ ids,
+                                                         float* __restrict__ out, int H, int V, float scale,
+                                                         const float* __restrict__ norm_w,
+                                                         bf16_t* __restrict__ raw, float* __restrict__ ssq) {
+  const int m = blockIdx.x;
+  int id = ids[m];
+  if (id < 0 || id >= V) id = 0;
+  const T* row = table + (size_t)id * H;
+  for (int i4 = threadIdx.x; i4 < H / 4; i4 += 256) {       // H / 4 is a multiple of 4: a tile's threads go together
+    float4 v = Conv4<T>::load(row + i4 * 4);
+    v.x *= scale; v.y *= scale; v.z *= scale; v.w *= scale;
+    *reinterpret_cast<float4*>(out + (size_t)m * H + i4 * 4) = v;
+    const float4 w = *reinterpret_cast<const float4*>(norm_w + i4 * 4);
+    Conv4<bf16_t>::store(raw + (size_t)m * H + i4 * 4, make_float4(v.x * w.x, v.y * w.y, v.z * w.z, v.w * w.w));
+    float ss = v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    ss += __shfl_xor(ss, 1, 64);
+    ss += __shfl_xor(ss, 2, 64);
+    if ((threadIdx.x & 3) == 0) ssq[(size_t)m * (H / 16) + i4 / 4] = ss;
+  }
+}
+
+extern "C" int llm_embed_norm(const void* table, int table_dtype, const int* ids, float* out, int M, int H,
+                              int V, float scale, const float* norm_w, void* raw, float* ssq,
+                              hipStream_t stream) {
+  if (M <= 0) return LLM_OK;
+  if (H <= 0 || (H & 15) || V <= 0 || !norm_w || !raw || !ssq ||
+      ((((uintptr_t)table) | ((uintptr_t)out) | ((uintptr_t)norm_w) | ((uintptr_t)raw)) & 15))
+    return LLM_ERR_ARG;
+  if (table_dtype == LLM_DTYPE_F32)
+    embed_norm_kernel<float><<<M, 256, 0, stream>>>((const float*)table, ids, out, H, V, scale, norm_w,
+                                                     (bf16_t*)raw, ssq);
+  else if (table_dtype == LLM_DTYPE_BF16)
+    embed_norm_kernel<bf16_t><<<M, 256, 0, stream>>>((const bf16_t*)table, ids, out, H, V, scale, norm_w,
+                                                      (bf16_t*)raw, ssq);
+  else
+    return LLM_ERR_ARG;
+  return llm_launch_status();
+}
+
 // ---------------------------------------------------------------------------------- add + RMS norm
 // For output row b (input row r = rows ? rows[b] : b):
 //   x = res[r] + delta[r] (stored back into res when delta is given)

@@ -138,12 +138,24 @@ class DecoderModel:
         s = self.spec
         n = len(s.schedule)
         if unit == 0:
+            # if a plain RMS norm reads the rows first, the embedding kernel may prepare it
+            first = self.blocks[s.schedule[0].layer].entry_norm() if n else self.final_norm
+            terms = first.rms_terms() if first is not None and (n or ctx.want_all_rows) else None
+            if terms is not None and hasattr(ctx.ops, "embed_prepared"):
+                got = ctx.ops.embed_prepared(self.embed_table, ctx.tokens, s.embedding.scale, terms[0], terms[1],
+                                             ctx.dtype)
+                if got is not None:
+                    stream = Stream(got[0])
+                    stream.pre = got[1]
+                    return stream
             return Stream(ctx.ops.embed(self.embed_table, ctx.tokens, s.embedding.scale))
         if unit == n + 1:
             ctx.norm_after_block = None
             if want_rows is None or want_rows.numel() == 0:
                 return None
-            h = self.final_norm.add_norm(ctx, stream, rows=want_rows,
+            # every row wanted, in order: no gather, and the product before may have prepared the norm
+            rows = None if ctx.want_all_rows else want_rows
+            h = self.final_norm.add_norm(ctx, stream, rows=rows,
                                          lazy=getattr(self.head, "takes_normed", False))
             return self.head.forward(ctx, h)
         i = unit - 1
@@ -151,7 +163,10 @@ class DecoderModel:
         # the block is told which norm reads the stream after it, so that its last product
         # may prepare that norm (the final norm gathers rows and is left alone)
         nxt = s.schedule[i + 1] if i + 1 < n else None
-        ctx.norm_after_block = self.blocks[nxt.layer].entry_norm() if nxt is not None else None
+        if nxt is not None:
+            ctx.norm_after_block = self.blocks[nxt.layer].entry_norm()
+        else:
+            ctx.norm_after_block = self.final_norm if ctx.want_all_rows else None
         self.blocks[entry.layer].forward(ctx, stream, entry)
         return None
 

@@ -184,6 +184,7 @@ class Engine:
         ctx.max_new = max(lens)
         ctx.max_ctx = max(p + n for p, n in zip(pos0, lens))
         ctx.decode = all(n == 1 for n in lens)
+        ctx.want_all_rows = want == list(range(m))
         self._attach_cache(ctx)
         return ctx, want_rows
 
@@ -342,6 +343,7 @@ class _DecodeGraph:
         ctx.max_ctx = max_ctx
         ctx.decode = True
         ctx.captured = True
+        ctx.want_all_rows = True       # the graph's wanted rows are all its rows, in order
         engine._attach_cache(ctx)
         self.ctx = ctx
         self._fill([0] * b, [engine.cache.sink_slot] * b, [0] * b)

@@ -32,6 +32,7 @@ def _code(dtype: torch.dtype) -> int:
 
 _SIGNATURES = {
     "llm_embed": [_vp, _i, _vp, _vp, _i, _i, _i, _f, _vp],
+    "llm_embed_norm": [_vp, _i, _vp, _vp, _i, _i, _i, _f, _vp, _vp, _vp, _vp],
     "llm_add_rmsnorm": [_vp, _vp, _i, _i, ctypes.c_size_t, _vp, _f, _vp, _i, _vp, _i, _i, _vp],
     "llm_silu_mul": [_vp, _vp, _i, _i, _i, _vp],
     "llm_add_bias": [_vp, _i, _vp, _i, _i, _vp],
@@ -164,7 +165,7 @@ class HipOps:
             self.start_timing()
 
     # ---- time per operation, behind a switch
-    _TIMED = ("embed", "add_rmsnorm", "linear", "linear_swiglu", "silu_mul", "qkv_rope", "rope_kv_write",
+    _TIMED = ("embed", "embed_prepared", "add_rmsnorm", "linear", "linear_swiglu", "silu_mul", "qkv_rope", "rope_kv_write",
               "attention", "argmax", "sample")
 
     def start_timing(self) -> None:
@@ -275,6 +276,25 @@ class HipOps:
                                        self._dev(ids, "token ids", torch.int32), out.data_ptr(),
                                        m, h, v, float(scale), self._stream()), "embed")
         return out
+
+    def embed_prepared(self, table, ids, scale, weight, eps, dtype):
+        """The embedding, and in the same kernel what the RMS norm with ``weight`` and ``eps`` that
+        reads these rows first needs (a ``Prenormed``, as ``linear(..., then_norm=)`` returns):
+        (rows, record), or None where that does not apply (more than ``ACCUM_ROWS`` rows, another
+        activation dtype than bfloat16, a width that is no multiple of 16)."""
+        v, h = table.shape
+        m = ids.shape[0]
+        if not (self.fold_norms and self.fast_gemm and dtype == torch.bfloat16 and m <= self.ACCUM_ROWS and h % 16 == 0):
+            return None
+        self._dev(weight, "norm weight", torch.float32, (h,))
+        out = torch.empty((m, h), dtype=torch.float32, device=self.device)
+        raw = torch.empty((m, h), dtype=torch.bfloat16, device=self.device)
+        ssq = torch.empty((m, h // 16), dtype=torch.float32, device=self.device)
+        self._check(self.lib.llm_embed_norm(self._dev(table, "embedding table"), _code(table.dtype),
+                                            self._dev(ids, "token ids", torch.int32), out.data_ptr(), m, h, v,
+                                            float(scale), weight.data_ptr(), raw.data_ptr(), ssq.data_ptr(),
+                                            self._stream()), "embed_norm")
+        return out, Prenormed(raw, ssq, weight, float(eps))
 
     def add_rmsnorm(self, res, delta, weight, eps, out_dtype, rows=None):
         m, h = res.shape

@@ -118,6 +118,7 @@ class StepContext:
         self.then_norm = None
         self.norm_after_block = None   # the norm that reads the stream first after the running block, if known
         self.captured = False      # running under graph capture: host lists are not valid
+        self.want_all_rows = False  # the logits of every row are wanted, in order (a decode step): the last norm gathers nothing
         self._kv: Dict[int, KVView] = {}
         self._state: Dict[int, torch.Tensor] = {}
 

@@ -471,9 +471,10 @@ def test_padding_changes_nothing(models):
 @pytest.mark.parametrize("name", list(CONFIGS))
 def test_norms_between_products_get_no_kernel(models, name):
     """Decoding up to 16 rows in bfloat16, the product that adds into the stream prepares the RMS
-    norm after it and the next product applies the row's scale: the norm kernel then runs only
-    for the first norm of a step and the last.  Logits against the plain implementation, and
-    against an engine that runs every norm as a kernel."""
+    norm after it and the next product applies the row's scale; the embedding prepares the first
+    norm of a step in the same way, and where every row's logits are wanted the last product
+    prepares the final norm: the norm kernel then does not run at all.  Logits against the plain
+    implementation, and against an engine that runs every norm as a kernel."""
     from libllm_amd.runtime import load_engine
     path, cfg, weights = models[name]
     requests = make_requests(cfg, [9, 30, 17, 6], seed=45)
@@ -491,7 +492,7 @@ def test_norms_between_products_get_no_kernel(models, name):
     n_layers = len(folded.model.spec.schedule)
     prompt = 2 * n_layers                                       # the prompt step: more than 16 rows, no logits wanted
     assert calls["kernels"] == prompt + 4 * (2 * n_layers + 1)
-    assert calls["folded"] == prompt + 4 * 2
+    assert calls.get("folded", 0) == prompt
     assert_logits_close(a, b.astype(np.float64), "bfloat16", "folded norms against norm kernels")
     for i, (rid, toks) in enumerate(requests.items()):
         ref, rounded = oracle(name, cfg, weights, toks), oracle(name, cfg, weights, toks, rounded=True)
