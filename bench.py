@@ -111,6 +111,9 @@ def time_decode(gen, params, torch, batch, context, steps, warmup, vocab):
 
 
 def time_prefill(engine, torch, tokens, vocab, reps):
+    """Seconds of one prompt step of ``tokens`` tokens with the last row's logits wanted: the best
+    of ``reps`` runs after the first (the second run of a shape captures its graph, the later ones
+    replay it; the first replays still run slower than the ones after)."""
     from libllm_amd.engine import StepEntry
     g = torch.Generator().manual_seed(99)
     prompt = torch.randint(0, vocab, (tokens,), generator=g).tolist()
@@ -236,7 +239,7 @@ def main() -> int:
     log("measured on this GPU: read %.0f GB/s, copy %.0f GB/s, bf16 matrix cores %.0f TFLOP/s, fp32 %.1f TFLOP/s"
         % (peaks["read_GBs"], peaks["copy_GBs"], peaks["bf16_TFs"], peaks["fp32_TFs"]))
 
-    pre_s = time_prefill(engine, torch, args.prefill, vocab, reps=3)
+    pre_s = time_prefill(engine, torch, args.prefill, vocab, reps=10)
     pf = prefill_flops(cfg, args.prefill)
     log("prefill of %d tokens: %.2f ms" % (args.prefill, pre_s * 1e3))
 
