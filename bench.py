@@ -158,7 +158,7 @@ def run_workload(args, torch):
     gen = Generator(engine, Sampler(engine.ops, cfg.vocab_size), (), cfg.max_position_embeddings,
                     engine.cache.n_pages, PAGE, max_batch=64)
     result = None
-    for rep in range(2):                                   # the first run warms up and captures graphs
+    for rep in range(3):                                   # the first run warms up; a shape's second coming captures its graph
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         first = []
