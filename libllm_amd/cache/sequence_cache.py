@@ -22,6 +22,7 @@ import torch
 
 from ..errors import CacheError
 from ..parts.base import CacheNeed, KVView, StateNeed
+from .layout import key_pages_shape, value_pages_shape
 from .pages import PagePool, SlotTable
 
 PAGE = 64
@@ -50,11 +51,10 @@ class CacheGroup:
         self.n_pages = n_pages
         self.sink_page = n_pages
         self.pages_per_seq = pages_per_seq
-        # keys lie [position, dim] in a page, values transposed [dim, position]: both are then
-        # read along their contiguous axis by the matrix-core attention kernels
-        self.k = torch.zeros((len(entries), n_pages + 1, need.n_kv_heads, PAGE, need.head_dim),
+        # keys in blocks of 16 dims, values in halves of 32 positions: see layout.py
+        self.k = torch.zeros((len(entries),) + key_pages_shape(n_pages + 1, need.n_kv_heads, need.head_dim),
                              dtype=dtype, device=device)
-        self.v = torch.zeros((len(entries), n_pages + 1, need.n_kv_heads, need.head_dim, PAGE),
+        self.v = torch.zeros((len(entries),) + value_pages_shape(n_pages + 1, need.n_kv_heads, need.head_dim),
                              dtype=dtype, device=device)
         self.table_host = np.full((n_slots + 1, pages_per_seq), self.sink_page, dtype=np.int32)
         self.table = torch.from_numpy(self.table_host.copy()).to(device)

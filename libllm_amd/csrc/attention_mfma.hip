@@ -66,7 +66,7 @@ struct AttnState {
   float l;            // running sum of exp2(score - m)
 };
 
-// One page.  kpage: [64][HD] keys; vpage: [HD][64] values; q: B fragments of this lane's query;
+// One page of one kv head, laid out as common.h says.  q: B fragments of this lane's query;
 // key0: absolute position of the page's first key; [kmin, kmax]: keys this lane's query may see.
 template <int HD>
 __device__ __forceinline__ void attn_page(const bf16_t* __restrict__ kpage,
@@ -79,12 +79,11 @@ __device__ __forceinline__ void attn_page(const bf16_t* __restrict__ kpage,
 #pragma unroll
   for (int t4 = 0; t4 < 4; ++t4) {
     const int key_row = (t4 >> 1) * 32 + 8 * (r >> 2) + 4 * (t4 & 1) + (r & 3);
-    const bf16_t* krow = kpage + (size_t)key_row * HD;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d = ks * 32 + g * 8;
-      const Frag a = (d < HD) ? frag_load(krow + d) : frag_zero();
+      const Frag a = (d < HD) ? frag_load(kpage + llm_key_offset(key_row, d)) : frag_zero();
       acc = mfma_bf16(a, q[ks], acc);
     }
 #pragma unroll
@@ -123,9 +122,9 @@ __device__ __forceinline__ void attn_page(const bf16_t* __restrict__ kpage,
     f32x4 o = st.o[dt];
 #pragma unroll
     for (int e = 0; e < 4; ++e) o[e] *= corr;
-    const bf16_t* vrow = vpage + (size_t)(dt * 16 + r) * PAGE + 8 * g;
+    const bf16_t* vrow = vpage + llm_value_offset(HD, dt * 16 + r, 8 * g);
     o = mfma_bf16(frag_load(vrow), p[0], o);
-    o = mfma_bf16(frag_load(vrow + 32), p[1], o);
+    o = mfma_bf16(frag_load(vrow + HD * 32), p[1], o);      // the same dims of positions 32 ..
     st.o[dt] = o;
   }
 }
@@ -189,15 +188,17 @@ template <int HD>
 __device__ __forceinline__ void stage_page(unsigned char* k_lds, unsigned char* v_lds,
                                            const u32x4 (&kreg)[(8 * HD + 255) / 256],
                                            const u32x4 (&vreg)[(8 * HD + 255) / 256]) {
-  constexpr int PIECES = 8 * HD, LOADS = (PIECES + 255) / 256, KPR = HD / 8, KRB = KeyRow<HD>::BYTES;
+  constexpr int PIECES = 8 * HD, LOADS = (PIECES + 255) / 256, KRB = KeyRow<HD>::BYTES;
 #pragma unroll
   for (int j = 0; j < LOADS; ++j) {
     const int ci = threadIdx.x + j * 256;
     if (PIECES % 256 == 0 || ci < PIECES) {
-      const int krow = ci / KPR, kc = ci % KPR;
+      // piece ci of the page as it lies in memory: keys in blocks of 16 dims (two pieces a key)
+      const int krow = (ci & 127) >> 1, kc = ((ci >> 7) << 1) | (ci & 1);
       const int kf = (krow & 3) | (((krow >> 3) & 1) << 2);
       *reinterpret_cast<u32x4*>(k_lds + krow * KRB + (((kc & ~7) | ((kc & 7) ^ kf)) * 16)) = kreg[j];
-      const int vrow = ci >> 3, vc = ci & 7;
+      // values in halves of 32 positions (four pieces a dim and half)
+      const int vrow = (ci % (4 * HD)) >> 2, vc = ((ci / (4 * HD)) << 2) | (ci & 3);
       *reinterpret_cast<u32x4*>(v_lds + vrow * 128 + ((vc ^ (vrow & 7)) * 16)) = vreg[j];
     }
   }
@@ -407,11 +408,10 @@ __device__ __forceinline__ void load_keys(const bf16_t* __restrict__ kpage, Page
 #pragma unroll
   for (int t4 = 0; t4 < 4; ++t4) {
     const int key_row = (t4 >> 1) * 32 + 8 * (r >> 2) + 4 * (t4 & 1) + (r & 3);
-    const bf16_t* krow = kpage + (size_t)key_row * HD;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const int d = ks * 32 + g * 8;
-      f.k[t4][ks] = (d < HD) ? frag_load(krow + d) : frag_zero();
+      f.k[t4][ks] = (d < HD) ? frag_load_stream(kpage + llm_key_offset(key_row, d)) : frag_zero();
     }
   }
 }
@@ -421,9 +421,9 @@ __device__ __forceinline__ void load_values(const bf16_t* __restrict__ vpage, Pa
   const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
 #pragma unroll
   for (int dt = 0; dt < HD / 16; ++dt) {
-    const bf16_t* vrow = vpage + (size_t)(dt * 16 + r) * PAGE + 8 * g;
-    f.v[dt][0] = frag_load(vrow);
-    f.v[dt][1] = frag_load(vrow + 32);
+    const bf16_t* vrow = vpage + llm_value_offset(HD, dt * 16 + r, 8 * g);
+    f.v[dt][0] = frag_load_stream(vrow);
+    f.v[dt][1] = frag_load_stream(vrow + HD * 32);
   }
 }
 

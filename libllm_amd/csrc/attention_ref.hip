@@ -34,14 +34,15 @@ __global__ __launch_bounds__(64) void attention_ref_kernel(
   const int* trow = table + (size_t)slot * table_stride;
   for (int pg = k_first / PAGE; pg <= pos / PAGE; ++pg) {
     const int page = trow[pg];
-    const size_t base = ((size_t)page * n_kv + kvh) * PAGE * hd;
+    const size_t kbase = ((size_t)page * n_kv + kvh) * llm_key_block(hd);
+    const size_t vbase = ((size_t)page * n_kv + kvh) * llm_value_block(hd);
     const int key = pg * PAGE + lane;
     const bool valid = key >= k_first && key <= pos;
     float s = -INFINITY;
     if (valid) {
-      const T* kr = k_pages + base + (size_t)lane * hd;
+      const T* kr = k_pages + kbase;
       float dot = 0.f;
-      for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], Conv<T>::load(kr + d), dot);
+      for (int d = 0; d < hd; ++d) dot = fmaf(qs[d], Conv<T>::load(kr + llm_key_offset(lane, d)), dot);
       s = dot;
     }
     const float new_max = fmaxf(run_max, wave_max(s));     // finite: the page holds a valid key
@@ -54,11 +55,11 @@ __global__ __launch_bounds__(64) void attention_ref_kernel(
     for (int j = 0; j < PAGE; ++j) {
       const float pj = __shfl(p, j, 64);
       if (pj == 0.f) continue;                             // uniform across the wave
-      const T* vr = v_pages + base + j;                    // values lie [dim, position]
+      const T* vr = v_pages + vbase;
 #pragma unroll
       for (int i = 0; i < ND; ++i) {
         const int d = lane + i * 64;
-        if (d < hd) acc[i] = fmaf(pj, Conv<T>::load(vr + (size_t)d * PAGE), acc[i]);
+        if (d < hd) acc[i] = fmaf(pj, Conv<T>::load(vr + llm_value_offset(hd, d, j)), acc[i]);
       }
     }
   }

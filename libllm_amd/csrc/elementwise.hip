@@ -294,8 +294,8 @@ extern "C" int llm_add_bias(void* x, int dtype, const float* b, int M, int N, hi
 //   With `adjacent` the pairs are (2j, 2j+1) instead, still with the angle of pair j: the layout of
 //   a projection whose output rows were reordered so that the two dims of a pair lie side by side.
 //   q is rotated in place; k (rotated) and v go to the sequence's page of the cache:
-//   page = table[slot, pos / PAGE]; keys at [page, kv_head, pos % PAGE, d], values transposed at
-//   [page, kv_head, d, pos % PAGE].
+//   page = table[slot, pos / PAGE], laid out as common.h says (keys in blocks of 16 dims, values
+//   in halves of 32 positions).
 template <typename T, int PAGE>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride, const float* __restrict__ bias,
                                      int n_heads, int n_kv, int hd, const float* __restrict__ cos_t,
@@ -311,13 +311,12 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride, const 
   const int pass = hd - rot_dim;                 // dims that do not rotate
   const int per_head = half + pass;              // work items per rotating head
   const int n_rot_heads = n_heads + (write_kv ? n_kv : 0);
-  size_t page_base = 0, v_base = 0;
+  size_t page_heads = 0;                         // (page, kv head 0) counted in kv heads
   if (write_kv) {
     const int slot = seq_slot[tok_seq[m]];
-    const int page = table[(size_t)slot * table_stride + pos / PAGE];
-    page_base = ((size_t)page * n_kv) * PAGE * hd + (size_t)(pos % PAGE) * hd;
-    v_base = ((size_t)page * n_kv) * PAGE * hd + (size_t)(pos % PAGE);
+    page_heads = (size_t)table[(size_t)slot * table_stride + pos / PAGE] * n_kv;
   }
+  const int in_page = pos % PAGE;
   const float* c = cos_t + (size_t)pos * half;
   const float* s = sin_t + (size_t)pos * half;
   const int rot_items = n_rot_heads * per_head;
@@ -327,19 +326,19 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride, const 
     T* x = row + (size_t)h * hd;
     const float* b = bias ? bias + (size_t)h * hd : nullptr;
     const bool is_k = h >= n_heads;
-    T* dst = is_k ? k_pages + page_base + (size_t)(h - n_heads) * PAGE * hd : x;
+    T* kdst = k_pages + (page_heads + (size_t)(is_k ? h - n_heads : 0)) * llm_key_block(hd);
     if (j < half) {
       const int d1 = adjacent ? 2 * j : j, d2 = adjacent ? 2 * j + 1 : j + half;
       float x1 = Conv<T>::load(x + d1), x2 = Conv<T>::load(x + d2);
       if (b) { x1 += b[d1]; x2 += b[d2]; }
       const float cj = c[j], sj = s[j];
-      Conv<T>::store(dst + d1, x1 * cj - x2 * sj);
-      Conv<T>::store(dst + d2, x2 * cj + x1 * sj);
+      Conv<T>::store(is_k ? kdst + llm_key_offset(in_page, d1) : x + d1, x1 * cj - x2 * sj);
+      Conv<T>::store(is_k ? kdst + llm_key_offset(in_page, d2) : x + d2, x2 * cj + x1 * sj);
     } else {
       const int d = rot_dim + (j - half);
       float v = Conv<T>::load(x + d);
       if (b) v += b[d];
-      Conv<T>::store(dst + d, v);
+      Conv<T>::store(is_k ? kdst + llm_key_offset(in_page, d) : x + d, v);
     }
   }
   if (write_kv) {
@@ -349,7 +348,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride, const 
       const int h = it / hd, d = it % hd;
       float v = Conv<T>::load(vrow + it);
       if (b) v += b[it];
-      Conv<T>::store(v_pages + v_base + ((size_t)h * hd + d) * PAGE, v);
+      Conv<T>::store(v_pages + (page_heads + h) * llm_value_block(hd) + llm_value_offset(hd, d, in_page), v);
     }
   }
 }
@@ -358,7 +357,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride, const 
 // (grid: row tiles x (q heads + k heads + v heads)).  q and k move as 16-byte vectors (four pairs
 // and their four angles at a time).  v is transposed through LDS, so that consecutive lanes write
 // consecutive positions of a page: rows of a prompt lie in order, and a wave's 64 stores of two
-// bytes then fall into one line instead of 64.  Needs hd and rot_dim in multiples of 8.
+// bytes then fall into two half lines instead of 64 lines.  Needs hd and rot_dim in multiples of 8.
 template <int PAGE>
 __global__ __launch_bounds__(256) void rope_kv_write_tile_kernel(
     bf16_t* __restrict__ qkv, int row_stride, const float* __restrict__ bias, int n_heads, int n_kv, int hd,
@@ -418,7 +417,8 @@ __global__ __launch_bounds__(256) void rope_kv_write_tile_kernel(
       out.z = (uint32_t)f32_to_bf16(x[4]) | ((uint32_t)f32_to_bf16(x[5]) << 16);
       out.w = (uint32_t)f32_to_bf16(x[6]) | ((uint32_t)f32_to_bf16(x[7]) << 16);
       bf16_t* dst = is_q ? src
-                         : k_pages + (((size_t)s_page[r] * n_kv + (h - n_heads)) * PAGE + pos % PAGE) * hd + d;
+                         : k_pages + ((size_t)s_page[r] * n_kv + (h - n_heads)) * llm_key_block(hd) +
+                               llm_key_offset(pos % PAGE, d);
       *reinterpret_cast<uint4*>(dst) = out;
     }
     return;
@@ -448,10 +448,10 @@ __global__ __launch_bounds__(256) void rope_kv_write_tile_kernel(
   const int lane = tid & 63, wave = tid >> 6;
   if (m0 + lane < M) {
     const int pos = s_pos[lane];
-    bf16_t* dst = v_pages + ((size_t)s_page[lane] * n_kv + kvh) * hd * PAGE + pos % PAGE;
+    bf16_t* dst = v_pages + ((size_t)s_page[lane] * n_kv + kvh) * llm_value_block(hd);
     for (int d = wave; d < hd; d += 4) {
       const uint32_t w = tile[lane * row_w + d / 2];
-      dst[(size_t)d * PAGE] = (bf16_t)((d & 1) ? (w >> 16) : (w & 0xffffu));
+      dst[llm_value_offset(hd, d, pos % PAGE)] = (bf16_t)((d & 1) ? (w >> 16) : (w & 0xffffu));
     }
   }
 }

@@ -20,7 +20,7 @@
 // dims of a rotating pair are neighbours (pair j of a head at 2j, 2j+1): bias, rotation at the
 // token's position (src/libllm/llama.cc:151-176 pairs j with j + rot_dim/2; the reordering only
 // moves them side by side), rotated q to the output, rotated k and v to the token's place in the
-// paged cache (keys [page, kv_head, position, dim], values [page, kv_head, dim, position]).
+// paged cache (laid out as common.h says).
 //
 // An RMS norm between two such products needs no kernel of its own (up to 16 rows): y = x w s with
 // s = rsqrt(mean(x^2) + eps) a factor of the whole row, so (x w s) W^T = s ((x w) W^T).  The
@@ -364,14 +364,16 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
         const int kn = n - q_dim;
         if (kn < kv_dim) {
           const int kvh = kn / rope.hd;
-          *reinterpret_cast<uint2*>(rope.k_pages + (((size_t)page * rope.n_kv + kvh) * 64 + pos % 64) * rope.hd + d) = pk;
+          *reinterpret_cast<uint2*>(rope.k_pages + ((size_t)page * rope.n_kv + kvh) * llm_key_block(rope.hd) +
+                                    llm_key_offset(pos % 64, d)) = pk;
         } else {
           const int kvh = (kn - kv_dim) / rope.hd;
-          bf16_t* vp = rope.v_pages + (((size_t)page * rope.n_kv + kvh) * rope.hd + d) * 64 + pos % 64;
+          bf16_t* vp = rope.v_pages + ((size_t)page * rope.n_kv + kvh) * llm_value_block(rope.hd) +
+                       llm_value_offset(rope.hd, d, pos % 64);         // dims d .. d + 3 lie 32 apart
           vp[0] = (bf16_t)(pk.x & 0xffffu);
-          vp[64] = (bf16_t)(pk.x >> 16);
-          vp[128] = (bf16_t)(pk.y & 0xffffu);
-          vp[192] = (bf16_t)(pk.y >> 16);
+          vp[32] = (bf16_t)(pk.x >> 16);
+          vp[64] = (bf16_t)(pk.y & 0xffffu);
+          vp[96] = (bf16_t)(pk.y >> 16);
         }
       }
       continue;

@@ -14,6 +14,7 @@ from typing import List, Optional
 import numpy as np
 import torch
 
+from ..cache.layout import key_pages_shape, value_pages_shape
 from ..errors import KernelError
 from . import build
 
@@ -639,10 +640,10 @@ class HipOps:
             raise KernelError("this layer has no cache entry")
         shape = tuple(kv.k_pages.shape)
         vshape = tuple(kv.v_pages.shape)
-        if (len(shape) != 4 or shape[1:] != (n_kv, 64, hd) or len(vshape) != 4
-                or vshape != (shape[0], n_kv, hd, 64)):
-            raise KernelError("cache pages have shapes %s / %s, expected [pages, %d, 64, %d] and "
-                              "[pages, %d, %d, 64]" % (shape, vshape, n_kv, hd, n_kv, hd))
+        want = key_pages_shape(shape[0] if shape else 0, n_kv, hd)
+        vwant = value_pages_shape(shape[0] if shape else 0, n_kv, hd)
+        if shape != want or vshape != vwant:
+            raise KernelError("cache pages have shapes %s / %s, expected %s and %s" % (shape, vshape, want, vwant))
         if kv.k_pages.dtype != dtype or kv.v_pages.dtype != dtype:
             raise KernelError("cache dtype %s differs from the activations' %s" % (kv.k_pages.dtype, dtype))
         self._dev(kv.k_pages, "key pages")

@@ -54,8 +54,9 @@ class StateNeed:
 
 
 class KVView:
-    """The keys and values of one cache entry: key pages ``[pages, kv_heads, page, head_dim]``,
-    value pages ``[pages, kv_heads, head_dim, page]`` (transposed), and the table that maps
+    """The keys and values of one cache entry: key pages ``[pages, kv_heads, ceil(head_dim / 16),
+    page, 16]`` (blocks of 16 dims), value pages ``[pages, kv_heads, 2, head_dim, page / 2]``
+    (halves of 32 positions; ``cache/layout.py`` says why), and the table that maps
     (slot, position // page) to a page."""
 
     def __init__(self, k_pages, v_pages, block_table, page_size, need):

@@ -2,6 +2,7 @@
 import numpy as np
 import torch
 
+from libllm_amd.cache import layout
 from libllm_amd.parts import CacheNeed, KVView, StepContext
 
 PAGE = 64
@@ -121,8 +122,8 @@ def make_kv(device, dtype, n_slots, pages_per_seq, n_kv, hd, seed=0, window=0):
     g = torch.Generator().manual_seed(seed)
     n_pages = n_slots * pages_per_seq
     perm = torch.randperm(n_pages, generator=g).reshape(n_slots, pages_per_seq).to(torch.int32)
-    k = torch.zeros((n_pages + 1, n_kv, PAGE, hd), dtype=dtype, device=device)
-    v = torch.zeros((n_pages + 1, n_kv, hd, PAGE), dtype=dtype, device=device)
+    k = torch.zeros(layout.key_pages_shape(n_pages + 1, n_kv, hd), dtype=dtype, device=device)
+    v = torch.zeros(layout.value_pages_shape(n_pages + 1, n_kv, hd), dtype=dtype, device=device)
     need = CacheNeed("window" if window else "full", n_kv, hd, window)
     return KVView(k, v, perm.to(device), PAGE, need)
 
@@ -133,15 +134,16 @@ def fill_kv(kv, slot, keys, values):
     pos = torch.arange(length)
     pages = kv.block_table[slot].cpu().long()[pos // PAGE].to(kv.k_pages.device)
     off = (pos % PAGE).to(kv.k_pages.device)
-    kv.k_pages[pages, :, off, :] = keys.to(kv.k_pages.device, kv.k_pages.dtype)
-    kv.v_pages[pages, :, :, off] = values.to(kv.v_pages.device, kv.v_pages.dtype)
+    layout.write_keys(kv.k_pages, pages, off, keys.to(kv.k_pages.device, kv.k_pages.dtype))
+    layout.write_values(kv.v_pages, pages, off, values.to(kv.v_pages.device, kv.v_pages.dtype))
 
 
 def read_kv(kv, slot, length):
     pos = torch.arange(length)
     pages = kv.block_table[slot].cpu().long()[pos // PAGE].to(kv.k_pages.device)
     off = (pos % PAGE).to(kv.k_pages.device)
-    return kv.k_pages[pages, :, off, :].float().cpu(), kv.v_pages[pages, :, :, off].float().cpu()
+    return (layout.read_keys(kv.k_pages, pages, off, kv.need.head_dim).float().cpu(),
+            layout.read_values(kv.v_pages, pages, off).float().cpu())
 
 
 def attention_oracle(q, keys, values, pos, scale, window=0):

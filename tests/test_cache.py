@@ -49,7 +49,9 @@ def test_random_traffic_keeps_the_books():
     states = [None, StateNeed((3,)), None, StateNeed((2, 2))]
     cache = SequenceCache(needs, states, max_tokens=64 * 12, max_position=640, dtype=torch.float32, device="cpu")
     assert len(cache.groups) == 2 and cache.groups[0].entries == [0, 1] and cache.groups[1].entries == [2]
-    assert cache.groups[0].k.shape == (2, 13, 2, PAGE, 16) and cache.groups[0].v.shape == (2, 13, 2, 16, PAGE)
+    # keys in blocks of 16 dims, values in halves of 32 positions (cache/layout.py)
+    assert cache.groups[0].k.shape == (2, 13, 2, 1, PAGE, 16) and cache.groups[0].v.shape == (2, 13, 2, 2, 16, 32)
+    assert cache.groups[1].k.shape == (1, 13, 1, 2, PAGE, 16) and cache.groups[1].v.shape == (1, 13, 1, 2, 32, 32)
     assert cache.state[1].shape == (13, 3) and cache.state[3].shape == (13, 2, 2) and 0 not in cache.state
     live = {}
     for step in range(400):
@@ -114,3 +116,29 @@ def test_reused_slot_starts_clean_and_tables_follow():
         cache.reserve(s2, 65)                               # 4 pages exist, 4 held after this would be 6
     cache.check()
     assert cache.tokens_held() == 256
+
+
+def test_page_layout_round_trip():
+    """Keys and values written through the layout's helpers come back; a head size that is no
+    multiple of 16 pads its last block of dims; the flat offsets are the kernels' formulas."""
+    from libllm_amd.cache import layout
+    for hd in (16, 24, 64, 80):
+        k = torch.zeros(layout.key_pages_shape(3, 2, hd))
+        v = torch.zeros(layout.value_pages_shape(3, 2, hd))
+        assert k.shape == (3, 2, (hd + 15) // 16, 64, 16) and v.shape == (3, 2, 2, hd, 32)
+        g = torch.Generator().manual_seed(hd)
+        keys, vals = torch.randn((5, 2, hd), generator=g), torch.randn((5, 2, hd), generator=g)
+        pages, offs = torch.tensor([0, 2, 2, 1, 0]), torch.tensor([0, 63, 31, 32, 17])
+        layout.write_keys(k, pages, offs, keys)
+        layout.write_values(v, pages, offs, vals)
+        assert torch.equal(layout.read_keys(k, pages, offs, hd), keys)
+        assert torch.equal(layout.read_values(v, pages, offs), vals)
+        kb, vb = k.shape[2] * 16 * 64, hd * 64                 # elements per (page, kv head)
+        for i in range(5):
+            for head in range(2):
+                for d in (0, 7, hd - 1):
+                    page, pos = int(pages[i]), int(offs[i])
+                    at = (page * 2 + head) * kb + (d // 16) * 1024 + pos * 16 + d % 16
+                    assert k.reshape(-1)[at] == keys[i, head, d]
+                    at = (page * 2 + head) * vb + (pos // 32) * hd * 32 + d * 32 + pos % 32
+                    assert v.reshape(-1)[at] == vals[i, head, d]
