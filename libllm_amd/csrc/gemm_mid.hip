@@ -1,4 +1,4 @@
-// C[M,N] = X[M,K] * W[N,K]^T for 65 to 128 rows: still bound by the one pass over W, but with too
+// C[M,N] = X[M,K] * W[N,K]^T for 33 to 128 rows: still bound by the one pass over W, but with too
 // many rows for a block to stage all of them per 16 rows of W, as the product for few rows does.
 // bfloat16 inputs, float32 accumulation on the matrix cores.
 //
@@ -275,6 +275,8 @@ static int launch_mid(const bf16_t* X, const bf16_t* W, void* C, int M, int N, i
                                                             w_steps, n_out);                         \
     break;
   switch ((M + 15) / 16) {
+    MID_CASE(3)
+    MID_CASE(4)
     MID_CASE(5)
     MID_CASE(6)
     MID_CASE(7)
@@ -285,13 +287,13 @@ static int launch_mid(const bf16_t* X, const bf16_t* W, void* C, int M, int N, i
   return llm_launch_status();
 }
 
-// X [M, K] bfloat16 with rows ldx apart, 65 <= M <= 128; W the tiled copy of a [N, K] matrix.
+// X [M, K] bfloat16 with rows ldx apart, 33 <= M <= 128; W the tiled copy of a [N, K] matrix.
 // epilogue 0: C [M, N] bfloat16, or with k_split > 1 float32 [k_split, M, N], the products over
 // the slices of K; K is a multiple of 128 * k_split; epilogue 1: C [M, N/2] bfloat16, SwiGLU over
 // W = [Wg; Wu], N/2 a multiple of 16.
 extern "C" int llm_gemm_mid_bf16(const void* X, int ldx, const void* W_tiled, void* C, int epilogue,
                                  int out_dtype, int M, int N, int K, int k_split, hipStream_t stream) {
-  if (M < 65 || M > 128 || N <= 0 || K <= 0 || (K & 7) || ldx < K || (ldx & 7) || k_split < 1)
+  if (M < 33 || M > 128 || N <= 0 || K <= 0 || (K & 7) || ldx < K || (ldx & 7) || k_split < 1)
     return LLM_ERR_ARG;
   if (X == nullptr || W_tiled == nullptr || C == nullptr) return LLM_ERR_ARG;
   if ((((uintptr_t)X) | ((uintptr_t)W_tiled) | ((uintptr_t)C)) & 15) return LLM_ERR_ARG;

@@ -34,8 +34,11 @@ __device__ __forceinline__ Frag frag_load(const bf16_t* p) {
 // product): the load carries the non-temporal hint, so the lines do not push what the other waves
 // read again and again (the rows of X, tables) out of the chiplet's cache.  Whole engines compared
 // in one process, the weights of the skinny product so: 0.856 against 0.900 ms a decode step at
-// batch 1, 1.010 against 1.037 at batch 8, 2.65 against 2.67 at batch 64 (1B shape); the pages of
-// keys and values read so in decode attention are 1 to 3 % slower and stay ordinary loads.
+// batch 1, 1.010 against 1.037 at batch 8, 2.65 against 2.67 at batch 64 (1B shape).  The hint
+// pays only where every load instruction of a wave takes whole 128-byte lines: a wave that takes
+// half a line now and the other half a few instructions later needs the near cache for the second
+// half, and the hint gives that up (pages of keys and values read so were 1 to 3 % slower until
+// the pages were laid out for whole-line loads; since then decode attention streams them too).
 typedef uint32_t u32x4_raw __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ Frag frag_load_stream(const bf16_t* p) {
   Frag f;

@@ -107,15 +107,20 @@ class HipOps:
     SKINNY_ROWS = 64        # most rows the streaming matrix product takes at once; beyond, the library's
     ACCUM_ROWS = 16         # most rows for which a product adds into the stream itself
     SPLIT_ROWS = 64         # beyond those and up to here it goes in slices of K that the next norm adds; then the library's
-    # 65 to MID_ROWS rows: a streaming product of their own for weights with a tiled copy; beyond,
+    # MID_FROM to MID_ROWS rows: a streaming product of their own for weights with a tiled copy; beyond,
     # the library's.  Whole engines compared in one process, prompt steps of 128 tokens: 3.27
     # against 4.18 ms at the 3B shape, 5.57 against 7.07 at 8B, 1.62 against 1.66 at 1B; decode
     # batches of 96: 3.56 against 4.34, 5.84 against 7.10, 1.72 against 1.82.  For the small o
     # weight of the 1B shape the library's product is as fast (10.2 against 10.4 us): hence the limit.
     MID_ROWS = 128
+    # From 33 rows on it also beats the product for few rows, which stages the rows of X anew for
+    # every 16 to 64 rows of the weight (decode steps of whole engines in one process, batches of
+    # 48 and 64: 2.04 against 2.09 and 2.38 against 2.46 ms at the 1B shape, 4.02 against 4.11 and
+    # 4.69 against 4.83 at 3B, 5.58 against 5.74 and 6.17 against 6.45 at 8B).
+    MID_FROM = 33
     # Launch sizes below are in blocks per compute unit; ``__init__`` multiplies them by the
     # device's number of units (the figures in the comments were measured on 256 units).
-    MID_BLOCKS_PER_UNIT = 1.0       # blocks that the slices of K of the product for 65 to 128 rows aim at (half and twice as many lose 8 to 10 % of a prompt step of 128 tokens at the 3B and 8B shapes: fewer blocks, or more matrices for the norm to add)
+    MID_BLOCKS_PER_UNIT = 1.0       # blocks that the slices of K of the product for 33 to 128 rows aim at (half and twice as many lose 8 to 10 % of a prompt step of 128 tokens at the 3B and 8B shapes: fewer blocks, or more matrices for the norm to add)
     MID_FILL = 0.75                 # it takes a product that adds into the stream only if slices of at least MID_MIN_SLICE elements of K give it blocks for this share of the units (a 2,048 x 2,048 weight gets 128 blocks: the library's product is as fast, 10.2 against 10.4 us; 3,072 x 3,072 gets 192 and gains)
     MID_MIN_SLICE = 512
     DECODE_BLOCKS_PER_UNIT = 3      # blocks of the decode attention grid beyond which sequences are not split further
@@ -154,11 +159,11 @@ class HipOps:
         self.fast_attention = True      # bfloat16 attention on the matrix cores (else the plain kernel, as for float32)
         self.pack_weights = True        # keep a tiled copy of every weight for the skinny product
         self.fast_gemm = True           # the skinny product for few rows (else the library's for every product)
-        self.mid_gemm = True            # the product for 65 to 128 rows (else the library's)
+        self.mid_gemm = True            # the product for 33 to 128 rows (else the one for few rows and the library's)
         if not build.trusted("gemm_mid.hip"):
             # its loads are invisible to the compiler: with a spilled register it would be wrong
             self.mid_gemm = False
-            build._say("the product for 65 to 128 rows spills registers in this build: the library's runs instead")
+            build._say("the product for 33 to 128 rows spills registers in this build: the one for few rows and the library's run instead")
         self.fold_norms = True          # up to ACCUM_ROWS rows, a norm between two products gets no kernel of its own
         self.prompt_tiles = 0           # tiles of rows a wave of prompt attention takes (1 or 2; 0: by the number of blocks)
         self.timing = False
@@ -389,12 +394,12 @@ class HipOps:
 
     def _mid_ok(self, x, w, m, k):
         return (self.fast_gemm and self.mid_gemm and isinstance(w, PreparedWeight)
-                and self.SKINNY_ROWS < m <= self.MID_ROWS and not isinstance(x, NormedRows)
+                and self.MID_FROM <= m <= self.MID_ROWS and not isinstance(x, NormedRows)
                 and x.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1 and x.stride(0) >= k
                 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and k % 128 == 0)
 
     def _k_split_mid(self, n, k):
-        """Slices of K for a product of 65 to 128 rows whose result the next norm adds: enough for
+        """Slices of K for a product of 33 to 128 rows whose result the next norm adds: enough for
         about MID_BLOCKS blocks at 64 weight rows a block, each at least MID_MIN_SLICE long and a
         multiple of 128."""
         ks = max(1, min(16, self.MID_BLOCKS // max(1, -(-n // 64))))
@@ -445,6 +450,10 @@ class HipOps:
             self._dev(x.weight, "norm weight", torch.float32, (k,))
         else:
             self._dev(x, "linear input")
+        if (m <= self.SKINNY_ROWS and residual is not None and bias is None and self._mid_ok(x, w, m, k)
+                and (ks := self._k_split_mid(n, k)) * -(-n // 64) >= self.MID_FILL * self.units):
+            return self._mid(x, w, torch.empty((ks, m, n), dtype=torch.float32, device=self.device),
+                             self._EPI_NONE, ks)
         if (self._skinny_ok(x, w, m, k) and bias is None and residual is not None
                 and self.ACCUM_ROWS < m <= self.SPLIT_ROWS and (ks := self._k_split(n, k)) > 1):
             # K in slices, one block for 64 rows of the weight and a slice: each slice of X is staged
@@ -519,7 +528,7 @@ class HipOps:
         if k != w.shape[1]:
             raise KernelError("linear_swiglu: x is [%d, %d] but the weight is %s" % (m, k, tuple(w.shape)))
         if (self._skinny_ok(x, w, m, k) and m <= self.SKINNY_ROWS and inter % 16 == 0
-                and dtype == torch.bfloat16):
+                and dtype == torch.bfloat16 and not self._mid_ok(x, w, m, k)):
             self._weight(self._plain(w), "linear weight")
             out = torch.empty((m, inter), dtype=torch.bfloat16, device=self.device)
             self._skinny(x, w, out, self._EPI_SWIGLU, 0, m)

@@ -372,12 +372,14 @@ def test_products_over_a_prepared_norm(ops, m, width, n):
 @pytest.mark.parametrize("m", [17, 33, 40, 64])
 @pytest.mark.parametrize("nk", [(128, 2048), (2048, 2048), (2048, 8192), (3072, 3072), (200, 1536)])
 def test_products_in_slices_of_k(ops, monkeypatch, m, nk):
-    """From 33 to 64 rows a product that adds into the stream is computed over slices of K, each
+    """From 17 to 64 rows a product that adds into the stream is computed over slices of K, each
     slice to a float32 matrix of its own, and the norm kernel that follows adds them in order:
     against the plain formulas, from the weight as it lies and from its tiled copy (the same
-    bits), and the same bits when other rows share the step."""
+    bits), and the same bits when other rows share the step.  (From 33 rows on the product for 33
+    to 128 rows takes the weights it can, see below; here it is switched off.)"""
     n, k = nk
     monkeypatch.setattr(ops, "ACCUM_ROWS", 16)               # so that 17 rows take this path too
+    monkeypatch.setattr(ops, "MID_FROM", 65)
     ks = ops._k_split(n, k)
     assert ks > 1 and k % (ks * 32) == 0
     x = rnd((m, k), torch.bfloat16, 80).cuda()
@@ -412,8 +414,8 @@ def test_products_in_slices_of_k(ops, monkeypatch, m, nk):
         ops._skinny(x, w, plain, ops._EPI_NONE, 0, m, k_split=7)
 
 
-# ---------------------------------------------------------------- the product for 65 to 128 rows
-@pytest.mark.parametrize("m", [65, 80, 97, 128])
+# ---------------------------------------------------------------- the product for 33 to 128 rows
+@pytest.mark.parametrize("m", [33, 48, 50, 64, 65, 80, 97, 128])
 @pytest.mark.parametrize("nk", [(64, 128), (48, 256), (1000, 640), (3072, 3072), (2048, 8192)])
 def test_gemm_mid(ops, m, nk):
     """Plain as bfloat16, and in slices of K as float32 matrices, against float64; weights whose
@@ -432,7 +434,7 @@ def test_gemm_mid(ops, m, nk):
         assert close(total, ref, torch.float32)
 
 
-@pytest.mark.parametrize("m", [66, 128])
+@pytest.mark.parametrize("m", [34, 64, 66, 128])
 @pytest.mark.parametrize("ik", [(32, 128), (208, 384), (8192, 2048)])
 def test_gemm_mid_swiglu(ops, m, ik):
     """silu(gate) * up over a stacked weight, gate and up rounded to bfloat16 first as the
@@ -451,12 +453,12 @@ def test_gemm_mid_swiglu(ops, m, ik):
 
 def test_gemm_mid_rows_do_not_depend_on_the_batch(ops):
     """A row's sums are added along K by the same two waves in the same order whatever the other
-    rows are: the same bits at 65, 100 and 128 rows, and with the row at another place."""
+    rows are: the same bits at 33, 48, 65, 100 and 128 rows, and with the row at another place."""
     n, k = 1024, 1024
     x = rnd((128, k), torch.bfloat16, 7).cuda()
     w = ops.prepare_weight(rnd((n, k), torch.bfloat16, 8, scale=0.05).cuda())
     full = ops._mid(x, w, torch.empty((128, n), dtype=torch.bfloat16, device="cuda"), ops._EPI_NONE)
-    for m in (65, 100):
+    for m in (33, 48, 64, 65, 100):
         part = ops._mid(x[:m].contiguous(), w, torch.empty((m, n), dtype=torch.bfloat16, device="cuda"), ops._EPI_NONE)
         assert torch.equal(part, full[:m])
     moved = torch.cat([x[64:], x[:64]]).contiguous()
@@ -464,11 +466,41 @@ def test_gemm_mid_rows_do_not_depend_on_the_batch(ops):
     assert torch.equal(out[:64], full[64:]) and torch.equal(out[64:], full[:64])
 
 
+def test_steps_of_33_to_64_rows_use_it_where_it_fills_the_device(ops):
+    """A product that adds into the stream goes to it if its slices of K give blocks enough, else to
+    the product for few rows; the gate and up product always; a row's bits are the same at 33, 48 and
+    64 rows."""
+    x = rnd((64, 8192), torch.bfloat16, 11).cuda()
+    down = ops.prepare_weight(rnd((2048, 8192), torch.bfloat16, 12, scale=0.05).cuda())
+    small = ops.prepare_weight(rnd((2048, 2048), torch.bfloat16, 13, scale=0.05).cuda())
+    gate_up = ops.prepare_weight(rnd((2 * 4096, 2048), torch.bfloat16, 14, scale=0.05).cuda())
+    res = torch.zeros((64, 2048), dtype=torch.float32, device="cuda")
+    ks = ops._k_split_mid(2048, 8192)
+    assert ks * 32 >= ops.MID_FILL * ops.units
+    whole = None
+    for m in (64, 48, 33):
+        parts = ops.linear(x[:m].contiguous(), down, None, torch.bfloat16, residual=res[:m].contiguous())
+        assert tuple(parts.shape) == (ks, m, 2048)
+        assert torch.equal(parts, ops._mid(x[:m].contiguous(), down, torch.empty_like(parts), ops._EPI_NONE, ks))
+        whole = parts if whole is None else whole
+        assert torch.equal(parts, whole[:, :m])
+    xs = x[:, :2048].contiguous()
+    few = ops.linear(xs, small, None, torch.bfloat16, residual=res)
+    ks_few = ops._k_split(2048, 2048)
+    assert ops._k_split_mid(2048, 2048) * 32 < ops.MID_FILL * ops.units and tuple(few.shape) == (ks_few, 64, 2048)
+    plain = torch.empty_like(few)
+    ops._skinny(xs, small, plain, ops._EPI_NONE, 0, 64, k_split=ks_few)
+    assert torch.equal(few, plain)
+    act = ops.linear_swiglu(xs, gate_up)
+    assert torch.equal(act, ops._mid(xs, gate_up, torch.empty_like(act), ops._EPI_SWIGLU))
+    assert torch.equal(ops.linear_swiglu(xs[:40].contiguous(), gate_up), act[:40])
+
+
 def test_gemm_mid_refuses(ops):
     from libllm_amd.errors import KernelError
     w = ops.prepare_weight(rnd((64, 256), torch.bfloat16, 1).cuda())
     x = rnd((128, 256), torch.bfloat16, 2).cuda()
-    for rows, ks in ((64, 1), (129, 1), (100, 3)):                     # too few rows, too many, slices that do not divide K
+    for rows, ks in ((32, 1), (129, 1), (100, 3)):                     # too few rows, too many, slices that do not divide K
         with pytest.raises(KernelError):
             xs = torch.cat([x, x])[:rows].contiguous()
             ops._mid(xs, w, torch.empty((ks, rows, 64), dtype=torch.float32, device="cuda"), ops._EPI_NONE, ks)
