@@ -47,6 +47,7 @@ _SIGNATURES = {
                           _f, _i, _vp],
     "llm_gemm_skinny_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "llm_gemm_mid_bf16": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
+    "llm_gemm_wide_bf16": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp],
     "llm_gemm_skinny_norm_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _f, _vp],
     "llm_attention_mfma_supported": [_i],
     "llm_attention_prefill_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i,
@@ -118,6 +119,16 @@ class HipOps:
     # 48 and 64: 2.04 against 2.09 and 2.38 against 2.46 ms at the 1B shape, 4.02 against 4.11 and
     # 4.69 against 4.83 at 3B, 5.58 against 5.74 and 6.17 against 6.45 at 8B).
     MID_FROM = 33
+    # Beyond MID_ROWS rows the gate/up product with its SwiGLU is a kernel of ours where its tiles
+    # (256 rows by 128 outputs) fill whole rounds of the compute units to at least WIDE_FILL, and K
+    # is at most WIDE_MAX_K: there it beats the library's product followed by the SiLU-mul kernel
+    # (the two timed in turns, 1B shape: 111 against 136 us at 2,048 rows, 58 against 74 at 1,024,
+    # 210 against 234 at 4,096, 870 against 931 at 16,384; 3B: 155 against 167, 81 against 89, 313
+    # against 328, 1,260 against 1,284).  With half-empty rounds (512 rows: 47 against 44) and at
+    # K = 4,096, where the library's product is at its best (8B: 413 against 392 at 2,048 rows, 773
+    # against 718 at 4,096), the library's stays.
+    WIDE_FILL = 0.8
+    WIDE_MAX_K = 3072
     # Launch sizes below are in blocks per compute unit; ``__init__`` multiplies them by the
     # device's number of units (the figures in the comments were measured on 256 units).
     MID_BLOCKS_PER_UNIT = 1.0       # blocks that the slices of K of the product for 33 to 128 rows aim at (half and twice as many lose 8 to 10 % of a prompt step of 128 tokens at the 3B and 8B shapes: fewer blocks, or more matrices for the norm to add)
@@ -159,6 +170,7 @@ class HipOps:
         self.fast_attention = True      # bfloat16 attention on the matrix cores (else the plain kernel, as for float32)
         self.pack_weights = True        # keep a tiled copy of every weight for the skinny product
         self.fast_gemm = True           # the skinny product for few rows (else the library's for every product)
+        self.wide_gemm = True           # the gate/up product with SwiGLU for many rows (else the library's and the SiLU-mul kernel)
         self.mid_gemm = True            # the product for 33 to 128 rows (else the one for few rows and the library's)
         if not build.trusted("gemm_mid.hip"):
             # its loads are invisible to the compiler: with a spilled register it would be wrong
@@ -398,6 +410,28 @@ class HipOps:
                 and x.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1 and x.stride(0) >= k
                 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and k % 128 == 0)
 
+    def _wide_ok(self, x, w, m, k, inter):
+        """Whether the gate/up product of ``m`` rows goes to the kernel for many rows."""
+        if not (self.fast_gemm and self.wide_gemm and m > self.MID_ROWS and not isinstance(x, NormedRows)):
+            return False
+        wp = self._plain(w)
+        if not (x.dtype == torch.bfloat16 and wp.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1
+                and x.stride(0) >= k and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
+                and wp.stride(1) == 1 and wp.stride(0) >= k and wp.stride(0) % 8 == 0 and wp.data_ptr() % 16 == 0
+                and k % 64 == 0 and k <= self.WIDE_MAX_K and inter % 16 == 0):
+            return False
+        tiles = -(-m // 256) * -(-inter // 128)
+        rounds = -(-tiles // self.units)
+        return tiles >= self.WIDE_FILL * rounds * self.units
+
+    def _wide(self, x, w, out, epilogue):
+        wp = self._plain(w)
+        n, k = wp.shape
+        self._check(self.lib.llm_gemm_wide_bf16(
+            x.data_ptr(), x.stride(0), wp.data_ptr(), wp.stride(0), out.data_ptr(), epilogue,
+            x.shape[0], n, k, self._stream()), "gemm_wide_bf16")
+        return out
+
     def _k_split_mid(self, n, k):
         """Slices of K for a product of 33 to 128 rows whose result the next norm adds: enough for
         about MID_BLOCKS blocks at 64 weight rows a block, each at least MID_MIN_SLICE long and a
@@ -542,6 +576,11 @@ class HipOps:
             self._weight(self._plain(w), "linear weight")
             return self._mid(x, w, torch.empty((m, inter), dtype=torch.bfloat16, device=self.device),
                              self._EPI_SWIGLU)
+        if dtype == torch.bfloat16 and self._wide_ok(x, w, m, k, inter):
+            self._weight(self._plain(w), "linear weight")
+            self._dev(x, "linear input")
+            return self._wide(x, w, torch.empty((m, inter), dtype=torch.bfloat16, device=self.device),
+                              self._EPI_SWIGLU)
         return self.silu_mul(self.linear(x, w, None, x.dtype))
 
     def silu_mul(self, gu):
