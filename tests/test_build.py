@@ -35,7 +35,7 @@ def test_the_report_of_spills_is_read():
     assert build.spills_in_report("", "gemm_mid_kernel") == (0, [])
 
 
-def test_the_build_records_that_the_product_for_65_to_128_rows_spills_no_register(tmp_path):
+def test_the_build_records_that_the_product_for_33_to_128_rows_spills_no_register(tmp_path):
     """gemm_mid.hip fills registers by load instructions that the compiler does not see, and waits
     for them by count.  A register that the compiler spilled to memory before its load arrived
     would be saved with its old contents.  The build itself reads the compiler's report, with the

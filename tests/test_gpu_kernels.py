@@ -928,9 +928,9 @@ def test_attention_decode_over_many_pages(ops, ctx_len, far):
     assert max_err(out, ref) < BF16_2ULP
 
 
-def test_a_build_whose_product_for_65_to_128_rows_spills_does_not_use_it(monkeypatch):
+def test_a_build_whose_product_for_33_to_128_rows_spills_does_not_use_it(monkeypatch):
     """The build's record decides (see test_build.py): with a spill on record the host sends
-    steps of 65 to 128 rows to the library's product."""
+    steps of 33 to 128 rows to the product for few rows and to the library's."""
     from libllm_amd.hip import HipOps, build
     assert HipOps().mid_gemm
     monkeypatch.setattr(build, "trusted", lambda source, path=None: False)

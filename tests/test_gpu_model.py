@@ -291,9 +291,9 @@ def test_layers_of_the_measured_shapes(tmp_path, shape):
     """Two layers of the sizes that the measurements run (a smaller vocabulary, no power of two)
     against the plain implementation.  The launcher picks the form of a product and of attention
     by the sizes and by the rows of a step, so the tiny configurations do not reach every form:
-    batches of 1, 8, 20, 48 and 64 decode through each form of the skinny product, batches of 96
-    and 128 and a prompt of 100 tokens through the product for 65 to 128 rows, the prompts of 700
-    tokens through the library's products."""
+    batches of 1, 8, 20, 48 and 64 decode through each form of the skinny product and, from 33
+    rows on, the product for 33 to 128 rows, as do batches of 96 and 128 and a prompt of 100
+    tokens; the prompts of 700 tokens go through the library's products."""
     sh = dict(BENCH_SHAPES[shape])
     cfg_dict = {"model_type": "llama", "num_hidden_layers": 2, "vocab_size": 8009, "rope_theta": 500000.0,
                 "rope_scaling": {"rope_type": "llama3", "factor": sh.pop("factor"), "low_freq_factor": 1.0,
@@ -690,8 +690,8 @@ def test_library_products_inside_prompt_graphs(rows):
 @pytest.mark.parametrize("widths", [(2048, 32, 64, 8192), (4096, 32, 128, 14336)])
 def test_decode_graphs_of_many_rows(widths, n_prompts):
     """From 17 rows on the products that add into the stream are computed over slices of K, which
-    the next norm kernel adds; from 65 rows on by the product for 65 to 128 rows, or the
-    library's.  Layers of real width: a graph of 48 or 96 rows replayed twelve times, an engine
+    the next norm kernel adds; from 33 rows on by the product for 33 to 128 rows where its
+    slices fill the device, beyond 128 by the library's.  Layers of real width: a graph of 48 or 96 rows replayed twelve times, an engine
     without graphs stepping beside it, other work and a synchronisation between the replays;
     every replay gives the bits of the eager step."""
     import torch
