@@ -80,15 +80,21 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
   // kernel waits for them itself, before the barrier that hands a buffer over.
   const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char*)lds;
   // wave w fills rows 8 w .. 8 w + 7 of each group of 64 rows: 1 KiB at (64 p + 8 w) * 128
+  // (the instruction takes its place in LDS from M0, which is put back afterwards: the compiler
+  // need not know)
 #define WD_LOAD1(GP, LA)                                                                          \
-  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" ::"s"(LA), "v"(GP) : "memory", "m0")
+  {                                                                                               \
+    uint32_t m0_was;                                                                              \
+    asm volatile("s_mov_b32 %0, m0\n\ts_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %2, off\n\ts_mov_b32 m0, %0" \
+                 : "=&s"(m0_was) : "s"(LA), "v"(GP) : "memory");                                  \
+  }
 #define WD_LOAD(KT, BUFI)                                                                         \
   {                                                                                               \
     const size_t ko = (size_t)(KT) * WD_BK;                                                      \
     const uint32_t base = __builtin_amdgcn_readfirstlane(lds0 + (BUFI) * BUF + wave * 1024);      \
     _Pragma("unroll") for (int p = 0; p < 4; ++p) {                                               \
-      WD_LOAD1(wp[p] + ko, base + p * 8192);                                                      \
-      WD_LOAD1(xp[p] + ko, base + OPER + p * 8192);                                               \
+      WD_LOAD1(wp[p] + ko, base + p * 8192)                                                       \
+      WD_LOAD1(xp[p] + ko, base + OPER + p * 8192)                                                \
     }                                                                                             \
   }
 
@@ -117,40 +123,57 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
     _Pragma("unroll") for (int nt = 0; nt < 8; ++nt)                                              \
       FA[nt].u = *reinterpret_cast<const uint4*>(la + a_row[nt] * 128 + ((((KS) * 4 + g) ^ (r & 7)) * 16)); \
   }
-#define WD_MMA(FA, FB)                                                                            \
-  _Pragma("unroll") for (int nt = 0; nt < 8; ++nt)                                                \
-    _Pragma("unroll") for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = mfma_bf16(FA[nt], FB[mt], acc[nt][mt]);
-
   WD_LOAD(0, 0)
   if (n_kt > 1) WD_LOAD(1, 1)
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");     // everything this wave asked for has arrived
   __syncthreads();
   WD_READ(f0a, f0b, 0, 0)
   // Round kt: the fragments of the tile's first step are in registers.  Those of the second step
-  // are asked for, then the first step's matrix instructions run; behind the barrier (every wave
-  // has read all of tile kt, tile kt + 1 lies in the other buffer) tile kt + 2 is asked for into the
-  // buffer that tile kt leaves, and the first fragments of tile kt + 1, and the second step runs.
+  // are asked for while the first step's matrix instructions run, three after every eight, so that
+  // the eight waves do not all come to LDS at once; behind the barrier (every wave has read all
+  // of tile kt, tile kt + 1 lies in the other buffer) the second step runs, and between its matrix
+  // instructions go the reads of the first fragments of tile kt + 1 and the direct loads of tile
+  // kt + 2 into the buffer that tile kt leaves (a wave that issued all of them in a row would hold
+  // its matrix instructions back for as long).
+  // fragment q of a step's twelve: 0..3 of X, 4..11 of W
+#define WD_READ1(FA, FB, BUFI, KS, Q)                                                             \
+  {                                                                                               \
+    const unsigned char* la = lds + (BUFI) * BUF;                                                 \
+    if ((Q) < 4)                                                                                  \
+      FB[(Q)].u = *reinterpret_cast<const uint4*>(la + OPER + b_row[(Q)] * 128 + ((((KS) * 4 + g) ^ (r & 7)) * 16)); \
+    else                                                                                          \
+      FA[(Q) - 4].u = *reinterpret_cast<const uint4*>(la + a_row[(Q) - 4] * 128 + ((((KS) * 4 + g) ^ (r & 7)) * 16)); \
+  }
   for (int kt = 0; kt < n_kt; ++kt) {
     const int buf = kt & 1;
-    WD_READ(f1a, f1b, buf, 1)
-    __builtin_amdgcn_sched_barrier(0);
-    WD_MMA(f0a, f0b)
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int q = 3 * p; q < 3 * p + 3; ++q) WD_READ1(f1a, f1b, buf, 1, q)
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int nt = 2 * p; nt < 2 * p + 2; ++nt)
+#pragma unroll
+        for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = mfma_bf16(f0a[nt], f0b[mt], acc[nt][mt]);
+    }
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
     __syncthreads();
-    if (kt + 1 < n_kt) WD_READ(f0a, f0b, buf ^ 1, 0)
-    // the loads of tile kt + 2 go out between the matrix instructions, two after every eight: a wave
-    // that issued all sixteen in a row would hold its matrix instructions back for as long
     {
-      const bool more = kt + 2 < n_kt;
+      const bool more = kt + 2 < n_kt, next = kt + 1 < n_kt;
       const size_t ko = (size_t)(more ? kt + 2 : kt) * WD_BK;
       const uint32_t base = __builtin_amdgcn_readfirstlane(lds0 + buf * BUF + wave * 1024);
 #pragma unroll
       for (int p = 0; p < 4; ++p) {
         __builtin_amdgcn_sched_barrier(0);
+        if (next) {
+#pragma unroll
+          for (int q = 3 * p; q < 3 * p + 3; ++q) WD_READ1(f0a, f0b, buf ^ 1, 0, q)
+        }
         if (more) {
-          WD_LOAD1(wp[p] + ko, base + p * 8192);
-          WD_LOAD1(xp[p] + ko, base + OPER + p * 8192);
+          WD_LOAD1(wp[p] + ko, base + p * 8192)
+          WD_LOAD1(xp[p] + ko, base + OPER + p * 8192)
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
