@@ -119,6 +119,7 @@ class HipOps:
     # 48 and 64: 2.04 against 2.09 and 2.38 against 2.46 ms at the 1B shape, 4.02 against 4.11 and
     # 4.69 against 4.83 at 3B, 5.58 against 5.74 and 6.17 against 6.45 at 8B).
     MID_FROM = 33
+    MID_HEAD = True         # logits of 65 to 128 rows by it too
     # Beyond MID_ROWS rows the gate/up product with its SwiGLU is a kernel of ours where its tiles
     # (256 rows by 128 outputs) fill whole rounds of the compute units to at least WIDE_FILL, and K
     # is at most WIDE_MAX_K: there it beats the library's product followed by the SiLU-mul kernel
@@ -488,6 +489,12 @@ class HipOps:
                 and (ks := self._k_split_mid(n, k)) * -(-n // 64) >= self.MID_FILL * self.units):
             return self._mid(x, w, torch.empty((ks, m, n), dtype=torch.float32, device=self.device),
                              self._EPI_NONE, ks)
+        if (self.MID_HEAD and out_dtype == torch.float32 and residual is None and bias is None
+                and self.SKINNY_ROWS < m and self._mid_ok(x, w, m, k)):
+            # float32 results (logits) for 65 to 128 rows in one pass over the weight, where the
+            # product for few rows would take two
+            return self._mid(x, w, torch.empty((1, m, n), dtype=torch.float32, device=self.device),
+                             self._EPI_NONE, 1)[0]
         if (self._skinny_ok(x, w, m, k) and bias is None and residual is not None
                 and self.ACCUM_ROWS < m <= self.SPLIT_ROWS and (ks := self._k_split(n, k)) > 1):
             # K in slices, one block for 64 rows of the weight and a slice: each slice of X is staged

@@ -496,6 +496,25 @@ def test_steps_of_33_to_64_rows_use_it_where_it_fills_the_device(ops):
     assert torch.equal(ops.linear_swiglu(xs[:40].contiguous(), gate_up), act[:40])
 
 
+def test_logits_of_65_to_128_rows_take_one_pass(ops):
+    """Float32 results without a stream to add to (the head) go through the product for 33 to 128
+    rows from 65 rows on, where the product for few rows would read the weight twice; a normed
+    record is made into rows first."""
+    x = rnd((100, 256), torch.bfloat16, 21).cuda()
+    w = ops.prepare_weight(rnd((1000, 256), torch.bfloat16, 22, scale=0.05).cuda())
+    out = ops.linear(x, w, None, torch.float32)
+    assert out.dtype == torch.float32 and tuple(out.shape) == (100, 1000)
+    assert torch.equal(out, ops._mid(x, w, torch.empty((1, 100, 1000), dtype=torch.float32, device="cuda"), ops._EPI_NONE, 1)[0])
+    assert close(out, x.double() @ w.w.double().t(), torch.float32)
+    few = ops.linear(x[:64].contiguous(), w, None, torch.float32)            # up to 64 rows: the product for few rows
+    assert max_err(few, out[:64]) < 2e-6
+    res = rnd((100, 256), torch.float32, 23, 2.0).cuda()
+    wn = (1.0 + 0.1 * rnd((256,), torch.float32, 24)).cuda()
+    lazy = ops.normed(res, wn, 1e-5)
+    rows = ops.add_rmsnorm(res, None, wn, 1e-5, torch.bfloat16)
+    assert torch.equal(ops.linear(lazy, w, None, torch.float32), ops.linear(rows, w, None, torch.float32))
+
+
 def test_gemm_mid_refuses(ops):
     from libllm_amd.errors import KernelError
     w = ops.prepare_weight(rnd((64, 256), torch.bfloat16, 1).cuda())
