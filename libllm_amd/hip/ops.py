@@ -125,9 +125,12 @@ class HipOps:
     # is at most WIDE_MAX_K: there it beats the library's product followed by the SiLU-mul kernel
     # (the two timed in turns, 1B shape: 111 against 136 us at 2,048 rows, 58 against 74 at 1,024,
     # 210 against 234 at 4,096, 870 against 931 at 16,384; 3B: 155 against 167, 81 against 89, 313
-    # against 328, 1,260 against 1,284).  With half-empty rounds (512 rows: 47 against 44) and at
-    # K = 4,096, where the library's product is at its best (8B: 413 against 392 at 2,048 rows, 773
-    # against 718 at 4,096), the library's stays.
+    # against 328, 1,260 against 1,284).  With half-empty rounds (512 rows: 47 against 44) the
+    # library's stays.  What the kernel saves is the SiLU-mul pass, 6 bytes an output against the
+    # product's 4 K flops: a fifth of the product's time at K = 2,048, an eighth at 3,072, a tenth
+    # at 4,096, while its plain product is 7 to 10 % behind the library's at large sizes; so beyond
+    # K of about 3,500 it loses (8B, K = 4,096: 413 against 392 at 2,048 rows, 773 against 718 at
+    # 4,096).
     WIDE_FILL = 0.8
     WIDE_MAX_K = 3072
     # Launch sizes below are in blocks per compute unit; ``__init__`` multiplies them by the
