@@ -293,7 +293,9 @@ def test_layers_of_the_measured_shapes(tmp_path, shape):
     by the sizes and by the rows of a step, so the tiny configurations do not reach every form:
     batches of 1, 8, 20, 48 and 64 decode through each form of the skinny product and, from 33
     rows on, the product for 33 to 128 rows, as do batches of 96 and 128 and a prompt of 100
-    tokens; the prompts of 700 tokens go through the library's products."""
+    tokens; the three prompts of 670 tokens (a step of some 2,030 rows) go through the library's
+    products and, for the gate and up weights of the 1B and 3B shapes, the product for many rows
+    (test_the_gate_and_up_product_of_a_long_prompt_is_ours sees that it runs)."""
     sh = dict(BENCH_SHAPES[shape])
     cfg_dict = {"model_type": "llama", "num_hidden_layers": 2, "vocab_size": 8009, "rope_theta": 500000.0,
                 "rope_scaling": {"rope_type": "llama3", "factor": sh.pop("factor"), "low_freq_factor": 1.0,
@@ -305,7 +307,7 @@ def test_layers_of_the_measured_shapes(tmp_path, shape):
     cfg = llama.PlainConfig(cfg_json)
     rng = np.random.default_rng(1)
     for batch, prompt, decode, dtypes in ((1, 40, 5, DTYPES), (8, 30, 5, DTYPES), (20, 20, 3, DTYPES),
-                                          (48, 10, 3, ["bfloat16"]), (64, 8, 3, DTYPES), (3, 700, 2, ["bfloat16"]),
+                                          (48, 10, 3, ["bfloat16"]), (64, 8, 3, DTYPES), (3, 670, 2, ["bfloat16"]),
                                           (96, 6, 3, ["bfloat16"]), (1, 100, 2, ["bfloat16"]), (128, 1, 2, ["bfloat16"])):
         group = {"s%d_%d" % (batch, i): rng.integers(0, cfg.vocab, size=prompt + int(rng.integers(0, 9)) + decode).tolist()
                  for i in range(batch)}
@@ -315,6 +317,37 @@ def test_layers_of_the_measured_shapes(tmp_path, shape):
             out_dir = tmp_path / ("%s_%d_%s" % (shape, batch, dtype))
             run_replay(path, dtype, steps, out_dir, max_tokens=traces.max_tokens_needed(steps) + 64)
             check(shape, cfg, weights, checked, traces.collect(steps, str(out_dir), cfg.vocab), dtype)
+
+
+def test_the_gate_and_up_product_of_a_long_prompt_is_ours():
+    """A step of 2,030 rows at the 1B shape's widths: every layer's gate and up product with its
+    SwiGLU is the kernel for many rows, also in the captured prompt graph that the second such step
+    makes; a step of 600 rows, whose tiles would fill half a round of the device, is the library's."""
+    from libllm_amd.config import config_from_dict
+    from libllm_amd.engine import StepEntry
+    from libllm_amd.runtime import random_engine
+    sh = dict(BENCH_SHAPES["1b"])
+    cfg_dict = {"model_type": "llama", "num_hidden_layers": 2, "vocab_size": 8009, "rope_theta": 500000.0,
+                "rope_scaling": {"rope_type": "llama3", "factor": sh.pop("factor"), "low_freq_factor": 1.0,
+                                 "high_freq_factor": 4.0, "original_max_position_embeddings": 8192},
+                "rms_norm_eps": 1e-5, "max_position_embeddings": 4096, "hidden_act": "silu",
+                "eos_token_id": 2, **sh}
+    engine = random_engine(config_from_dict(cfg_dict), seed=5, dtype="bfloat16", max_tokens=8192)
+    calls = []
+    real = engine.ops._wide
+    engine.ops._wide = lambda *a: (calls.append(a[0].shape[0]), real(*a))[1]
+    rng = np.random.default_rng(9)
+    outs = []
+    toks = rng.integers(0, 8009, size=2030).tolist()
+    for rep in range(3):                                   # the second coming of the shape captures a graph
+        outs.append(engine.step([StepEntry(("long", rep), toks, [2029])]).clone())
+        engine.end([("long", rep)])
+    assert calls and all(m >= 2030 for m in calls) and len(calls) >= 2 * 2, calls
+    assert torch.equal(outs[1], outs[2])                   # the same prompt from the graph, twice
+    assert (outs[0] - outs[1]).abs().max().item() < 0.05 * outs[0].abs().max().item()
+    calls.clear()
+    engine.step([StepEntry("short", rng.integers(0, 8009, size=600).tolist(), [599])])
+    assert not calls
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
