@@ -199,6 +199,8 @@ def main() -> int:
     ap.add_argument("--prefill", type=int, default=2048)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
     ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64")
+    ap.add_argument("--sampling", default="greedy", choices=["greedy", "default"],
+                    help="greedy, or the command line's default (temperature 1, top-k 50, top-p 0.8)")
     ap.add_argument("--workload", choices=["unequal16", "batch64"],
                     help="run a generation workload through the generation loop instead")
     args = ap.parse_args()
@@ -233,7 +235,7 @@ def main() -> int:
     engine = random_engine(cfg, seed=0, dtype=args.dtype, max_tokens=max_tokens)
     gen = Generator(engine, Sampler(engine.ops, cfg.vocab_size), (), cfg.max_position_embeddings,
                     engine.cache.n_pages, PAGE, max_batch=biggest)
-    params = SamplingParams(temperature=0.0)
+    params = SamplingParams(temperature=0.0) if args.sampling == "greedy" else SamplingParams()
     vocab = cfg.vocab_size
     peaks = engine.ops.measured_peaks()
     log("measured on this GPU: read %.0f GB/s, copy %.0f GB/s, bf16 matrix cores %.0f TFLOP/s, fp32 %.1f TFLOP/s"
@@ -272,7 +274,7 @@ def main() -> int:
             "intermediate": cfg.intermediate_size, "vocab": cfg.vocab_size,
             "tied_head": cfg.tie_word_embeddings,
             "rope": "theta 5e5, llama3 factor %g" % cfg.rope_scaling["factor"], "global_batch": args.batch, "seq_len": args.context,
-            "prefill_tokens": args.prefill, "sampling": "greedy", "parallelism": "single GPU",
+            "prefill_tokens": args.prefill, "sampling": "greedy" if args.sampling == "greedy" else "temperature 1, top-k 50, top-p 0.8", "parallelism": "single GPU",
         },
         "prefill": {"value": round(args.prefill / pre_s, 1), "tokens": args.prefill,
                     "ms": round(pre_s * 1e3, 3), "frac": round(pf / pre_s / DENSE_FLOPS[short], 4),

@@ -244,7 +244,7 @@ __global__ __launch_bounds__(SP_NT) void sample_part_kernel(const float* __restr
   __shared__ float fbuf[SP_NT / 64];
   __shared__ int ibuf[SP_NT / 64];
   __shared__ unsigned int hist[256], wsum[4];
-  __shared__ unsigned int sh_prefix, sh_need, sh_count, sh_bin, sh_rest;
+  __shared__ unsigned int sh_prefix, sh_need, sh_count, sh_bin, sh_rest, sh_all;
   const int part = blockIdx.x, row = blockIdx.y, parts = gridDim.x, tid = threadIdx.x;
   const int lo = part * per;
   const int n = min(per, V - lo);                       // >= 1 by the choice of parts
@@ -283,10 +283,15 @@ __global__ __launch_bounds__(SP_NT) void sample_part_kernel(const float* __restr
     __syncthreads();
     select_bin(hist, sh_need, wsum, &sh_bin, &sh_rest);
     if (tid == 0) {
-      sh_need = sh_rest;
-      sh_prefix = (prefix << 8) | sh_bin;
+      // every key of the chosen bin is wanted: the bins below need not be told apart.  All keys
+      // from the bin's lowest on are taken then, none by its index.
+      const unsigned low = ((prefix << 8) | sh_bin) << shift;
+      sh_all = (sh_rest == hist[sh_bin] && low > 0u && pass < 3);
+      sh_need = sh_all ? 0u : sh_rest;
+      sh_prefix = sh_all ? low - 1u : ((prefix << 8) | sh_bin);
     }
     __syncthreads();
+    if (sh_all) break;
   }
   const uint32_t kth = sh_prefix;
   const int need_eq = (int)sh_need;          // how many logits equal to the k-th are taken: the lowest indices
@@ -332,7 +337,7 @@ __global__ __launch_bounds__(NT) void sample_final_kernel(const float* __restric
   __shared__ unsigned int hist[256], wsum[4];
   __shared__ unsigned long long cand[SP_KMAX];
   __shared__ unsigned long long sh_prefix;
-  __shared__ unsigned int sh_need, sh_count, sh_bin, sh_rest;
+  __shared__ unsigned int sh_need, sh_count, sh_bin, sh_rest, sh_all;
   __shared__ int sh_result, sh_part;
   __shared__ float sh_before;
   const int row = blockIdx.x, tid = threadIdx.x;
@@ -406,12 +411,15 @@ __global__ __launch_bounds__(NT) void sample_final_kernel(const float* __restric
     __syncthreads();
     select_bin(hist, sh_need, wsum, &sh_bin, &sh_rest);
     if (tid == 0) {
+      // every key of the chosen bin is wanted: the bin's lowest possible key is the bound
+      sh_all = (sh_rest == hist[sh_bin] && pass < 7);
       sh_need = sh_rest;
-      sh_prefix = (prefix << 8) | (unsigned long long)sh_bin;
+      sh_prefix = ((prefix << 8) | (unsigned long long)sh_bin) << (sh_all ? shift : 0);
     }
     __syncthreads();
+    if (sh_all) break;
   }
-  const unsigned long long kth = sh_prefix;             // the top_k-th largest key; keys are distinct
+  const unsigned long long kth = sh_prefix;             // the top_k-th largest key, or a bound just below it; keys are distinct
   if (tid == 0) sh_count = 0;
   for (int i = tid; i < SP_KMAX; i += NT) cand[i] = 0ull;
   __syncthreads();

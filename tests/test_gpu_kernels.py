@@ -1035,6 +1035,26 @@ def test_sampling_matches_plain(ops):
         assert bad <= 2
 
 
+def test_sampling_with_many_equal_logits(ops):
+    """Logits of few distinct values: the top-k cut falls inside a run of equal ones (the lowest
+    indices are kept), or takes a whole run (where the selection stops early)."""
+    from plain import sampling
+    g = torch.Generator().manual_seed(5)
+    for vocab, top_k, top_p, temp, step in [(3000, 50, 0.9, 1.0, 1.0), (128256, 50, 0.8, 1.0, 0.5),
+                                            (9000, 200, 1.0, 0.7, 2.0), (5000, 64, 0.95, 1.5, 4.0)]:
+        logits = torch.round(torch.randn((16, vocab), generator=g) * 3.0 / step) * step
+        streams, counters = list(range(16)), list(range(50, 66))
+        got = ops.sample(logits.cuda(), temp, top_k, top_p, 9, streams, counters).tolist()
+        bad = 0
+        for r in range(16):
+            u = sampling.uniform(9, streams[r], counters[r])
+            want = sampling.sample(logits[r].double().numpy(), temp, top_k, top_p, u)
+            if got[r] != want:
+                assert sampling.margin(logits[r].double().numpy(), temp, top_k, top_p, u) < 1e-5, (vocab, r)
+                bad += 1
+        assert bad <= 2, (vocab, bad)
+
+
 @pytest.mark.parametrize("vocab", [5003, 128256])
 def test_nucleus_without_a_limit_on_the_candidates(ops, vocab):
     """top_k 0 with top_p below 1 (the reference's sampler takes any top_k up to the vocabulary,
