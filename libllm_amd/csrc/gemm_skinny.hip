@@ -483,6 +483,11 @@ static int pick_shape(const SkinnyArgs& a) {
       // needs few enough registers for two of them to share a unit, and the tail of one overlaps
       // the head of the next (3 % of a decode step at the 1B and 8B shapes, whole engines compared)
       if constexpr (EPI == SK_EPI_SWIGLU) return launch_skinny<1, RT, 1, 1, EPI, OutT>(a);
+      // likewise any weight with more tiles than units whose K gives fewer than three chunks of
+      // 1,024: with the narrow chunk a block still has loads ahead of its arithmetic (the head of
+      // the 1B shape, K = 2,048: 0.829 against 0.838 ms a decode step at batch 1, 0.977 against
+      // 0.985 at batch 8; with K = 3,072 and 4,096 the two are the same)
+      if ((a.K + 1023) / 1024 < 3) return launch_skinny<1, RT, 1, 1, EPI, OutT>(a);
       return launch_skinny<1, RT, 1, 2, EPI, OutT>(a);
     // More rows of W per block where W has rows enough to fill the GPU with such blocks: the rows
     // of X are then staged once for 64 rows of W instead of 16.
