@@ -8,38 +8,43 @@
 // rows of the same columns): at that size a unit reads 64 KiB for 64 elements of K, which the
 // caches deliver in about the time the matrix cores need for them.  A wave owns 64 x 128 of the
 // tile (SwiGLU: 64 x (64 gate + 64 up)): 32 sums of 16 x 16, with W as the A operand, so that a
-// lane ends with four consecutive columns of one row of C.
+// lane ends with four consecutive columns of one row of C.  A second form takes 128 rows of X a
+// block (a wave 64 x 64): half the arithmetic for three quarters of the bytes, but twice the
+// blocks, for steps whose tiles of 256 rows would leave compute units idle.
 //
 // Tiles of 64 elements of K go from global memory straight into LDS (global_load_lds_dwordx4, no
-// registers in between), two buffers of 64 KiB.  A row of a tile is 128 bytes in 8 pieces of 16;
+// registers in between), two buffers of 64 (48) KiB.  A row of a tile is 128 bytes in 8 pieces of 16;
 // piece p of row r lies at p ^ (r & 7), so that the 16 rows a fragment read touches fall into
 // different banks; the swizzle is applied on the global side, since a direct load fills LDS in lane
 // order.  The fragments of a step of 32 are read into registers one step ahead of the matrix
-// instructions that use them (two sets of 12), and the direct loads of the tile after next go out
+// instructions that use them (two sets of 12 or 8), and the direct loads of the tile after next go out
 // between matrix instructions: one barrier per tile of K.
 //
 // Blocks are numbered so that the blocks of a chiplet (every eighth) share operands in its cache:
 // a chiplet takes every eighth tile of W rows and, at a time, a band of 8 tiles of X rows.
 #include "mfma.h"
 
-#define WD_BM 256          // rows of X a block
 #define WD_BN 256          // rows of W a block
 #define WD_BK 64           // elements of K a tile
 #define WD_NT 512          // threads of a block
 #define WD_EPI_NONE 0
 #define WD_EPI_SWIGLU 1
 
-template <int EPI>
+template <int EPI, int BM>
 __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restrict__ X, int ldx,
                                                           const bf16_t* __restrict__ W, int ldw,
                                                           bf16_t* __restrict__ C, int M, int N, int K,
                                                           int n_out, int m_tiles, int n_tiles) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
-  constexpr int OPER = 256 * 128;                 // bytes of an operand's tile
-  constexpr int BUF = 2 * OPER;
+  static_assert(BM == 256 || BM == 128, "rows of X a block");
+  constexpr int OPER = 256 * 128;                 // bytes of W's tile; X's follows it
+  constexpr int BUF = OPER + BM * 128;
+  constexpr int WM = BM / 64, WNW = 8 / WM;       // waves along the rows of X and of W
+  constexpr int NTW = 256 / WNW / 16;             // tiles of 16 rows of W a wave: 8 or 4
+  constexpr int XP = BM / 64;                     // pieces of X a thread loads per tile of K
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int r = lane & 15, g = lane >> 4;
-  const int wm = wave & 3, wn = wave >> 2;
+  const int wm = wave % WM, wn = wave / WM;
 
   // blocks i, i + 8, ... share a chiplet: a chiplet takes every eighth tile of W rows and, at a
   // time, a band of 8 tiles of X rows; its 32 units then share 8 tiles of X and 4 of W whatever
@@ -50,20 +55,23 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
   const int band_rows = (m_tiles - band * 8 < 8) ? m_tiles - band * 8 : 8;     // the last band may be short
   const int mt_blk = band * 8 + jj % band_rows, nt_blk = (jj / band_rows) * 8 + xcd;
   if (nt_blk >= n_tiles || jj >= band_rows * n_per) return;
-  const int m0 = mt_blk * WD_BM;
+  const int m0 = mt_blk * BM;
 
   // global -> LDS without registers in between: a wave's load instruction fills 1 KiB of LDS in
   // lane order, 8 rows of 8 pieces; lane l fills slot (l & 7) of row (l >> 3) and so fetches
   // piece (l & 7) ^ (row & 7) of that row.  A thread carries rows (tid >> 3) + 64 p of both operands.
   const int row0 = tid >> 3, piece = (tid & 7) ^ (row0 & 7);
-  const bf16_t* xp[4];
+  const bf16_t* xp[XP];
   const bf16_t* wp[4];
+#pragma unroll
+  for (int p = 0; p < XP; ++p) {
+    int m = m0 + row0 + 64 * p;
+    if (m > M - 1) m = M - 1;
+    xp[p] = X + (size_t)m * ldx + piece * 8;
+  }
 #pragma unroll
   for (int p = 0; p < 4; ++p) {
     const int row = row0 + 64 * p;
-    int m = m0 + row;
-    if (m > M - 1) m = M - 1;
-    xp[p] = X + (size_t)m * ldx + piece * 8;
     int n;
     if (EPI == WD_EPI_SWIGLU) {
       n = nt_blk * 128 + (row & 127);
@@ -92,35 +100,34 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
   {                                                                                               \
     const size_t ko = (size_t)(KT) * WD_BK;                                                      \
     const uint32_t base = __builtin_amdgcn_readfirstlane(lds0 + (BUFI) * BUF + wave * 1024);      \
-    _Pragma("unroll") for (int p = 0; p < 4; ++p) {                                               \
-      WD_LOAD1(wp[p] + ko, base + p * 8192)                                                       \
-      WD_LOAD1(xp[p] + ko, base + OPER + p * 8192)                                                \
-    }                                                                                             \
+    _Pragma("unroll") for (int p = 0; p < 4; ++p) WD_LOAD1(wp[p] + ko, base + p * 8192)           \
+    _Pragma("unroll") for (int p = 0; p < XP; ++p) WD_LOAD1(xp[p] + ko, base + OPER + p * 8192)   \
   }
 
-  f32x4 acc[8][4];
+  f32x4 acc[NTW][4];
 #pragma unroll
-  for (int nt = 0; nt < 8; ++nt)
+  for (int nt = 0; nt < NTW; ++nt)
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
   // rows of this wave's tiles within the block's operands
-  int a_row[8], b_row[4];
+  int a_row[NTW], b_row[4];
 #pragma unroll
-  for (int nt = 0; nt < 8; ++nt)
-    a_row[nt] = (EPI == WD_EPI_SWIGLU) ? ((nt >> 2) * 128 + wn * 64 + (nt & 3) * 16 + r) : (wn * 128 + nt * 16 + r);
+  for (int nt = 0; nt < NTW; ++nt)
+    a_row[nt] = (EPI == WD_EPI_SWIGLU) ? ((nt / (NTW / 2)) * 128 + wn * (NTW / 2) * 16 + (nt % (NTW / 2)) * 16 + r)
+                                       : (wn * NTW * 16 + nt * 16 + r);
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt) b_row[mt] = wm * 64 + mt * 16 + r;
 
   const int n_kt = K / WD_BK;
-  Frag f0a[8], f0b[4], f1a[8], f1b[4];
+  Frag f0a[NTW], f0b[4], f1a[NTW], f1b[4];
 #define WD_READ(FA, FB, BUFI, KS)                                                                 \
   {                                                                                               \
     const unsigned char* la = lds + (BUFI) * BUF;                                                 \
     const unsigned char* lb = la + OPER;                                                          \
     _Pragma("unroll") for (int mt = 0; mt < 4; ++mt)                                              \
       FB[mt].u = *reinterpret_cast<const uint4*>(lb + b_row[mt] * 128 + ((((KS) * 4 + g) ^ (r & 7)) * 16)); \
-    _Pragma("unroll") for (int nt = 0; nt < 8; ++nt)                                              \
+    _Pragma("unroll") for (int nt = 0; nt < NTW; ++nt)                                            \
       FA[nt].u = *reinterpret_cast<const uint4*>(la + a_row[nt] * 128 + ((((KS) * 4 + g) ^ (r & 7)) * 16)); \
   }
   WD_LOAD(0, 0)
@@ -135,7 +142,9 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
   // instructions go the reads of the first fragments of tile kt + 1 and the direct loads of tile
   // kt + 2 into the buffer that tile kt leaves (a wave that issued all of them in a row would hold
   // its matrix instructions back for as long).
-  // fragment q of a step's twelve: 0..3 of X, 4..11 of W
+  // fragment q of a step's: 0..3 of X, then those of W
+  constexpr int R = 4 + NTW;                      // fragments a step
+  constexpr int L = 4 + XP;                       // direct loads a thread and tile: 0..3 of W, then those of X
 #define WD_READ1(FA, FB, BUFI, KS, Q)                                                             \
   {                                                                                               \
     const unsigned char* la = lds + (BUFI) * BUF;                                                 \
@@ -144,18 +153,17 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
     else                                                                                          \
       FA[(Q) - 4].u = *reinterpret_cast<const uint4*>(la + a_row[(Q) - 4] * 128 + ((((KS) * 4 + g) ^ (r & 7)) * 16)); \
   }
+  // NTW groups of four matrix instructions a step; the reads (and loads) are dealt out over them
   for (int kt = 0; kt < n_kt; ++kt) {
     const int buf = kt & 1;
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
+    for (int nt = 0; nt < NTW; ++nt) {
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int q = 3 * p; q < 3 * p + 3; ++q) WD_READ1(f1a, f1b, buf, 1, q)
+      for (int q = (R * nt) / NTW; q < (R * (nt + 1)) / NTW; ++q) WD_READ1(f1a, f1b, buf, 1, q)
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int nt = 2 * p; nt < 2 * p + 2; ++nt)
-#pragma unroll
-        for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = mfma_bf16(f0a[nt], f0b[mt], acc[nt][mt]);
+      for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = mfma_bf16(f0a[nt], f0b[mt], acc[nt][mt]);
     }
     __builtin_amdgcn_sched_barrier(0);
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
@@ -165,32 +173,34 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
       const size_t ko = (size_t)(more ? kt + 2 : kt) * WD_BK;
       const uint32_t base = __builtin_amdgcn_readfirstlane(lds0 + buf * BUF + wave * 1024);
 #pragma unroll
-      for (int p = 0; p < 4; ++p) {
+      for (int nt = 0; nt < NTW; ++nt) {
         __builtin_amdgcn_sched_barrier(0);
         if (next) {
 #pragma unroll
-          for (int q = 3 * p; q < 3 * p + 3; ++q) WD_READ1(f0a, f0b, buf ^ 1, 0, q)
+          for (int q = (R * nt) / NTW; q < (R * (nt + 1)) / NTW; ++q) WD_READ1(f0a, f0b, buf ^ 1, 0, q)
         }
         if (more) {
-          WD_LOAD1(wp[p] + ko, base + p * 8192)
-          WD_LOAD1(xp[p] + ko, base + OPER + p * 8192)
+#pragma unroll
+          for (int j = (L * nt) / NTW; j < (L * (nt + 1)) / NTW; ++j) {
+            if (j < 4) { WD_LOAD1(wp[j] + ko, base + j * 8192) }
+            else { WD_LOAD1(xp[j - 4] + ko, base + OPER + (j - 4) * 8192) }
+          }
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-        for (int nt = 2 * p; nt < 2 * p + 2; ++nt)
-#pragma unroll
-          for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = mfma_bf16(f1a[nt], f1b[mt], acc[nt][mt]);
+        for (int mt = 0; mt < 4; ++mt) acc[nt][mt] = mfma_bf16(f1a[nt], f1b[mt], acc[nt][mt]);
       }
     }
     __builtin_amdgcn_sched_barrier(0);
   }
 
   // ---- epilogue: lane holds C[m = .. + r][n = .. + 4 g + e].  Each wave turns its tile (64 rows
-  // of 128 or, after SwiGLU, 64 outputs) round through a region of LDS of its own, rows 16
+  // of its outputs) round through a region of LDS of its own, rows 16
   // bytes longer than they are so that the 16 rows of a store fall into different banks, and then
   // stores whole rows, 16 bytes a lane.
   __syncthreads();                                   // every wave has read the last tile
-  constexpr int OUT_COLS = (EPI == WD_EPI_SWIGLU) ? 64 : 128;     // of a wave
+  constexpr int OUT_T = (EPI == WD_EPI_SWIGLU) ? NTW / 2 : NTW;   // tiles of 16 outputs of a wave
+  constexpr int OUT_COLS = OUT_T * 16;
   constexpr int ROW_B = OUT_COLS * 2 + 16;
   unsigned char* mine = lds + wave * (64 * ROW_B);
 #pragma unroll
@@ -203,7 +213,7 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
         // and the reciprocal by the hardware's instructions (their error is far below the rounding
         // of the result)
         const uint32_t g01 = pack2_bf16(acc[nt][mt][0], acc[nt][mt][1]), g23 = pack2_bf16(acc[nt][mt][2], acc[nt][mt][3]);
-        const uint32_t u01 = pack2_bf16(acc[nt + 4][mt][0], acc[nt + 4][mt][1]), u23 = pack2_bf16(acc[nt + 4][mt][2], acc[nt + 4][mt][3]);
+        const uint32_t u01 = pack2_bf16(acc[nt + NTW / 2][mt][0], acc[nt + NTW / 2][mt][1]), u23 = pack2_bf16(acc[nt + NTW / 2][mt][2], acc[nt + NTW / 2][mt][3]);
         const float gt[4] = {__uint_as_float(g01 << 16), __uint_as_float(g01 & 0xffff0000u), __uint_as_float(g23 << 16), __uint_as_float(g23 & 0xffff0000u)};
         const float up[4] = {__uint_as_float(u01 << 16), __uint_as_float(u01 & 0xffff0000u), __uint_as_float(u23 << 16), __uint_as_float(u23 & 0xffff0000u)};
         float v[4];
@@ -222,7 +232,7 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
   constexpr int LPR = OUT_COLS / 8;                  // lanes a row
   constexpr int RPP = 64 / LPR;                      // rows a pass
   const int ldc = (EPI == WD_EPI_SWIGLU) ? n_out : N;
-  const int n_wave = (EPI == WD_EPI_SWIGLU) ? nt_blk * 128 + wn * 64 : nt_blk * WD_BN + wn * 128;
+  const int n_wave = (EPI == WD_EPI_SWIGLU) ? nt_blk * 128 + wn * OUT_COLS : nt_blk * WD_BN + wn * OUT_COLS;
   const int col = (lane % LPR) * 8;
 #pragma unroll
   for (int pass = 0; pass < 64 / RPP; ++pass) {
@@ -243,38 +253,48 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
   }
 }
 
-// X [M, K] rows ldx apart, W [N, K] rows ldw apart (both bfloat16, K a multiple of 64, 16-byte aligned rows);
-// epilogue 0: C [M, N]; 1: C [M, N/2], SwiGLU over W = [Wg; Wu], N/2 a multiple of 16.
-extern "C" int llm_gemm_wide_bf16(const void* X, int ldx, const void* W, int ldw, void* C, int epilogue,
-                                  int M, int N, int K, hipStream_t stream) {
-  if (M <= 0 || N <= 0 || K < WD_BK || (K % WD_BK) || ldx < K || ldw < K || (ldx & 7) || (ldw & 7)) return LLM_ERR_ARG;
-  if ((((uintptr_t)X) | ((uintptr_t)W) | ((uintptr_t)C)) & 15) return LLM_ERR_ARG;
-  const int n_out = (epilogue == WD_EPI_SWIGLU) ? N / 2 : N;
-  if (epilogue != WD_EPI_NONE && epilogue != WD_EPI_SWIGLU) return LLM_ERR_ARG;
-  if (X == nullptr || W == nullptr || C == nullptr) return LLM_ERR_ARG;
-  if (epilogue == WD_EPI_SWIGLU && (N & 31)) return LLM_ERR_ARG;
-  if (n_out & 3) return LLM_ERR_ARG;
-  const int m_tiles = (M + WD_BM - 1) / WD_BM;
-  const int per = (epilogue == WD_EPI_SWIGLU) ? 128 : WD_BN;
+template <int EPI, int BM>
+static int launch_wide(const void* X, int ldx, const void* W, int ldw, void* C, int M, int N, int K,
+                       int n_out, hipStream_t stream) {
+  const int m_tiles = (M + BM - 1) / BM;
+  const int per = (EPI == WD_EPI_SWIGLU) ? 128 : WD_BN;
   const int n_tiles = (n_out + per - 1) / per;
   const long long blocks = 8LL * ((m_tiles + 7) / 8) * 8 * ((n_tiles + 7) / 8);   // bands of 8 tiles of X rows; surplus blocks leave at once
   if (blocks > 0x7fffffffLL) return LLM_ERR_ARG;
-  const int lds_bytes = 8 * 64 * (256 + 16);      // the epilogue's regions; the two buffers of the loop take 128 KiB
+  // the two buffers of the loop, or the epilogue's regions (8 waves x 64 rows of up to 272 bytes)
+  const int lds_bytes = (2 * (256 + BM) * 128 > 8 * 64 * 272) ? 2 * (256 + BM) * 128 : 8 * 64 * 272;
   // more than 64 KiB of LDS has to be asked for, once per device and kernel
-  static bool asked[2][64];
+  static bool asked[64];
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return LLM_ERR_LAUNCH;
-  const int e = (epilogue == WD_EPI_SWIGLU) ? 1 : 0;
-  const void* fn = e ? (const void*)gemm_wide_kernel<WD_EPI_SWIGLU> : (const void*)gemm_wide_kernel<WD_EPI_NONE>;
-  if (!asked[e][dev]) {
-    if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes) != hipSuccess) return LLM_ERR_LAUNCH;
-    asked[e][dev] = true;
+  if (!asked[dev]) {
+    if (hipFuncSetAttribute((const void*)gemm_wide_kernel<EPI, BM>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                            lds_bytes) != hipSuccess)
+      return LLM_ERR_LAUNCH;
+    asked[dev] = true;
   }
-  if (e)
-    gemm_wide_kernel<WD_EPI_SWIGLU><<<(unsigned)blocks, WD_NT, lds_bytes, stream>>>(
-        (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (bf16_t*)C, M, N, K, n_out, m_tiles, n_tiles);
-  else
-    gemm_wide_kernel<WD_EPI_NONE><<<(unsigned)blocks, WD_NT, lds_bytes, stream>>>(
-        (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (bf16_t*)C, M, N, K, n_out, m_tiles, n_tiles);
+  gemm_wide_kernel<EPI, BM><<<(unsigned)blocks, WD_NT, lds_bytes, stream>>>(
+      (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (bf16_t*)C, M, N, K, n_out, m_tiles, n_tiles);
   return llm_launch_status();
+}
+
+// X [M, K] rows ldx apart, W [N, K] rows ldw apart (both bfloat16, K a multiple of 64, 16-byte aligned rows);
+// epilogue 0: C [M, N]; 1: C [M, N/2], SwiGLU over W = [Wg; Wu], N/2 a multiple of 16.
+// block_rows: rows of X a block takes, 256 or 128 (half the arithmetic per byte a unit reads, twice
+// the blocks: for steps whose tiles of 256 rows would leave units idle).
+extern "C" int llm_gemm_wide_bf16(const void* X, int ldx, const void* W, int ldw, void* C, int epilogue,
+                                  int block_rows, int M, int N, int K, hipStream_t stream) {
+  if (M <= 0 || N <= 0 || K < WD_BK || (K % WD_BK) || ldx < K || ldw < K || (ldx & 7) || (ldw & 7)) return LLM_ERR_ARG;
+  if ((((uintptr_t)X) | ((uintptr_t)W) | ((uintptr_t)C)) & 15) return LLM_ERR_ARG;
+  if (epilogue != WD_EPI_NONE && epilogue != WD_EPI_SWIGLU) return LLM_ERR_ARG;
+  if (block_rows != 256 && block_rows != 128) return LLM_ERR_ARG;
+  if (X == nullptr || W == nullptr || C == nullptr) return LLM_ERR_ARG;
+  const int n_out = (epilogue == WD_EPI_SWIGLU) ? N / 2 : N;
+  if (epilogue == WD_EPI_SWIGLU && (N & 31)) return LLM_ERR_ARG;
+  if (n_out & 3) return LLM_ERR_ARG;
+  if (epilogue == WD_EPI_SWIGLU)
+    return block_rows == 256 ? launch_wide<WD_EPI_SWIGLU, 256>(X, ldx, W, ldw, C, M, N, K, n_out, stream)
+                             : launch_wide<WD_EPI_SWIGLU, 128>(X, ldx, W, ldw, C, M, N, K, n_out, stream);
+  return block_rows == 256 ? launch_wide<WD_EPI_NONE, 256>(X, ldx, W, ldw, C, M, N, K, n_out, stream)
+                           : launch_wide<WD_EPI_NONE, 128>(X, ldx, W, ldw, C, M, N, K, n_out, stream);
 }

@@ -47,7 +47,7 @@ _SIGNATURES = {
                           _f, _i, _vp],
     "llm_gemm_skinny_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp],
     "llm_gemm_mid_bf16": [_vp, _i, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp],
-    "llm_gemm_wide_bf16": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _vp],
+    "llm_gemm_wide_bf16": [_vp, _i, _vp, _i, _vp, _i, _i, _i, _i, _i, _vp],
     "llm_gemm_skinny_norm_bf16": [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp, _i, _f, _vp],
     "llm_attention_mfma_supported": [_i],
     "llm_attention_prefill_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i,
@@ -121,18 +121,17 @@ class HipOps:
     MID_FROM = 33
     MID_HEAD = True         # logits of 65 to 128 rows by it too
     # Beyond MID_ROWS rows the gate/up product with its SwiGLU is a kernel of ours where its tiles
-    # (256 rows by 128 outputs) fill whole rounds of the compute units to at least WIDE_FILL, and K
-    # is at most WIDE_MAX_K: there it beats the library's product followed by the SiLU-mul kernel
-    # (the two timed in turns, 1B shape: 111 against 136 us at 2,048 rows, 58 against 74 at 1,024,
-    # 210 against 234 at 4,096, 870 against 931 at 16,384; 3B: 155 against 167, 81 against 89, 313
-    # against 328, 1,260 against 1,284).  With half-empty rounds (512 rows: 47 against 44) the
-    # library's stays.  What the kernel saves is the SiLU-mul pass, 6 bytes an output against the
-    # product's 4 K flops: a fifth of the product's time at K = 2,048, an eighth at 3,072, a tenth
-    # at 4,096, while its plain product is 7 to 10 % behind the library's at large sizes; so beyond
-    # K of about 3,500 it loses (8B, K = 4,096: 413 against 392 at 2,048 rows, 773 against 718 at
-    # 4,096).
-    WIDE_FILL = 0.8
-    WIDE_MAX_K = 3072
+    # (256 or 128 rows by 128 outputs) would be filled, over whole rounds of the compute units, to
+    # at least WIDE_FILL: there it beats the library's product followed by the SiLU-mul kernel, which reads
+    # gate and up again (the two timed in turns, 1B shape: 105 against 121 us at 2,048 rows, 56
+    # against 69 at 1,024, 206 against 234 at 4,096, 817 against 927 at 16,384, and with 128 rows a
+    # block 35 against 42 at 512 and 32 against 36 at 384; 3B: 152 against 163, 79 against 90, 297
+    # against 315, 1,195 against 1,269, and 52 against 55 at 512; 8B: 95 against 112 at 512, 191
+    # against 207 at 1,024, the same from 2,048 on).  With half-empty rounds the library's stays
+    # (1B, 256 rows: a tile of 128 rows fills half a round, 31 against 33; some such steps would
+    # gain, others lose 10 %).  K beyond WIDE_MAX_K has not been measured.
+    WIDE_FILL = 0.75
+    WIDE_MAX_K = 4096
     # Launch sizes below are in blocks per compute unit; ``__init__`` multiplies them by the
     # device's number of units (the figures in the comments were measured on 256 units).
     MID_BLOCKS_PER_UNIT = 1.0       # blocks that the slices of K of the product for 33 to 128 rows aim at (half and twice as many lose 8 to 10 % of a prompt step of 128 tokens at the 3B and 8B shapes: fewer blocks, or more matrices for the norm to add)
@@ -415,24 +414,29 @@ class HipOps:
                 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and k % 128 == 0)
 
     def _wide_ok(self, x, w, m, k, inter):
-        """Whether the gate/up product of ``m`` rows goes to the kernel for many rows."""
+        """The rows of X a block takes (256 or 128) if the gate/up product of ``m`` rows goes to
+        the kernel for many rows, else 0."""
         if not (self.fast_gemm and self.wide_gemm and m > self.MID_ROWS and not isinstance(x, NormedRows)):
-            return False
+            return 0
         wp = self._plain(w)
         if not (x.dtype == torch.bfloat16 and wp.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1
                 and x.stride(0) >= k and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0
                 and wp.stride(1) == 1 and wp.stride(0) >= k and wp.stride(0) % 8 == 0 and wp.data_ptr() % 16 == 0
                 and k % 64 == 0 and k <= self.WIDE_MAX_K and inter % 16 == 0):
-            return False
-        tiles = -(-m // 256) * -(-inter // 128)
-        rounds = -(-tiles // self.units)
-        return tiles >= self.WIDE_FILL * rounds * self.units
+            return 0
+        for block_rows in (256, 128):
+            tiles = -(-m // block_rows) * -(-inter // 128)
+            rounds = -(-tiles // self.units)
+            # the share of the rounds' tiles that the step's rows and outputs really fill
+            if m * inter >= self.WIDE_FILL * rounds * self.units * block_rows * 128:
+                return block_rows
+        return 0
 
-    def _wide(self, x, w, out, epilogue):
+    def _wide(self, x, w, out, epilogue, block_rows=256):
         wp = self._plain(w)
         n, k = wp.shape
         self._check(self.lib.llm_gemm_wide_bf16(
-            x.data_ptr(), x.stride(0), wp.data_ptr(), wp.stride(0), out.data_ptr(), epilogue,
+            x.data_ptr(), x.stride(0), wp.data_ptr(), wp.stride(0), out.data_ptr(), epilogue, block_rows,
             x.shape[0], n, k, self._stream()), "gemm_wide_bf16")
         return out
 
@@ -586,11 +590,11 @@ class HipOps:
             self._weight(self._plain(w), "linear weight")
             return self._mid(x, w, torch.empty((m, inter), dtype=torch.bfloat16, device=self.device),
                              self._EPI_SWIGLU)
-        if dtype == torch.bfloat16 and self._wide_ok(x, w, m, k, inter):
+        if dtype == torch.bfloat16 and (block_rows := self._wide_ok(x, w, m, k, inter)):
             self._weight(self._plain(w), "linear weight")
             self._dev(x, "linear input")
             return self._wide(x, w, torch.empty((m, inter), dtype=torch.bfloat16, device=self.device),
-                              self._EPI_SWIGLU)
+                              self._EPI_SWIGLU, block_rows)
         return self.silu_mul(self.linear(x, w, None, x.dtype))
 
     def silu_mul(self, gu):

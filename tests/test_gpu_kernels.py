@@ -530,38 +530,43 @@ def test_gemm_mid_refuses(ops):
 
 
 # ---------------------------------------------------------------- the product for many rows
+@pytest.mark.parametrize("block_rows", [256, 128])
 @pytest.mark.parametrize("mnk", [(129, 64, 64), (300, 520, 128), (2048, 512, 256), (257, 1000, 192), (600, 264, 4096)])
-def test_gemm_wide(ops, mnk):
-    """Plain, against float64: rows and weight rows that are no multiples of the tile, one tile of
-    K and many, a weight whose rows are no multiple of 8 (single stores at the edge)."""
+def test_gemm_wide(ops, mnk, block_rows):
+    """Plain, against float64, both sizes of block: rows and weight rows that are no multiples of
+    the tile, one tile of K and many, a weight whose rows are no multiple of 8 (single stores at
+    the edge)."""
     m, n, k = mnk
     x = rnd((m, k), torch.bfloat16, 3).cuda()
     w = rnd((n, k), torch.bfloat16, 4, scale=0.05).cuda()
-    out = ops._wide(x, w, torch.full((m, n), 7.0, dtype=torch.bfloat16, device="cuda"), ops._EPI_NONE)
+    out = ops._wide(x, w, torch.full((m, n), 7.0, dtype=torch.bfloat16, device="cuda"), ops._EPI_NONE, block_rows)
     assert close(out, x.double() @ w.double().t(), torch.bfloat16)
     # rows of X that lie apart, a prepared weight
     wide_x = torch.cat([x, x], dim=1)[:, :k]
     assert wide_x.stride(0) == 2 * k
-    again = ops._wide(wide_x, ops.prepare_weight(w), torch.empty((m, n), dtype=torch.bfloat16, device="cuda"), ops._EPI_NONE)
+    again = ops._wide(wide_x, ops.prepare_weight(w), torch.empty((m, n), dtype=torch.bfloat16, device="cuda"), ops._EPI_NONE, block_rows)
     assert torch.equal(again, out)
 
 
+@pytest.mark.parametrize("block_rows", [256, 128])
 @pytest.mark.parametrize("mik", [(257, 512, 192), (1000, 208, 64), (130, 16, 128), (2048, 8192, 2048)])
-def test_gemm_wide_swiglu(ops, mik):
+def test_gemm_wide_swiglu(ops, mik, block_rows):
     """silu(gate) * up over a stacked weight, gate and up rounded to bfloat16 first as the unfused
     path stores them; outputs that are no multiple of the tile."""
     m, inter, k = mik
     x = rnd((m, k), torch.bfloat16, 5).cuda()
     w = rnd((2 * inter, k), torch.bfloat16, 6, scale=0.05).cuda()
-    out = ops._wide(x, w, torch.empty((m, inter), dtype=torch.bfloat16, device="cuda"), ops._EPI_SWIGLU)
+    out = ops._wide(x, w, torch.empty((m, inter), dtype=torch.bfloat16, device="cuda"), ops._EPI_SWIGLU, block_rows)
     gu = (x.double() @ w.double().t()).bfloat16().double()
     g, u = gu[:, :inter], gu[:, inter:]
     ref = u * g / (1 + torch.exp(-g))
     err = ((out.double() - ref).abs() / (ref.abs() + ref.abs().mean())).max().item()
     assert err < 0.02, err
-    # a row's bits do not depend on the other rows of the step
-    fewer = ops._wide(x[:129].contiguous(), w, torch.empty((129, inter), dtype=torch.bfloat16, device="cuda"), ops._EPI_SWIGLU)
+    # a row's bits do not depend on the other rows of the step, nor on the size of block
+    fewer = ops._wide(x[:129].contiguous(), w, torch.empty((129, inter), dtype=torch.bfloat16, device="cuda"), ops._EPI_SWIGLU, block_rows)
     assert torch.equal(fewer, out[:129])
+    other = ops._wide(x, w, torch.empty((m, inter), dtype=torch.bfloat16, device="cuda"), ops._EPI_SWIGLU, 384 - block_rows)
+    assert torch.equal(other, out)
 
 
 def test_gemm_wide_is_used_where_its_tiles_fill_the_device(ops, monkeypatch):
@@ -572,11 +577,13 @@ def test_gemm_wide_is_used_where_its_tiles_fill_the_device(ops, monkeypatch):
     real = ops._wide
     monkeypatch.setattr(ops, "_wide", lambda *a: (calls.append(a[0].shape[0]), real(*a))[1])
     w = ops.prepare_weight(rnd((2 * 8192, 256), torch.bfloat16, 6, scale=0.05).cuda())
-    for m, used in ((1024, True), (2048, True), (520, False), (128, False)):
+    sizes = []
+    monkeypatch.setattr(ops, "_wide", lambda *a: (calls.append(a[0].shape[0]), sizes.append(a[4]), real(*a))[2])
+    for m, used in ((1024, 256), (2048, 256), (768, 256), (512, 128), (384, 128), (520, 0), (700, 0), (200, 0), (128, 0)):
         x = rnd((m, 256), torch.bfloat16, m).cuda()
-        calls.clear()
+        calls.clear(), sizes.clear()
         out = ops.linear_swiglu(x, w)
-        assert bool(calls) == used, (m, calls)
+        assert (sizes[0] if calls else 0) == used and ops._wide_ok(x, w, m, 256, 8192) == used, (m, calls, sizes)
         gu = (x.double() @ w.w.double().t()).bfloat16().double()
         ref = gu[:, 8192:] * gu[:, :8192] / (1 + torch.exp(-gu[:, :8192]))
         err = ((out.double() - ref).abs() / (ref.abs() + ref.abs().mean())).max().item()
