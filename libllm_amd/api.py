@@ -112,12 +112,14 @@ class Model:
     def __init__(self, config_file: str, device: Union[Device, str] = Device.AUTO, dtype: str = "bfloat16",
                  max_tokens: int = 8192, max_batch: int = 64, ops=None, use_graphs: bool = True,
                  random_weights: bool = False, seed: int = 0, keep_float32: bool = False,
-                 tiled_weights: bool = True) -> None:
+                 tiled_weights: bool = True, max_prompt_rows: int = 16384) -> None:
         """``config_file``: the model folder, or the config.json inside it.  ``device``: a Device
         or one of "auto", "cuda", "hip", "cpu".  With ``random_weights`` only config.json is read
         and every tensor is drawn from ``seed``.  ``keep_float32``: in bfloat16 mode, matrices
         that the file stores in 32-bit stay float32 instead of becoming bfloat16.
-        ``tiled_weights=False``: the matrices are held once, not twice (see ``load_engine``)."""
+        ``tiled_weights=False``: the matrices are held once, not twice (see ``load_engine``).
+        ``max_prompt_rows``: the most rows one prompt step of ``generate`` and ``complete``
+        brings (it bounds a step's activations); longer batches of prompts take several steps."""
         if int(parse_device(device)) == int(Device.CPU):
             raise ConfigError("this library has no CPU path; use Device.AUTO or Device.GPU")
         model_dir = os.path.dirname(config_file) if os.path.isfile(config_file) else config_file
@@ -134,7 +136,8 @@ class Model:
         spec = self.engine.model.spec
         self._sampler = Sampler(self.engine.ops, spec.vocab)
         self._generator = Generator(self.engine, self._sampler, spec.stop_tokens, spec.max_position,
-                                    self.engine.cache.n_pages, PAGE, max_batch=max_batch)
+                                    self.engine.cache.n_pages, PAGE, max_batch=max_batch,
+                                    max_prompt_rows=max_prompt_rows)
         self._tok = None
 
     @property

@@ -5,8 +5,9 @@
   ends; a slot that is taken again starts at length 0 with zeroed state.
 * A *group* collects the cache entries whose mixers keep the same kind of keys and values (all
   positions, or a window of them, with given head count and size).  Each group has page pools of
-  its own: ``k`` of shape ``[entries, pages + 1, kv_heads, page, head_dim]``, ``v`` of shape
-  ``[entries, pages + 1, kv_heads, head_dim, page]`` and a table
+  its own: ``k`` of shape ``[entries, pages + 1, kv_heads, ceil(head_dim / 16), page, 16]``
+  (blocks of 16 dims), ``v`` of shape ``[entries, pages + 1, kv_heads, 2, head_dim, page / 2]``
+  (halves of 32 positions; ``layout.py`` says why) and a table
   ``[slots + 1, pages_per_sequence]`` from (slot, position // page) to a page.  The last page and
   the last slot are a sink for padding rows and belong to nobody.
 * Per-sequence *state* of fixed size: for each cache entry whose mixer asks for it, a tensor

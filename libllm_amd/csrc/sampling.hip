@@ -515,7 +515,7 @@ __device__ __forceinline__ unsigned long long nucleus_mass(float x, float inv_te
 __device__ void nucleus_cross(const float* __restrict__ x, int V, float inv_temp, float mx, float inv_z,
                               unsigned long long target, bool strict, NucleusShared& sh) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  if (tid == 0) { sh.prefix = 0u; sh.above = 0ull; }
+  if (tid == 0) { sh.prefix = 0u; sh.above = 0ull; sh.pe = 0ull; }
   __syncthreads();
   for (int pass = 0; pass < 4; ++pass) {
     const int shift = 24 - 8 * pass;
@@ -587,7 +587,10 @@ __device__ void nucleus_cross(const float* __restrict__ x, int V, float inv_temp
   int eq_total;
   const int eq_inc = block_inclusive_scan<int, NUC_NT>(eq_mine, sh.ibuf, &eq_total);
   if (eq_mine > 0 && eq_inc == eq_mine) sh.pe = nucleus_mass(eq_val, inv_temp, mx, inv_z);   // the first thread that has one
-  if (tid == 0) { sh.n_eq = eq_total; sh.pick = 0; }
+  // (the descent may end on a key that no token has, when every probability rounds to nothing or
+  // the logits are not finite: then nobody writes the place, and it is token 0 with nothing kept
+  // beyond what lies above)
+  if (tid == 0) { sh.n_eq = eq_total; sh.pick = 0; sh.kept = sh.above; }
   __syncthreads();
   const unsigned long long pe = sh.pe, above = sh.above;
   long long c = 1;

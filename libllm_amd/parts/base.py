@@ -91,9 +91,17 @@ class StepContext:
     Device tensors (int32): ``tokens`` [M], ``tok_pos`` [M] absolute position of each token,
     ``tok_seq`` [M] index of its sequence in this step, ``seq_start`` [B+1] offsets of the
     sequences in the packed rows, ``seq_slot`` [B], ``seq_pos0`` [B] tokens already cached
-    before the step.  Host values: ``seq_lens`` and ``seq_pos0_host`` (lists), ``max_new``
-    (largest number of new tokens of a sequence) and ``max_ctx`` (largest cached length after
-    the step); under a captured graph the last two are upper bounds.
+    before the step.  Host values: ``seq_lens``, ``seq_pos0_host`` and ``seq_slot_host`` (lists),
+    ``max_new`` (largest number of new tokens of a sequence) and ``max_ctx`` (largest cached
+    length after the step).
+
+    ``captured`` says that the step runs over the fixed buffers of a captured shape.  Then
+    ``max_new`` and ``max_ctx`` are upper bounds (kernels size their grids by them and read the
+    true lengths from device memory), and the host lists describe the padded step: padding rows
+    are sequences in the sink slot.  The lists are filled in before every run of the step, so a
+    part that runs from the host (``graph_safe = False``) finds them valid, with ``captured`` set
+    or not; a part whose work is recorded into a graph (``graph_safe = True``) must not read them
+    at all, since what it read at the recording would be replayed for every later step.
     """
 
     def __init__(self, ops, dtype, n_tokens, n_seqs):
@@ -118,7 +126,7 @@ class StepContext:
         # may then prepare that norm (``ops.linear(..., then_norm=)``).  Set by blocks.
         self.then_norm = None
         self.norm_after_block = None   # the norm that reads the stream first after the running block, if known
-        self.captured = False      # running under graph capture: host lists are not valid
+        self.captured = False      # the step runs over the fixed buffers of a captured shape (see above)
         self.want_all_rows = False  # the logits of every row are wanted, in order (a decode step): the last norm gathers nothing
         self._kv: Dict[int, KVView] = {}
         self._state: Dict[int, torch.Tensor] = {}

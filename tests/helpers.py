@@ -149,12 +149,12 @@ def read_kv(kv, slot, length):
 def attention_oracle(q, keys, values, pos, scale, window=0):
     """q [n_heads, hd], keys/values [L, n_kv, hd] (float64): the query at position ``pos`` sees
     keys max(0, pos - window + 1) .. pos; softmax(q k / sqrt) v with grouped heads."""
-    n_heads = q.shape[0]
+    n_heads, hd = q.shape
     n_kv = keys.shape[1]
     group = n_heads // n_kv
     first = max(0, pos - window + 1) if window else 0
-    k = keys[first:pos + 1].repeat_interleave(group, dim=1)
-    v = values[first:pos + 1].repeat_interleave(group, dim=1)
-    s = torch.einsum("hd,lhd->hl", q, k) * scale
+    k, v = keys[first:pos + 1], values[first:pos + 1]
+    # query head h reads kv head h // group (src/flint/operators.cc:43-56 repeats the kv heads)
+    s = torch.einsum("kgd,lkd->kgl", q.reshape(n_kv, group, hd), k) * scale
     p = torch.softmax(s, dim=-1)
-    return torch.einsum("hl,lhd->hd", p, v)
+    return torch.einsum("kgl,lkd->kgd", p, v).reshape(n_heads, hd)

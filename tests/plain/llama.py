@@ -152,11 +152,35 @@ def attention(q, k, v, causal, store=None):
         k = expand_kv_heads(k, n_heads)
         v = expand_kv_heads(v, n_heads)
     s = math.sqrt(1.0 / math.sqrt(hd))
+    if causal and lq > ROW_BLOCK:
+        # Long sequences, a block of query rows at a time with the keys that the block's last row
+        # sees: the keys left out are masked for every row of the block, so each row's softmax is
+        # over the same terms as in one piece; only the memory for the scores is smaller.
+        out = np.empty_like(q)
+        for r0 in range(0, lq, ROW_BLOCK):
+            r1 = min(lq, r0 + ROW_BLOCK)
+            seen = lk - lq + r1
+            out[:, r0:r1] = _attention_rows(q[:, r0:r1], k[:, :seen], v[:, :seen], s, True, store)
+        return out
+    return _attention_rows(q, k, v, s, causal, store)
+
+
+ROW_BLOCK = 1024
+
+
+def _attention_rows(q, k, v, s, causal, store):
+    lq, lk = q.shape[1], k.shape[1]
     scores = (q * s) @ np.swapaxes(k * s, -1, -2)
     if causal and lq > 1:
-        scores = scores + causal_mask(lk)[lk - lq:lk][None]
+        scores = scores + causal_mask_rows(lk, lq)[None]
     p = softmax(scores)
     return (p if store is None else store(p)) @ v
+
+
+def causal_mask_rows(lk, lq):
+    """The last ``lq`` rows of causal_mask(lk), made without the rows above them."""
+    rows = np.arange(lk - lq, lk)[:, None]
+    return np.where(np.arange(lk)[None, :] > rows, -np.inf, 0.0)
 
 
 # --------------------------------------------------------------------------- blocks

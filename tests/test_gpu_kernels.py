@@ -531,16 +531,20 @@ def test_gemm_mid_refuses(ops):
 
 # ---------------------------------------------------------------- the product for many rows
 @pytest.mark.parametrize("block_rows", [256, 128])
-@pytest.mark.parametrize("mnk", [(129, 64, 64), (300, 520, 128), (2048, 512, 256), (257, 1000, 192), (600, 264, 4096)])
+@pytest.mark.parametrize("mnk", [(129, 64, 64), (300, 520, 128), (2048, 512, 256), (257, 1000, 192), (600, 264, 4096),
+                                 (300, 268, 128), (129, 100, 64), (513, 4, 64)])
 def test_gemm_wide(ops, mnk, block_rows):
     """Plain, against float64, both sizes of block: rows and weight rows that are no multiples of
-    the tile, one tile of K and many, a weight whose rows are no multiple of 8 (single stores at
-    the edge)."""
+    the tile, one tile of K and many, and weights whose number of rows is a multiple of 4 and not
+    of 8 (268, 100, 4: every store is then of single elements, and the last lanes of a row store
+    four).  The output lies inside a larger buffer of sentinels: nothing is written past it."""
     m, n, k = mnk
     x = rnd((m, k), torch.bfloat16, 3).cuda()
     w = rnd((n, k), torch.bfloat16, 4, scale=0.05).cuda()
-    out = ops._wide(x, w, torch.full((m, n), 7.0, dtype=torch.bfloat16, device="cuda"), ops._EPI_NONE, block_rows)
+    buf = torch.full((m * n + 64,), 7.0, dtype=torch.bfloat16, device="cuda")
+    out = ops._wide(x, w, buf[:m * n].view(m, n), ops._EPI_NONE, block_rows)
     assert close(out, x.double() @ w.double().t(), torch.bfloat16)
+    assert (buf[m * n:] == 7.0).all()
     # rows of X that lie apart, a prepared weight
     wide_x = torch.cat([x, x], dim=1)[:, :k]
     assert wide_x.stride(0) == 2 * k
@@ -831,14 +835,17 @@ def test_rope_pairing_and_sign(ops):
 
 
 # ------------------------------------------------------------------------------- attention
-def run_attention(ops, dtype, n_heads, n_kv, hd, seqs, window=0, seed=0, boost=None, fast=True, tiles=0):
-    """seqs: (slot, past, new).  Returns (out, oracle) over all new tokens."""
+def run_attention(ops, dtype, n_heads, n_kv, hd, seqs, window=0, seed=0, boost=None, fast=True, tiles=0,
+                  checked=None):
+    """seqs: (slot, past, new).  Returns (out, oracle) over all new tokens, or, with ``checked``,
+    over that many rows of every sequence (its first and last, those next to every border of a
+    block of 128 rows among them, the others drawn)."""
     ctx = make_ctx(ops, dtype, seqs)
     pages = max((p + n + PAGE - 1) // PAGE for _, p, n in seqs)
     kv = make_kv("cuda", dtype, max(s for s, _, _ in seqs) + 1, pages, n_kv, hd, seed=seed)
     scale = hd ** -0.5
     q = rnd((ctx.n_tokens, n_heads * hd + 24), dtype, seed + 1)   # wider rows: a stride is honoured
-    ref, o = [], 0
+    ref, rows, o = [], [], 0
     for slot, past, new in seqs:
         keys = rnd((past + new, n_kv, hd), dtype, seed + 10 + slot)
         vals = rnd((past + new, n_kv, hd), dtype, seed + 20 + slot)
@@ -846,16 +853,24 @@ def run_attention(ops, dtype, n_heads, n_kv, hd, seqs, window=0, seed=0, boost=N
             key_pos, gain = boost
             keys[key_pos] = keys[key_pos] * gain
         fill_kv(kv, slot, keys, vals)
-        for t in range(new):
+        which = range(new)
+        if checked is not None and new > checked:
+            g = np.random.default_rng(seed + slot)
+            edge = [t for b in (g.integers(1, max(2, new // 128), size=4) * 128).tolist() for t in (b - 1, b)]
+            which = sorted({0, new - 1, *[t for t in edge if 0 <= t < new],
+                            *g.integers(0, new, size=checked).tolist()})[:checked + 10]
+        keys, vals = keys.double(), vals.double()
+        for t in which:
             qt = q[o + t, :n_heads * hd].double().reshape(n_heads, hd)
-            ref.append(attention_oracle(qt, keys.double(), vals.double(), past + t, scale, window).reshape(-1))
+            ref.append(attention_oracle(qt, keys, vals, past + t, scale, window).reshape(-1))
+            rows.append(o + t)
         o += new
     ops.fast_attention, ops.prompt_tiles = fast, tiles
     try:
         out = ops.attention(q.cuda(), n_heads, n_kv, hd, ctx, kv, scale, window)
     finally:
         ops.fast_attention, ops.prompt_tiles = True, 0
-    return out.double().cpu(), torch.stack(ref)
+    return out[torch.tensor(rows, device=out.device)].double().cpu(), torch.stack(ref)
 
 
 # (heads, kv heads, queries, keys, head size): the cases of src/flint/cuda/test.cc:349-362
@@ -951,6 +966,33 @@ def test_attention_decode_over_many_pages(ops, ctx_len, far):
     out, ref = run_attention(ops, torch.bfloat16, 8, 2, 64, [(0, ctx_len, 1)], seed=3, boost=(far, 12.0))
     assert max_err(out, ref) < BF16_2ULP
     out, ref = run_attention(ops, torch.bfloat16, 4, 1, 128, [(1, ctx_len // 2, 1), (0, ctx_len, 1)], seed=4)
+    assert max_err(out, ref) < BF16_2ULP
+
+
+@pytest.mark.parametrize("hd", [64, 128])
+@pytest.mark.parametrize("ctx_len,far", [(32768, 17), (131072, 70001), (131072, 131071)])
+def test_attention_decode_over_tens_of_thousands_of_keys(ops, hd, ctx_len, far):
+    """Contexts at which the measurements run and whose grids differ from the shorter ones': a
+    wave walks several pages in a row, and at 131,072 keys the merge is its loop form.  One
+    sequence with one far key that dominates, then eight of unequal lengths in one step."""
+    out, ref = run_attention(ops, torch.bfloat16, 8, 2, hd, [(0, ctx_len - 1, 1)], seed=hd, boost=(far, 12.0))
+    assert max_err(out, ref) < BF16_2ULP
+    lens = [ctx_len - 1, 5, ctx_len // 2 + 33, 4097, ctx_len - 64, 63, ctx_len // 3, 20000]
+    out, ref = run_attention(ops, torch.bfloat16, 4, 2, hd, [(i, n, 1) for i, n in enumerate(lens)], seed=hd + 5)
+    assert max_err(out, ref) < BF16_2ULP
+
+
+@pytest.mark.parametrize("tiles", [1, 2])
+@pytest.mark.parametrize("hd,rows", [(64, 8192), (128, 8192), (64, 16384), (128, 16384)])
+def test_prompt_attention_over_thousands_of_rows(ops, hd, rows, tiles):
+    """Prompts as long as the measured ones, in both forms of the kernel (one and two tiles of
+    rows a wave): some hundred rows of a fresh prompt against the oracle, one far key dominating;
+    then a prompt that continues a sequence, beside a short one."""
+    out, ref = run_attention(ops, torch.bfloat16, 4, 2, hd, [(0, 0, rows)], seed=rows + hd, boost=(rows // 3, 12.0),
+                             tiles=tiles, checked=120)
+    assert max_err(out, ref) < BF16_2ULP
+    out, ref = run_attention(ops, torch.bfloat16, 6, 2, hd, [(1, 0, 70), (0, 1000, rows - 1500)], seed=rows + hd + 1,
+                             tiles=tiles, checked=60)
     assert max_err(out, ref) < BF16_2ULP
 
 
@@ -1068,15 +1110,22 @@ def test_nucleus_without_a_limit_on_the_candidates(ops, vocab):
     src/libllm/generator.cc:66-90): the nucleus is the shortest prefix, in falling probability,
     that reaches top_p, however long.  Rows whose nucleus lies within the most probable 1,024
     tokens, rows as flat as to need most of the vocabulary (the walk over the whole vocabulary),
-    and a row of few distinct values (equal logits are ranked by index)."""
+    a row of few distinct values (equal logits are ranked by index), and flat rows in which a
+    third of the tokens are ruled out by a logit of minus infinity."""
     from plain import sampling
     g = torch.Generator().manual_seed(vocab)
     peaked = torch.randn((8, vocab), generator=g) * 4.0
     flat = torch.randn((8, vocab), generator=g) * 0.3
     stepped = torch.randint(0, 3, (8, vocab), generator=g).float() * 1.5
-    logits = torch.cat([peaked, flat, stepped])
+    holes = torch.randn((4, vocab), generator=g) * 0.3             # flat, with a third of the tokens ruled out
+    holes[:, ::3] = -math.inf
+    logits = torch.cat([peaked, flat, stepped, holes])
     rows = logits.shape[0]
     streams, counters = list(range(50, 50 + rows)), list(range(rows))
+    # a row in which nothing has any probability decides nothing, and still names a token
+    nothing = torch.full((2, vocab), -math.inf)
+    got = ops.sample(nothing.cuda(), 1.0, 0, 0.9, 99, [1, 2], [0, 0]).tolist()
+    assert all(0 <= t < vocab for t in got)
     for top_p, temp in ((0.9, 1.0), (0.5, 0.7), (0.999, 1.5)):
         got = ops.sample(logits.cuda(), temp, 0, top_p, 99, streams, counters).tolist()
         bad, long_ones = 0, 0

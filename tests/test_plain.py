@@ -179,6 +179,18 @@ def test_attention_mask_is_aligned_bottom_right():
     assert np.allclose(out2[:, :3], out[:, :3]) and not np.allclose(out2[:, 3:], out[:, 3:])
 
 
+def test_attention_in_blocks_of_rows_is_attention(monkeypatch):
+    """Long sequences go a block of query rows at a time; the mask's rows are then made without
+    the rows above them.  Both are the one-piece computation, term for term."""
+    assert np.array_equal(llama.causal_mask_rows(10, 4), llama.causal_mask(10)[6:10])      # src/flint/cpu/tensor.cc:86-98
+    assert np.array_equal(llama.causal_mask_rows(5, 5), llama.causal_mask(5))
+    k, v = rng(30).normal(size=(2, 23, 8)), rng(31).normal(size=(2, 23, 8))
+    q = rng(32).normal(size=(4, 19, 8))
+    whole = llama.attention(q, k, v, True)
+    monkeypatch.setattr(llama, "ROW_BLOCK", 5)
+    assert np.allclose(llama.attention(q, k, v, True), whole, rtol=1e-13, atol=1e-15)
+
+
 def test_grouped_heads_equal_repeated_kv_heads():
     q = rng(19).normal(size=(6, 4, 8))
     k, v = rng(20).normal(size=(2, 4, 8)), rng(21).normal(size=(2, 4, 8))
