@@ -4,14 +4,17 @@ random weights at batch 8 and a context of 4,096 tokens, plus the prefill of 2,0
 decoding at batch 1 and 64.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
+    python bench.py --sweep            # decode at batch 1..128 x context 4,096..131,072, as a table
 
 A step is one decode step inside the generation loop (``Generator.stream``, the loop that serves
 requests): the step function over the cache as a captured graph, arg-max sampling on the device,
 the sampled tokens fed back, the loop's own bookkeeping.  The prompts go through the loop's prompt
 steps, sized so that the timed steps end at the context length.  Beside the published peaks the
 line gives what this GPU reaches in kernels of this library that only read memory or only issue
-matrix instructions (``peak_measured``).  One JSON line is printed; everything else goes to
-standard error.
+matrix instructions (``peak_measured``).  The default run then builds the 3B and the 8B shape and
+runs their generation workloads (16 unequal prompts with 256 tokens each; 64 prompts of 1,024
+tokens with 512 tokens each), whose figures go into ``points``.  One JSON line is printed;
+everything else goes to standard error.
 
 The reference's own tool reports prompt and decoding speed of one sequence
 (src/libllm/benchmark_main.cc:52-86); it publishes no numbers, so ``vs_baseline`` is null.
@@ -111,54 +114,57 @@ def time_decode(gen, params, torch, batch, context, steps, warmup, vocab):
 
 
 def time_prefill(engine, torch, tokens, vocab, reps):
-    """Seconds of one prompt step of ``tokens`` tokens with the last row's logits wanted: the best
-    of ``reps`` runs after the first (the second run of a shape captures its graph, the later ones
-    replay it; the first replays still run slower than the ones after)."""
+    """Seconds of one prompt step of ``tokens`` tokens with the last row's logits wanted, ``reps``
+    runs after the first two (the second run of a shape captures its graph, the later ones replay
+    it): (median, minimum)."""
     from libllm_amd.engine import StepEntry
     g = torch.Generator().manual_seed(99)
     prompt = torch.randint(0, vocab, (tokens,), generator=g).tolist()
-    best = None
-    for r in range(reps + 1):
+    times = []
+    for r in range(reps + 2):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         engine.step([StepEntry("prefill", prompt, [tokens - 1])])
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         engine.end(["prefill"])
-        if r > 0:                                           # the first run warms up
-            best = dt if best is None else min(best, dt)
-    return best
+        if r > 1:                                           # the first run warms up, the second captures
+            times.append(dt)
+    times.sort()
+    return times[len(times) // 2], times[0]
 
 
-def run_workload(args, torch):
-    """The two generation workloads beside the headline: 16 prompts of unequal lengths (uniform in
-    [64, 2048]) with 256 tokens each, or 64 prompts of 1,024 tokens with 512 tokens each, through
-    the generation loop (greedy, no stop token)."""
+def workload_prompts(workload, vocab):
+    """(prompts, new tokens each) of a generation workload: 16 prompts of unequal lengths
+    (uniform in [64, 2048]) with 256 tokens each, or 64 prompts of 1,024 tokens with 512 each."""
     import numpy as np
+    rng = np.random.default_rng(0)
+    if workload == "batch64":
+        return [rng.integers(0, vocab, size=1024).tolist() for _ in range(64)], 512
+    return [rng.integers(0, vocab, size=int(n)).tolist() for n in rng.integers(64, 2049, size=16)], 256
 
+
+def time_workload(shape, workload, dtype, torch, reps=3):
+    """A generation workload through the generation loop (greedy, no stop token) on an engine of
+    its own: what the last of ``reps`` runs took (the first warms up; a shape's second coming
+    captures its graph).  Returns a record of plain numbers."""
     from libllm_amd.cache import PAGE
     from libllm_amd.config import config_from_dict
     from libllm_amd.engine import Generator
     from libllm_amd.runtime import random_engine
     from libllm_amd.sampling import Sampler, SamplingParams
     d = dict(FULL)
-    d.update(SHAPES[args.shape])
+    d.update(SHAPES[shape])
     d["eos_token_id"] = None
     cfg = config_from_dict(d)
-    rng = np.random.default_rng(0)
-    if args.workload == "batch64":
-        prompts = [rng.integers(0, cfg.vocab_size, size=1024).tolist() for _ in range(64)]
-        new = 512
-    else:
-        prompts = [rng.integers(0, cfg.vocab_size, size=int(n)).tolist()
-                   for n in rng.integers(64, 2049, size=16)]
-        new = 256
+    prompts, new = workload_prompts(workload, cfg.vocab_size)
     need = sum((len(p) + new + PAGE) // PAGE * PAGE for p in prompts) + 4096
-    engine = random_engine(cfg, seed=0, dtype=args.dtype, max_tokens=need)
+    engine = random_engine(cfg, seed=0, dtype=dtype, max_tokens=need)
     gen = Generator(engine, Sampler(engine.ops, cfg.vocab_size), (), cfg.max_position_embeddings,
                     engine.cache.n_pages, PAGE, max_batch=64)
-    result = None
-    for rep in range(3):                                   # the first run warms up; a shape's second coming captures its graph
+    itemsize = 2 if dtype == "bfloat16" else 4
+    rec = None
+    for rep in range(reps):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
         first = []
@@ -171,19 +177,110 @@ def run_workload(args, torch):
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         n_prompt, n_out = sum(len(p) for p in prompts), sum(len(o) for o in out)
-        result = {
-            "metric": "generated tok/s, %s workload (%s)" % (args.workload, NAMES[args.shape]),
-            "value": round((n_out - len(prompts)) / (dt - first[0]), 1), "unit": "tokens/s", "n_gpus": 1,
-            "steps": new - 1, "warmup": 0, "ms_per_step": round((dt - first[0]) / (new - 1) * 1e3, 3),
-            "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-            "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
-            "data": "synthetic: uniform random token ids, random weights N(0, 0.02)",
-            "config": {"model": NAMES[args.shape], "layers": cfg.num_hidden_layers, "prompts": len(prompts),
-                       "prompt_tokens": n_prompt, "new_tokens_each": new, "sampling": "greedy"},
-            "prefill": {"value": round(n_prompt / first[0], 1), "tokens": n_prompt, "ms": round(first[0] * 1e3, 2)},
-        }
-        log("run %d: first tokens after %.1f ms, then %.2f ms a step" % (rep, first[0] * 1e3, result["ms_per_step"]))
+        step_s = (dt - first[0]) / (new - 1)
+        # bytes of a decode step in the middle of the run: every weight once, and the cache the live requests hold
+        held = n_prompt + len(prompts) * new / 2.0
+        step_bytes = weight_bytes(cfg, itemsize) + held * kv_bytes_per_token(cfg, itemsize)
+        rec = {"cfg": cfg, "prompts": len(prompts), "prompt_tokens": n_prompt, "new": new,
+               "tok_s": (n_out - len(prompts)) / (dt - first[0]), "ms_per_step": step_s * 1e3,
+               "prefill_ms": first[0] * 1e3, "prefill_tok_s": n_prompt / first[0],
+               "prefill_frac": sum(prefill_flops(cfg, len(p)) for p in prompts) / first[0] / DENSE_FLOPS["bf16" if itemsize == 2 else "fp32"],
+               "hbm_frac": step_bytes / step_s / HBM_BYTES_PER_S}
+        log("%s %s run %d: first tokens after %.1f ms, then %.2f ms a step" % (shape, workload, rep, rec["prefill_ms"], rec["ms_per_step"]))
+    del gen, engine
+    import gc
+    gc.collect()
+    torch.cuda.empty_cache()
+    return rec
+
+
+def run_workload(args, torch):
+    """One of the two generation workloads beside the headline, as a line of its own."""
+    rec = time_workload(args.shape, args.workload, args.dtype, torch)
+    cfg = rec["cfg"]
+    result = {
+        "metric": "generated tok/s, %s workload (%s)" % (args.workload, NAMES[args.shape]),
+        "value": round(rec["tok_s"], 1), "unit": "tokens/s", "n_gpus": 1,
+        "steps": rec["new"] - 1, "warmup": 0, "ms_per_step": round(rec["ms_per_step"], 3),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: uniform random token ids, random weights N(0, 0.02)",
+        "config": {"model": NAMES[args.shape], "layers": cfg.num_hidden_layers, "prompts": rec["prompts"],
+                   "prompt_tokens": rec["prompt_tokens"], "new_tokens_each": rec["new"], "sampling": "greedy"},
+        "prefill": {"value": round(rec["prefill_tok_s"], 1), "tokens": rec["prompt_tokens"], "ms": round(rec["prefill_ms"], 2),
+                    "frac": round(rec["prefill_frac"], 4)},
+        "roofline": {"bound": "hbm", "achieved": round(rec["hbm_frac"] * HBM_BYTES_PER_S / 1e9, 1),
+                     "peak": HBM_BYTES_PER_S / 1e9, "unit": "GB/s", "frac": round(rec["hbm_frac"], 4)},
+    }
     print(json.dumps(result), flush=True)
+    return 0
+
+
+SWEEP_BATCHES = (1, 8, 16, 32, 64, 128)
+SWEEP_CONTEXTS = (4096, 16384, 32768, 131072)
+
+
+def run_sweep(args, torch):
+    """Decode steps at batch 1 to 128 and contexts of 4,096 to 131,072 tokens (where the cache fits
+    the device), each with its bytes / time against 8 TB/s.  The cache is not filled by prompts
+    (at 131,072 tokens a batch that alone would take minutes): the requests are given their pages
+    and lengths in the cache's books, the pages hold random values, and the step function decodes
+    from there, arg-max on the device and the tokens fed back without the host reading them, as
+    the generation loop queues them."""
+    from libllm_amd.config import config_from_dict
+    from libllm_amd.engine import StepEntry
+    from libllm_amd.runtime import random_engine
+    d = dict(FULL)
+    d.update(SHAPES[args.shape])
+    cfg = config_from_dict(d)
+    itemsize = 2 if args.dtype == "bfloat16" else 4
+    free, _ = torch.cuda.mem_get_info()
+    per_token = kv_bytes_per_token(cfg, itemsize)
+    room = int((free - 2.2 * weight_bytes(cfg, itemsize) - (8 << 30)) / per_token)
+    cells = [(b, c) for c in SWEEP_CONTEXTS for b in SWEEP_BATCHES if b * (c + 64) <= room]
+    max_tokens = max(b * (c + 64) for b, c in cells)
+    log("cache for %d tokens (%.0f GB); %d cells" % (max_tokens, max_tokens * per_token / 1e9, len(cells)))
+    engine = random_engine(cfg, seed=0, dtype=args.dtype, max_tokens=max_tokens, max_slots=max(SWEEP_BATCHES))
+    for g in engine.cache.groups:
+        for plane in g.planes.values():
+            plane.normal_()
+    steps, warmup = args.steps, args.warmup
+    points, table = {}, {}
+    for b, c in cells:
+        ids = [("sweep", b, c, i) for i in range(b)]
+        for r in ids:                                       # the books only: pages and lengths, no prompt step
+            slot = engine.cache.admit(r)
+            engine.cache.reserve(slot, c - steps - warmup - 1)
+            engine.cache.commit(slot, c - steps - warmup - 1)
+        engine.cache.flush()
+        tokens = torch.zeros((b,), dtype=torch.int32, device=engine.device)
+        entries = [StepEntry(r, [0], [0]) for r in ids]
+        for k in range(warmup + steps):
+            if k == warmup:
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+            tokens = engine.ops.argmax(engine.step(entries, tokens_device=tokens))
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        engine.end(ids)
+        step_bytes = weight_bytes(cfg, itemsize) + b * (c - steps / 2.0) * per_token
+        frac = step_bytes / dt / HBM_BYTES_PER_S
+        points["b%d_c%d" % (b, c)] = round(b / dt, 1)
+        points["b%d_c%d_hbm_frac" % (b, c)] = round(frac, 4)
+        table[(b, c)] = (dt * 1e3, frac)
+        log("batch %3d, context %6d: %.3f ms a step, %.0f tok/s, %.2f of 8 TB/s" % (b, c, dt * 1e3, b / dt, frac))
+    log("ms a step (fraction of 8 TB/s), %s, %s:" % (NAMES[args.shape], args.dtype))
+    log("%8s" % "batch" + "".join("%18d" % c for c in SWEEP_CONTEXTS))
+    for b in SWEEP_BATCHES:
+        log("%8d" % b + "".join(("%11.3f (%.2f)" % table[(b, c)]) if (b, c) in table else "%18s" % "-" for c in SWEEP_CONTEXTS))
+    best = max(points[k] for k in points if not k.endswith("_frac"))
+    print(json.dumps({
+        "metric": "decode tok/s over batch x context (%s)" % NAMES[args.shape], "value": best, "unit": "tokens/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": None, "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "bf16" if itemsize == 2 else "fp32",
+        "data": "synthetic: random cache contents, random weights N(0, 0.02)",
+        "config": {"model": NAMES[args.shape], "layers": cfg.num_hidden_layers, "sampling": "greedy"},
+        "points": points}), flush=True)
     return 0
 
 
@@ -203,6 +300,10 @@ def main() -> int:
                     help="greedy, or the command line's default (temperature 1, top-k 50, top-p 0.8)")
     ap.add_argument("--workload", choices=["unequal16", "batch64"],
                     help="run a generation workload through the generation loop instead")
+    ap.add_argument("--sweep", action="store_true",
+                    help="decode steps at batch 1 to 128 and contexts of 4,096 to 131,072 tokens, as a table")
+    ap.add_argument("--no-workloads", action="store_true",
+                    help="skip the generation workloads of the 3B and 8B shapes")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU only: this library does not run on several (--gpus %d)" % args.gpus)
@@ -212,6 +313,8 @@ def main() -> int:
 
     if args.workload:
         return run_workload(args, torch)
+    if args.sweep:
+        return run_sweep(args, torch)
 
     from libllm_amd.cache import PAGE
     from libllm_amd.config import config_from_dict
@@ -241,9 +344,9 @@ def main() -> int:
     log("measured on this GPU: read %.0f GB/s, copy %.0f GB/s, bf16 matrix cores %.0f TFLOP/s, fp32 %.1f TFLOP/s"
         % (peaks["read_GBs"], peaks["copy_GBs"], peaks["bf16_TFs"], peaks["fp32_TFs"]))
 
-    pre_s = time_prefill(engine, torch, args.prefill, vocab, reps=10)
+    pre_s, pre_min = time_prefill(engine, torch, args.prefill, vocab, reps=11)
     pf = prefill_flops(cfg, args.prefill)
-    log("prefill of %d tokens: %.2f ms" % (args.prefill, pre_s * 1e3))
+    log("prefill of %d tokens: %.2f ms (the median of 11 runs; the fastest %.2f)" % (args.prefill, pre_s * 1e3, pre_min * 1e3))
 
     dt = time_decode(gen, params, torch, args.batch, args.context, args.steps, args.warmup, vocab)
     ms = dt / args.steps * 1e3
@@ -259,7 +362,24 @@ def main() -> int:
         for b in (1, 64):
             dtb = time_decode(gen, params, torch, b, args.context, args.steps, args.warmup, vocab)
             points["decode_b%d" % b] = round(b * args.steps / dtb, 1)
+            bytes_b = weight_bytes(cfg, itemsize) + b * mean_ctx * kv_bytes_per_token(cfg, itemsize)
+            points["decode_b%d_hbm_frac" % b] = round(bytes_b / (dtb / args.steps) / HBM_BYTES_PER_S, 4)
             log("decode at batch %d: %.3f ms a step, %.0f tokens/s" % (b, dtb / args.steps * 1e3, b * args.steps / dtb))
+    if not (args.no_points or args.no_workloads) and args.shape == "1b" and args.layers == layers_full:
+        # the family's other two shapes with the workloads named for them, each on an engine of its own
+        del gen, engine
+        import gc
+        gc.collect()
+        torch.cuda.empty_cache()
+        for shape, workload, reps in (("3b", "unequal16", 3), ("8b", "batch64", 2)):
+            rec = time_workload(shape, workload, args.dtype, torch, reps=reps)
+            name = "%s_%s" % (shape, workload)
+            points["decode_" + name] = round(rec["tok_s"], 1)
+            points["decode_%s_ms_per_step" % name] = round(rec["ms_per_step"], 3)
+            points["decode_%s_hbm_frac" % name] = round(rec["hbm_frac"], 4)
+            points["prefill_" + name] = round(rec["prefill_tok_s"], 1)
+            points["prefill_%s_ms" % name] = round(rec["prefill_ms"], 2)
+            points["prefill_%s_frac" % name] = round(rec["prefill_frac"], 4)
 
     out = {
         "metric": "decode tok/s at batch %d, context %d (%s)" % (args.batch, args.context, NAMES[args.shape]),
@@ -278,6 +398,7 @@ def main() -> int:
         },
         "prefill": {"value": round(args.prefill / pre_s, 1), "tokens": args.prefill,
                     "ms": round(pre_s * 1e3, 3), "frac": round(pf / pre_s / DENSE_FLOPS[short], 4),
+                    "statistic": "median of 11 runs", "ms_min": round(pre_min * 1e3, 3),
                     "peak_measured": round(flops_measured / 1e12, 1), "unit_measured": "TFLOP/s",
                     "frac_measured": round(pf / pre_s / flops_measured, 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_BYTES_PER_S / 1e9,

@@ -3,11 +3,11 @@
 * A *slot* is the identity of a live sequence: its length, one row of each group's page table and
   one row of each state tensor.  Slots are taken when a request starts and given back when it
   ends; a slot that is taken again starts at length 0 with zeroed state.
-* A *group* collects the cache entries whose mixers keep the same kind of keys and values (all
-  positions, or a window of them, with given head count and size).  Each group has page pools of
-  its own: ``k`` of shape ``[entries, pages + 1, kv_heads, ceil(head_dim / 16), page, 16]``
-  (blocks of 16 dims), ``v`` of shape ``[entries, pages + 1, kv_heads, 2, head_dim, page / 2]``
-  (halves of 32 positions; ``layout.py`` says why) and a table
+* A *group* collects the cache entries whose mixers keep the same things per token (the same
+  planes, for all positions or for a window of them).  Each group has storage of its own: for
+  every plane that the mixers asked for a tensor ``[entries, pages + 1, *page_shape]``, whose
+  page shape is the mixer's business (attention keeps a plane of keys and one of values in the
+  layouts its kernels read; another mixer may keep one latent row a token), and a table
   ``[slots + 1, pages_per_sequence]`` from (slot, position // page) to a page.  The last page and
   the last slot are a sink for padding rows and belong to nobody.
 * Per-sequence *state* of fixed size: for each cache entry whose mixer asks for it, a tensor
@@ -22,8 +22,7 @@ import numpy as np
 import torch
 
 from ..errors import CacheError
-from ..parts.base import CacheNeed, KVView, StateNeed
-from .layout import key_pages_shape, value_pages_shape
+from ..parts.base import CacheNeed, CacheView, StateNeed
 from .pages import PagePool, SlotTable
 
 PAGE = 64
@@ -52,19 +51,22 @@ class CacheGroup:
         self.n_pages = n_pages
         self.sink_page = n_pages
         self.pages_per_seq = pages_per_seq
-        # keys in blocks of 16 dims, values in halves of 32 positions: see layout.py
-        self.k = torch.zeros((len(entries),) + key_pages_shape(n_pages + 1, need.n_kv_heads, need.head_dim),
-                             dtype=dtype, device=device)
-        self.v = torch.zeros((len(entries),) + value_pages_shape(n_pages + 1, need.n_kv_heads, need.head_dim),
-                             dtype=dtype, device=device)
+        self.planes = {}
+        for plane in need.planes:
+            if plane.name in self.planes:
+                raise CacheError("a mixer names the plane %r twice" % plane.name)
+            if any(int(n) <= 0 for n in plane.page_shape):
+                raise CacheError("plane %r has the page shape %s" % (plane.name, tuple(plane.page_shape)))
+            self.planes[plane.name] = torch.zeros((len(entries), n_pages + 1) + tuple(plane.page_shape),
+                                                  dtype=plane.dtype or dtype, device=device)
         self.table_host = np.full((n_slots + 1, pages_per_seq), self.sink_page, dtype=np.int32)
         self.table = torch.from_numpy(self.table_host.copy()).to(device)
         self.held: Dict[int, Dict[int, int]] = {}      # slot -> {page index in sequence: page}
         self.dirty = set()
 
-    def view(self, entry: int) -> KVView:
+    def view(self, entry: int) -> CacheView:
         i = self.index_of[entry]
-        return KVView(self.k[i], self.v[i], self.table, PAGE, self.need)
+        return CacheView({name: t[i] for name, t in self.planes.items()}, self.table, PAGE, self.need)
 
     def first_needed(self, length_after: int) -> int:
         """Index of the first page a sequence still needs once it holds ``length_after`` tokens:
@@ -225,7 +227,7 @@ class SequenceCache:
             g.flush()
 
     # ---- views for a step
-    def kv_view(self, entry: int) -> Optional[KVView]:
+    def kv_view(self, entry: int) -> Optional[CacheView]:
         g = self.group_of.get(entry)
         return None if g is None else g.view(entry)
 

@@ -36,10 +36,15 @@ class ScheduleEntry:
 
 @dataclass
 class EmbeddingSpec:
+    """The input layer.  ``kind`` names the registered class that turns a step's tokens into the
+    residual stream ("lookup": a row of the table a token, times ``scale``); one that adds learned
+    positions or normalises the rows is another kind with a record of its own that extends this
+    one."""
     vocab: int
     width: int
     tensor: str                         # tensor name of the table
     scale: float = 1.0
+    kind: str = "lookup"
 
 
 @dataclass

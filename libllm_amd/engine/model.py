@@ -10,8 +10,8 @@ import torch
 
 from ..config.spec import ModelSpec, validate_schedule
 from ..errors import ConfigError
-from ..parts import (Stream, StepContext, WeightDecl, build_block, build_feed_forward, build_head,
-                     build_mixer, build_norm)
+from ..parts import (Stream, StepContext, WeightDecl, build_block, build_embedding, build_feed_forward,
+                     build_head, build_mixer, build_norm)
 
 
 def _build_layers(spec: ModelSpec):
@@ -41,10 +41,10 @@ class DecoderModel:
     def __init__(self, spec: ModelSpec):
         validate_schedule(spec)
         self.spec = spec
+        self.embedding = build_embedding(spec.embedding)
         self.blocks = _build_layers(spec)
         self.final_norm = build_norm(spec.final_norm)
         self.head = build_head(spec.head)
-        self.embed_table: Optional[torch.Tensor] = None
         self._decls = None
 
     # ---- weights
@@ -52,9 +52,15 @@ class DecoderModel:
         if self._decls is None:
             s = self.spec
             d = {}
-            d[s.embedding.tensor] = (None, "embedding", WeightDecl((s.embedding.vocab, s.embedding.width)))
+            for name, decl in self.embedding.weights().items():      # an input layer names its tensors in full
+                d[name] = (self.embedding, name, decl)
             if not s.head.tied:
+                if s.head.tensor in d:
+                    raise ConfigError("tensor %r is declared by two parts" % s.head.tensor)
                 d[s.head.tensor] = (None, "head", WeightDecl((s.head.vocab, s.head.width)))
+            elif s.head.tensor not in d or tuple(d[s.head.tensor][2].shape) != (s.head.vocab, s.head.width):
+                raise ConfigError("the output layer is tied to %r, which the input layer does not declare as a "
+                                  "[%d, %d] matrix" % (s.head.tensor, s.head.vocab, s.head.width))
             for block, ls in zip(self.blocks, s.layers):
                 for name, item in _layer_decls(block, ls).items():
                     if name in d:
@@ -83,15 +89,17 @@ class DecoderModel:
             for part in [block.mixer, block.feed_forward] + list(block.norms):
                 if id(part) not in parts:
                     part.bind({}, ops, dtype)
-        self.embed_table = tensors[s.embedding.tensor]
-        self.head.bind(self.embed_table if s.head.tied else tensors[s.head.tensor], ops, dtype)
+        if id(self.embedding) not in parts:
+            self.embedding.bind({}, ops, dtype)
+        self.head.bind(tensors[s.head.tensor], ops, dtype)      # the input layer's table, if tied
 
     # ---- what the cache has to hold
-    def cache_needs(self):
+    def cache_needs(self, page: int):
+        """What every cache entry keeps per token, for a cache whose pages hold ``page`` positions."""
         needs = [None] * self.spec.n_cache_entries()
         for e in self.spec.schedule:
             if e.writes:
-                needs[e.cache] = self.blocks[e.layer].mixer.cache_need()
+                needs[e.cache] = self.blocks[e.layer].mixer.cache_need(page)
         return needs
 
     def state_needs(self):
@@ -113,7 +121,7 @@ class DecoderModel:
         """Whether a unit reads nothing from the host while it runs (so it can be captured)."""
         n = len(self.spec.schedule)
         if unit == 0:
-            return True
+            return getattr(self.embedding, "graph_safe", False)
         if unit == n + 1:
             return getattr(self.final_norm, "graph_safe", False) and getattr(self.head, "graph_safe", False)
         block = self.blocks[self.spec.schedule[unit - 1].layer]
@@ -138,17 +146,10 @@ class DecoderModel:
         s = self.spec
         n = len(s.schedule)
         if unit == 0:
-            # if a plain RMS norm reads the rows first, the embedding kernel may prepare it
+            # if a plain RMS norm reads the rows first, the input layer may prepare it
             first = self.blocks[s.schedule[0].layer].entry_norm() if n else self.final_norm
             terms = first.rms_terms() if first is not None and (n or ctx.want_all_rows) else None
-            if terms is not None and hasattr(ctx.ops, "embed_prepared"):
-                got = ctx.ops.embed_prepared(self.embed_table, ctx.tokens, s.embedding.scale, terms[0], terms[1],
-                                             ctx.dtype)
-                if got is not None:
-                    stream = Stream(got[0])
-                    stream.pre = got[1]
-                    return stream
-            return Stream(ctx.ops.embed(self.embed_table, ctx.tokens, s.embedding.scale))
+            return self.embedding.forward(ctx, terms)
         if unit == n + 1:
             ctx.norm_after_block = None
             if want_rows is None or want_rows.numel() == 0:

@@ -52,7 +52,7 @@ class Engine:
         self.dtype = dtype
         self.device = ops.device
         self.vocab = model.spec.vocab
-        self.cache = SequenceCache(model.cache_needs(), model.state_needs(), max_tokens,
+        self.cache = SequenceCache(model.cache_needs(PAGE), model.state_needs(), max_tokens,
                                    model.spec.max_position, dtype, self.device, max_slots)
         # a part that reads the step's host-side data cannot be captured; the stretches of the
         # schedule around it still are (see _CapturedForward)

@@ -14,7 +14,7 @@ from typing import List, Optional
 import numpy as np
 import torch
 
-from ..cache.layout import key_pages_shape, value_pages_shape
+from ..parts.kv_pages import K_LAYOUT, V_LAYOUT, key_pages_shape, value_pages_shape
 from ..errors import KernelError
 from . import build
 
@@ -623,7 +623,7 @@ class HipOps:
             raise KernelError("qkv_rope: the weight is %s, expected %s" % (tuple(w.shape), (n, k)))
         fused = (dtype == torch.bfloat16 and (adjacent or rot_dim == 0) and hd % 16 == 0
                  and m <= self.SKINNY_ROWS and m == ctx.n_tokens
-                 and (not write or (kv is not None and kv.k_pages.dtype == torch.bfloat16)))
+                 and (not write or (kv is not None and "k" in kv.planes and kv.planes["k"].dtype == torch.bfloat16)))
         pre = x.pre if lazy and fused and self._skinny_ok(x, w, m, k) else None
         if pre is not None:
             x, lazy = pre.raw, False             # rows that lack their norm's scale: see Prenormed
@@ -647,8 +647,8 @@ class HipOps:
             kptr = vptr = tptr = None
             stride = 0
             if write:
-                self._check_kv(kv, n_kv, hd, torch.bfloat16)
-                kptr, vptr, tptr = kv.k_pages.data_ptr(), kv.v_pages.data_ptr(), kv.block_table.data_ptr()
+                k_pages, v_pages = self._kv_planes(kv, n_kv, hd, torch.bfloat16)
+                kptr, vptr, tptr = k_pages.data_ptr(), v_pages.data_ptr(), kv.block_table.data_ptr()
                 stride = kv.block_table.shape[1]
             xp = self._dev(x, "qkv input", torch.bfloat16)
             q = torch.empty((m, n_heads * hd), dtype=torch.bfloat16, device=self.device)
@@ -689,28 +689,41 @@ class HipOps:
         kptr = vptr = tptr = None
         stride = 0
         if write:
-            self._check_kv(kv, n_kv, hd, qkv.dtype)
-            kptr, vptr, tptr = kv.k_pages.data_ptr(), kv.v_pages.data_ptr(), kv.block_table.data_ptr()
+            k_pages, v_pages = self._kv_planes(kv, n_kv, hd, qkv.dtype)
+            kptr, vptr, tptr = k_pages.data_ptr(), v_pages.data_ptr(), kv.block_table.data_ptr()
             stride = kv.block_table.shape[1]
         self._check(self.lib.llm_rope_kv_write(
             qkv.data_ptr(), _code(qkv.dtype), width, bptr, n_heads, n_kv, hd, cptr, sptr, rot_dim,
             ctx.tok_pos.data_ptr(), ctx.tok_seq.data_ptr(), ctx.seq_slot.data_ptr(), tptr, stride,
             kptr, vptr, 64, 1 if write else 0, 1 if adjacent else 0, m, self._stream()), "rope_kv_write")
 
-    def _check_kv(self, kv, n_kv, hd, dtype):
+    def _kv_planes(self, kv, n_kv, hd, dtype):
+        """The planes of keys and values that the attention kernels read and write, checked: the
+        cache entry holds planes "k" and "v" in the layouts of ``parts/kv_pages.py``, for these
+        head counts and sizes, in the activations' dtype, with a page table beside them."""
         if kv is None:
             raise KernelError("this layer has no cache entry")
-        shape = tuple(kv.k_pages.shape)
-        vshape = tuple(kv.v_pages.shape)
+        for name, layout in (("k", K_LAYOUT), ("v", V_LAYOUT)):
+            plane = kv.need.plane(name) if kv.need is not None else None
+            if name not in kv.planes or plane is None:
+                raise KernelError("attention needs a cache entry with planes \"k\" and \"v\"; this one has: %s"
+                                  % (", ".join(sorted(kv.planes)) or "none"))
+            if plane.layout != layout:
+                raise KernelError("plane %r is laid out as %r, the attention kernels read %r" % (name, plane.layout, layout))
+        if kv.page_size != 64:
+            raise KernelError("the attention kernels read pages of 64 positions, not %d" % kv.page_size)
+        k_pages, v_pages = kv.planes["k"], kv.planes["v"]
+        shape, vshape = tuple(k_pages.shape), tuple(v_pages.shape)
         want = key_pages_shape(shape[0] if shape else 0, n_kv, hd)
         vwant = value_pages_shape(shape[0] if shape else 0, n_kv, hd)
         if shape != want or vshape != vwant:
             raise KernelError("cache pages have shapes %s / %s, expected %s and %s" % (shape, vshape, want, vwant))
-        if kv.k_pages.dtype != dtype or kv.v_pages.dtype != dtype:
-            raise KernelError("cache dtype %s differs from the activations' %s" % (kv.k_pages.dtype, dtype))
-        self._dev(kv.k_pages, "key pages")
-        self._dev(kv.v_pages, "value pages")
+        if k_pages.dtype != dtype or v_pages.dtype != dtype:
+            raise KernelError("cache dtype %s differs from the activations' %s" % (k_pages.dtype, dtype))
+        self._dev(k_pages, "key pages")
+        self._dev(v_pages, "value pages")
         self._dev(kv.block_table, "page table", torch.int32)
+        return k_pages, v_pages
 
     def attention(self, qkv, n_heads, n_kv, hd, ctx, kv, scale, window):
         m, width = qkv.shape
@@ -720,7 +733,7 @@ class HipOps:
             raise KernelError("attention: %d heads are not a multiple of %d kv heads" % (n_heads, n_kv))
         if hd > 256:
             raise KernelError("attention: head_dim %d above 256 is not supported" % hd)
-        self._check_kv(kv, n_kv, hd, qkv.dtype)
+        k_pages, v_pages = self._kv_planes(kv, n_kv, hd, qkv.dtype)
         out = torch.empty((m, n_heads * hd), dtype=qkv.dtype, device=self.device)
         table = kv.block_table
         if (self.fast_attention and qkv.dtype == torch.bfloat16 and width % 8 == 0
@@ -746,7 +759,7 @@ class HipOps:
                 part_o = torch.empty((m, n_heads, n_blocks, hd), dtype=torch.float32, device=self.device)
                 part_ml = torch.empty((m, n_heads, n_blocks, 2), dtype=torch.float32, device=self.device)
                 self._check(self.lib.llm_attention_decode_bf16(
-                    qkv.data_ptr(), width, kv.k_pages.data_ptr(), kv.v_pages.data_ptr(),
+                    qkv.data_ptr(), width, k_pages.data_ptr(), v_pages.data_ptr(),
                     table.data_ptr(), table.shape[1], 64, ctx.seq_slot.data_ptr(),
                     ctx.seq_pos0.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), m, n_heads, n_kv, hd, float(scale),
                     int(window), n_blocks, self._stream()), "attention_decode_bf16")
@@ -755,14 +768,14 @@ class HipOps:
                 if not tiles:
                     tiles = 2 if hd <= 128 and ctx.max_new >= self.PROMPT_TILE_ROWS[0 if hd <= 64 else 1] else 1
                 self._check(self.lib.llm_attention_prefill_bf16(
-                    qkv.data_ptr(), width, kv.k_pages.data_ptr(), kv.v_pages.data_ptr(),
+                    qkv.data_ptr(), width, k_pages.data_ptr(), v_pages.data_ptr(),
                     table.data_ptr(), table.shape[1], 64, ctx.seq_start.data_ptr(),
                     ctx.seq_slot.data_ptr(), ctx.seq_pos0.data_ptr(), out.data_ptr(), ctx.n_seqs,
                     ctx.max_new, n_heads, n_kv, hd, float(scale), int(window), tiles, self._stream()),
                     "attention_prefill_bf16")
             return out
         self._check(self.lib.llm_attention_ref(
-            qkv.data_ptr(), _code(qkv.dtype), width, kv.k_pages.data_ptr(), kv.v_pages.data_ptr(),
+            qkv.data_ptr(), _code(qkv.dtype), width, k_pages.data_ptr(), v_pages.data_ptr(),
             kv.block_table.data_ptr(), kv.block_table.shape[1], 64, ctx.tok_pos.data_ptr(),
             ctx.tok_seq.data_ptr(), ctx.seq_slot.data_ptr(), out.data_ptr(), m, n_heads, n_kv, hd,
             float(scale), int(window), self._stream()), "attention")

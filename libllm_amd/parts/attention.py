@@ -12,7 +12,8 @@ from typing import Optional
 import torch
 
 from ..errors import ConfigError
-from .base import PartSpec, CacheNeed, Mixer, StepContext, WeightDecl
+from .base import PartSpec, Mixer, StepContext, WeightDecl
+from .kv_pages import kv_need
 from .linear import Linear
 from .registry import build_position, register_mixer
 
@@ -62,9 +63,9 @@ class Attention(Mixer):
         self.bias = None
         self.adjacent = False
 
-    def cache_need(self):
+    def cache_need(self, page):
         s = self.spec
-        return CacheNeed("window" if s.window else "full", s.n_kv_heads, s.head_dim, s.window)
+        return kv_need(s.n_kv_heads, s.head_dim, s.window, page)
 
     def weights(self):
         s = self.spec

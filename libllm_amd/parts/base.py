@@ -32,18 +32,39 @@ class WeightDecl:
     init: str = "normal"
 
 
+@dataclass(frozen=True)
+class Plane:
+    """One array that a mixer keeps per cached token: keys, values, a latent row, whatever its
+    kernels read back.  The cache allocates ``[pages + 1, *page_shape]`` for it per cache entry
+    and never looks inside a page: ``page_shape`` is the shape of one page (the cache's page size
+    in positions, arranged as the mixer's kernels want them), ``layout`` a name for that
+    arrangement, which whoever reads or writes the plane checks, and ``dtype`` the element type
+    (None: the dtype of the activations)."""
+    name: str
+    page_shape: Tuple[int, ...]
+    layout: str = "rows"
+    dtype: Optional[torch.dtype] = None
+
+
+def rows_plane(name: str, per_token: Tuple[int, ...], page: int, dtype=None) -> Plane:
+    """The plain arrangement: a page is ``[page, *per_token]``, position after position."""
+    return Plane(name, (page,) + tuple(per_token), "rows", dtype)
+
+
 @dataclass
 class CacheNeed:
-    """Keys and values a mixer keeps per token.  ``kind`` "full" keeps every position;
-    "window" needs only the last ``window`` positions.  Layers with equal needs share a group
-    of the cache, and each group has storage of its own."""
+    """What a mixer keeps per token: its planes, and which positions.  ``kind`` "full" keeps
+    every position; "window" needs only the last ``window`` positions.  Cache entries with equal
+    needs share a group of the cache, and each group has storage of its own."""
     kind: str
-    n_kv_heads: int
-    head_dim: int
+    planes: Tuple[Plane, ...]
     window: int = 0
 
     def key(self):
-        return (self.kind, self.n_kv_heads, self.head_dim, self.window)
+        return (self.kind, tuple(self.planes), self.window)
+
+    def plane(self, name: str) -> Optional[Plane]:
+        return next((p for p in self.planes if p.name == name), None)
 
 
 @dataclass
@@ -53,18 +74,20 @@ class StateNeed:
     dtype: torch.dtype = torch.float32
 
 
-class KVView:
-    """The keys and values of one cache entry: key pages ``[pages, kv_heads, ceil(head_dim / 16),
-    page, 16]`` (blocks of 16 dims), value pages ``[pages, kv_heads, 2, head_dim, page / 2]``
-    (halves of 32 positions; ``cache/layout.py`` says why), and the table that maps
-    (slot, position // page) to a page."""
+class CacheView:
+    """One cache entry as a mixer sees it: its planes by name, each ``[pages, *page_shape]``, and
+    the table that maps (slot, position // page_size) to a page."""
 
-    def __init__(self, k_pages, v_pages, block_table, page_size, need):
-        self.k_pages = k_pages
-        self.v_pages = v_pages
+    def __init__(self, planes: Dict[str, torch.Tensor], block_table, page_size, need: CacheNeed):
+        self.planes = dict(planes)
         self.block_table = block_table
         self.page_size = page_size
         self.need = need
+
+    def plane(self, name: str) -> torch.Tensor:
+        if name not in self.planes:
+            raise KeyError("this cache entry has no plane %r (it has: %s)" % (name, ", ".join(sorted(self.planes)) or "none"))
+        return self.planes[name]
 
 
 class Stream:
@@ -128,10 +151,10 @@ class StepContext:
         self.norm_after_block = None   # the norm that reads the stream first after the running block, if known
         self.captured = False      # the step runs over the fixed buffers of a captured shape (see above)
         self.want_all_rows = False  # the logits of every row are wanted, in order (a decode step): the last norm gathers nothing
-        self._kv: Dict[int, KVView] = {}
+        self._kv: Dict[int, CacheView] = {}
         self._state: Dict[int, torch.Tensor] = {}
 
-    def kv(self, cache_entry: int) -> Optional[KVView]:
+    def kv(self, cache_entry: int) -> Optional[CacheView]:
         return self._kv.get(cache_entry)
 
     def state(self, cache_entry: int) -> Optional[torch.Tensor]:
@@ -150,12 +173,27 @@ class Part:
         pass
 
 
+class Embedding(Part):
+    """The input layer: makes the residual stream of a step from its tokens.
+
+    ``weights()`` names its tensors in full (an input layer has no prefix); ``forward(ctx,
+    then_norm)`` returns a ``Stream`` whose ``res`` is the float32 matrix ``[tokens, width]``.
+    ``then_norm`` = (weight, eps) says that a plain RMS norm with these reads the rows first; an
+    input layer may prepare it in the same kernel (``Stream.pre``) or ignore the hint.  It reads
+    ``ctx.tokens`` and, if it wants, ``ctx.tok_pos`` (learned positions); ``graph_safe`` as for
+    the other parts."""
+    graph_safe = False
+
+    def forward(self, ctx: "StepContext", then_norm=None) -> "Stream":
+        raise NotImplementedError
+
+
 class Mixer(Part):
     """Mixes information between the tokens of a sequence (attention, a recurrence, ...).
 
     ``forward(ctx, x, entry)`` takes the normalised rows ``[M, width]`` in the activation dtype
     and returns rows of the same shape.  ``entry`` is the schedule entry of this run; the mixer
-    reads its keys/values through ``ctx.kv(entry.cache)`` and its state through
+    reads what it keeps per token through ``ctx.kv(entry.cache)`` (a ``CacheView``) and its state through
     ``ctx.state(entry.cache)``, and writes them only if ``entry.writes``.
 
     Two optional abilities, off unless the class sets them (they apply to feed-forwards too):
@@ -168,7 +206,8 @@ class Mixer(Part):
     takes_normed = False
     adds_to_stream = False
 
-    def cache_need(self) -> Optional[CacheNeed]:
+    def cache_need(self, page: int) -> Optional[CacheNeed]:
+        """What the mixer keeps per token, for a cache whose pages hold ``page`` positions."""
         return None
 
     def state_need(self) -> Optional[StateNeed]:

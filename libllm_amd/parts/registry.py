@@ -17,6 +17,7 @@ _NORMS: Dict[str, Callable] = {}
 _POSITIONS: Dict[str, Callable] = {}
 _BLOCKS: Dict[str, Callable] = {}
 _HEADS: Dict[str, Callable] = {}
+_EMBEDDINGS: Dict[str, Callable] = {}
 
 
 def _register(table, what):
@@ -44,6 +45,7 @@ register_norm = _register(_NORMS, "norm")
 register_position = _register(_POSITIONS, "position encoding")
 register_block = _register(_BLOCKS, "block")
 register_head = _register(_HEADS, "output layer")
+register_embedding = _register(_EMBEDDINGS, "input layer")
 
 build_mixer = _build(_MIXERS, "mixer")
 build_feed_forward = _build(_FEED_FORWARDS, "feed-forward")
@@ -51,3 +53,4 @@ build_norm = _build(_NORMS, "norm")
 build_position = _build(_POSITIONS, "position encoding")
 build_block = _build(_BLOCKS, "block")
 build_head = _build(_HEADS, "output layer")
+build_embedding = _build(_EMBEDDINGS, "input layer")

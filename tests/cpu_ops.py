@@ -5,7 +5,7 @@ same method signatures as ``libllm_amd.hip.ops.HipOps``; the library itself neve
 import numpy as np
 import torch
 
-from libllm_amd.cache import layout
+from libllm_amd.parts import kv_pages as layout
 
 
 class CpuOps:
@@ -65,8 +65,8 @@ class CpuOps:
             slots = ctx.seq_slot.long()[ctx.tok_seq.long()]
             pos = ctx.tok_pos.long()
             pages = kv.block_table.long()[slots, pos // kv.page_size]
-            layout.write_keys(kv.k_pages, pages, pos % kv.page_size, k.to(kv.k_pages.dtype))
-            layout.write_values(kv.v_pages, pages, pos % kv.page_size, v.to(kv.v_pages.dtype))
+            layout.write_keys(kv.plane("k"), pages, pos % kv.page_size, k.to(kv.plane("k").dtype))
+            layout.write_values(kv.plane("v"), pages, pos % kv.page_size, v.to(kv.plane("v").dtype))
 
     def attention(self, qkv, n_heads, n_kv, hd, ctx, kv, scale, window):
         m = qkv.shape[0]
@@ -79,8 +79,8 @@ class CpuOps:
             first = max(0, pos - window + 1) if window else 0
             keys = torch.arange(first, pos + 1)
             pages = kv.block_table[slot].long()[keys // page]
-            k = layout.read_keys(kv.k_pages, pages, keys % page, hd).float()       # [L, n_kv, hd]
-            v = layout.read_values(kv.v_pages, pages, keys % page).float()
+            k = layout.read_keys(kv.plane("k"), pages, keys % page, hd).float()       # [L, n_kv, hd]
+            v = layout.read_values(kv.plane("v"), pages, keys % page).float()
             q = qkv[t, :n_heads * hd].float().reshape(n_heads, hd)
             k = k.repeat_interleave(group, dim=1)
             v = v.repeat_interleave(group, dim=1)

@@ -2,8 +2,8 @@
 import numpy as np
 import torch
 
-from libllm_amd.cache import layout
-from libllm_amd.parts import CacheNeed, KVView, StepContext
+from libllm_amd.parts import CacheView, StepContext
+from libllm_amd.parts import kv_pages as layout
 
 PAGE = 64
 
@@ -122,28 +122,30 @@ def make_kv(device, dtype, n_slots, pages_per_seq, n_kv, hd, seed=0, window=0):
     g = torch.Generator().manual_seed(seed)
     n_pages = n_slots * pages_per_seq
     perm = torch.randperm(n_pages, generator=g).reshape(n_slots, pages_per_seq).to(torch.int32)
-    k = torch.zeros(layout.key_pages_shape(n_pages + 1, n_kv, hd), dtype=dtype, device=device)
-    v = torch.zeros(layout.value_pages_shape(n_pages + 1, n_kv, hd), dtype=dtype, device=device)
-    need = CacheNeed("window" if window else "full", n_kv, hd, window)
-    return KVView(k, v, perm.to(device), PAGE, need)
+    need = layout.kv_need(n_kv, hd, window, PAGE)
+    planes = {p.name: torch.zeros((n_pages + 1,) + p.page_shape, dtype=dtype, device=device) for p in need.planes}
+    return CacheView(planes, perm.to(device), PAGE, need)
 
 
 def fill_kv(kv, slot, keys, values):
     """keys, values: [L, n_kv, hd] (any float dtype) written at positions 0..L-1 of the slot."""
+    k_pages, v_pages = kv.plane("k"), kv.plane("v")
     length = keys.shape[0]
     pos = torch.arange(length)
-    pages = kv.block_table[slot].cpu().long()[pos // PAGE].to(kv.k_pages.device)
-    off = (pos % PAGE).to(kv.k_pages.device)
-    layout.write_keys(kv.k_pages, pages, off, keys.to(kv.k_pages.device, kv.k_pages.dtype))
-    layout.write_values(kv.v_pages, pages, off, values.to(kv.v_pages.device, kv.v_pages.dtype))
+    pages = kv.block_table[slot].cpu().long()[pos // PAGE].to(k_pages.device)
+    off = (pos % PAGE).to(k_pages.device)
+    layout.write_keys(k_pages, pages, off, keys.to(k_pages.device, k_pages.dtype))
+    layout.write_values(v_pages, pages, off, values.to(v_pages.device, v_pages.dtype))
 
 
 def read_kv(kv, slot, length):
+    k_pages, v_pages = kv.plane("k"), kv.plane("v")
     pos = torch.arange(length)
-    pages = kv.block_table[slot].cpu().long()[pos // PAGE].to(kv.k_pages.device)
-    off = (pos % PAGE).to(kv.k_pages.device)
-    return (layout.read_keys(kv.k_pages, pages, off, kv.need.head_dim).float().cpu(),
-            layout.read_values(kv.v_pages, pages, off).float().cpu())
+    pages = kv.block_table[slot].cpu().long()[pos // PAGE].to(k_pages.device)
+    off = (pos % PAGE).to(k_pages.device)
+    head_dim = v_pages.shape[-2]
+    return (layout.read_keys(k_pages, pages, off, head_dim).float().cpu(),
+            layout.read_values(v_pages, pages, off).float().cpu())
 
 
 def attention_oracle(q, keys, values, pos, scale, window=0):

@@ -7,7 +7,8 @@ import torch
 
 from libllm_amd import CacheError
 from libllm_amd.cache import PAGE, PagePool, SequenceCache, SlotTable, pages_for
-from libllm_amd.parts import CacheNeed, StateNeed
+from libllm_amd.parts import CacheNeed, Plane, StateNeed, rows_plane
+from libllm_amd.parts.kv_pages import kv_need
 
 
 def test_page_pool():
@@ -45,14 +46,27 @@ def test_slot_table():
 
 def test_random_traffic_keeps_the_books():
     rnd = random.Random(1)
-    needs = [CacheNeed("full", 2, 16), CacheNeed("full", 2, 16), CacheNeed("window", 1, 32, 100), None]
-    states = [None, StateNeed((3,)), None, StateNeed((2, 2))]
+    # two attention layers of one shape, one with a window and another shape, a mixer that keeps
+    # one latent row a token in a type of its own, and a layer that caches nothing
+    latent = CacheNeed("full", (rows_plane("z", (5,), PAGE, torch.float64),))
+    needs = [kv_need(2, 16, 0, PAGE), kv_need(2, 16, 0, PAGE), kv_need(1, 32, 100, PAGE), latent, None]
+    states = [None, StateNeed((3,)), None, StateNeed((2, 2)), None]
     cache = SequenceCache(needs, states, max_tokens=64 * 12, max_position=640, dtype=torch.float32, device="cpu")
-    assert len(cache.groups) == 2 and cache.groups[0].entries == [0, 1] and cache.groups[1].entries == [2]
-    # keys in blocks of 16 dims, values in halves of 32 positions (cache/layout.py)
-    assert cache.groups[0].k.shape == (2, 13, 2, 1, PAGE, 16) and cache.groups[0].v.shape == (2, 13, 2, 2, 16, 32)
-    assert cache.groups[1].k.shape == (1, 13, 1, 2, PAGE, 16) and cache.groups[1].v.shape == (1, 13, 1, 2, 32, 32)
+    assert [g.entries for g in cache.groups] == [[0, 1], [2], [3]]
+    # keys in blocks of 16 dims, values in halves of 32 positions (parts/kv_pages.py)
+    g0, g1, g2 = cache.groups
+    assert g0.planes["k"].shape == (2, 13, 2, 1, PAGE, 16) and g0.planes["v"].shape == (2, 13, 2, 2, 16, 32)
+    assert g1.planes["k"].shape == (1, 13, 1, 2, PAGE, 16) and g1.planes["v"].shape == (1, 13, 1, 2, 32, 32)
+    assert list(g2.planes) == ["z"] and g2.planes["z"].shape == (1, 13, PAGE, 5) and g2.planes["z"].dtype == torch.float64
+    view = cache.kv_view(3)
+    assert view.plane("z").shape == (13, PAGE, 5) and view.need.plane("z").layout == "rows" and view.need.plane("k") is None
+    with pytest.raises(KeyError, match="no plane 'k'"):
+        view.plane("k")
+    assert cache.kv_view(4) is None
     assert cache.state[1].shape == (13, 3) and cache.state[3].shape == (13, 2, 2) and 0 not in cache.state
+    with pytest.raises(CacheError, match="twice"):
+        SequenceCache([CacheNeed("full", (Plane("a", (PAGE, 2)), Plane("a", (PAGE, 3))))], [None], max_tokens=64,
+                      max_position=64, dtype=torch.float32, device="cpu")
     live = {}
     for step in range(400):
         op = rnd.random()
@@ -78,10 +92,10 @@ def test_random_traffic_keeps_the_books():
             cache.release(rid)
             del live[rid]
         cache.check()
-        full, win = cache.groups
+        full, win, lat = cache.groups
         for rid, slot in live.items():
             n = cache.length(slot)
-            assert sorted(full.held.get(slot, {})) == list(range(pages_for(n)))
+            assert sorted(full.held.get(slot, {})) == list(range(pages_for(n))) == sorted(lat.held.get(slot, {}))
             if n:
                 first = max(0, n + 1 - 100) // PAGE       # pages wholly behind the window are given back
                 assert sorted(win.held.get(slot, {})) == list(range(first, pages_for(n)))
@@ -92,7 +106,7 @@ def test_random_traffic_keeps_the_books():
 
 
 def test_reused_slot_starts_clean_and_tables_follow():
-    cache = SequenceCache([CacheNeed("full", 1, 16)], [StateNeed((4,))], max_tokens=256, max_position=256,
+    cache = SequenceCache([kv_need(1, 16, 0, PAGE)], [StateNeed((4,))], max_tokens=256, max_position=256,
                           dtype=torch.float32, device="cpu")
     s = cache.admit("a")
     cache.reserve(s, 100)
@@ -121,7 +135,7 @@ def test_reused_slot_starts_clean_and_tables_follow():
 def test_page_layout_round_trip():
     """Keys and values written through the layout's helpers come back; a head size that is no
     multiple of 16 pads its last block of dims; the flat offsets are the kernels' formulas."""
-    from libllm_amd.cache import layout
+    from libllm_amd.parts import kv_pages as layout
     for hd in (16, 24, 64, 80):
         k = torch.zeros(layout.key_pages_shape(3, 2, hd))
         v = torch.zeros(layout.value_pages_shape(3, 2, hd))

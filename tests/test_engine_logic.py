@@ -133,7 +133,7 @@ def test_layers_may_differ_and_groups_get_storage_of_their_own():
     spec.layers[1].mixer.window = 70                                 # and a window
     spec.layers[1].feed_forward.intermediate = 96
     engine, _ = build(spec, 6, CpuOps(), max_tokens=256)
-    kinds = [(g.need.kind, g.need.n_kv_heads, g.need.window, g.entries) for g in engine.cache.groups]
+    kinds = [(g.need.kind, g.planes["k"].shape[2], g.need.window, g.entries) for g in engine.cache.groups]
     assert kinds == [("full", 2, 0, [0]), ("window", 4, 70, [1])]
     ids = np.random.default_rng(4).integers(0, 256, size=128).tolist()
     whole = engine.step([StepEntry("a", ids, list(range(128)))])
@@ -168,6 +168,35 @@ def test_toy_mixer_with_state_of_its_own():
     for rid, toks in (("a", reqs["a"]), ("b", reqs["b"]), ("c", reqs["b"])):   # c reuses a slot: clean state
         ref = toy.toy_oracle(cfg, w, w["model.layers.1.toy.mix.weight"], toks)
         assert err(np.stack(got[rid]), ref) < 1e-4
+
+
+def test_toy_mixer_with_a_plane_of_its_own_and_toy_input_layer():
+    """A mixer that keeps one latent row a token in the cache's pages (no keys and values), and an
+    input layer with learned positions, both defined in tests/toy.py: batches of unequal prompts
+    cut in two ways, slots and pages used again."""
+    cfg_t = config_from_dict(dict(TINY_A, max_position_embeddings=256))
+    cfg = llama.PlainConfig(cfg_t.to_dict())
+    engine, w = build(toy.planes_spec(cfg_t), 9, CpuOps(), max_tokens=320)
+    g_latent, g_kv = engine.cache.groups
+    assert g_latent.entries == [0] and list(g_latent.planes) == ["z"] and g_latent.planes["z"].dtype == torch.float32
+    assert g_latent.planes["z"].shape == (1, 6, 64, 8) and sorted(g_kv.planes) == ["k", "v"]
+    assert "model.embed_positions.weight" in engine.model.declared()
+    rng = np.random.default_rng(6)
+    reqs = {"a": rng.integers(0, 256, size=150).tolist(), "b": rng.integers(0, 256, size=70).tolist()}
+    steps = traces.batches([reqs, {"c": reqs["b"], "d": reqs["a"][:100]}], {"a": 12, "b": 8, "c": 3, "d": 40})
+    got = {}
+    for s in steps:
+        out = engine.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        row = 0
+        for e in s["entries"]:
+            for _ in e["want"]:
+                got.setdefault(e["id"], []).append(out[row].double().numpy())
+                row += 1
+        engine.end(s["end"])
+        engine.cache.check()
+    for rid, toks in (("a", reqs["a"]), ("b", reqs["b"]), ("c", reqs["b"]), ("d", reqs["a"][:100])):
+        assert err(np.stack(got[rid]), toy.planes_oracle(cfg, w, toks)) < 1e-4
+    assert all(g.pool.n_free == g.pool.n_pages for g in engine.cache.groups)
 
 
 def test_a_dropped_engine_goes_at_once(models):

@@ -363,7 +363,7 @@ def test_products_over_a_prepared_norm(ops, m, width, n):
         for rows in (lazy, hb):
             kv = make_kv("cuda", torch.bfloat16, m, 1, n_kv, hd, seed=1)
             q = ops.qkv_rope(rows, pw, None, n_heads, n_kv, hd, cos, sin, hd, ctx, kv, True, True, torch.bfloat16)
-            outs.append((q[:, :n_heads * hd].clone(), kv.k_pages.clone(), kv.v_pages.clone()))
+            outs.append((q[:, :n_heads * hd].clone(), kv.plane("k").clone(), kv.plane("v").clone()))
         for a, b in zip(*outs):
             assert max_err(a, b) < BF16_2ULP
         assert float(outs[0][1].float().abs().max()) > 0
@@ -762,7 +762,7 @@ def test_projection_with_rotation_and_cache_write(ops, dtype, shape, bias, seqs)
     q_only = ops.qkv_rope(x.cuda().to(dtype), wd[:n_heads * hd].contiguous(), bd, n_heads, n_kv, hd, cos, sin,
                           rot, ctx, kv, False, bool(rot), dtype)
     assert close(q_only[:, :n_heads * hd].reshape(m, n_heads, hd), heads[:, :n_heads][..., head_order], dtype, **tol)
-    assert torch.count_nonzero(kv.k_pages) == 0
+    assert torch.count_nonzero(kv.plane("k")) == 0
 
 
 @pytest.mark.parametrize("shape", [(4, 2, 16, 16), (6, 3, 48, 24), (5, 1, 64, 64), (8, 2, 128, 128), (2, 2, 256, 64),
@@ -804,7 +804,7 @@ def test_rope_kv_write_on_many_rows(ops, shape, bias):
         q = qkv[:, :n_heads * hd].reshape(m, n_heads, hd)
         assert close(q, heads[:, :n_heads][..., head_order], dtype)
         if not write:
-            assert torch.count_nonzero(kv.k_pages) == 0 and torch.count_nonzero(kv.v_pages) == 0
+            assert torch.count_nonzero(kv.plane("k")) == 0 and torch.count_nonzero(kv.plane("v")) == 0
             continue
         o = 0
         for slot, p0, n_new in seqs:
@@ -814,7 +814,7 @@ def test_rope_kv_write_on_many_rows(ops, shape, bias):
             assert torch.count_nonzero(k_got[:p0]) == 0 and torch.count_nonzero(v_got[:p0]) == 0
             o += n_new
         written = sum(n for _, _, n in seqs) * n_kv * hd
-        assert torch.count_nonzero(kv.k_pages) <= written and torch.count_nonzero(kv.v_pages) <= written
+        assert torch.count_nonzero(kv.plane("k")) <= written and torch.count_nonzero(kv.plane("v")) <= written
 
 
 def test_rope_pairing_and_sign(ops):
@@ -946,7 +946,7 @@ def test_prompt_attention_takes_two_tiles_for_long_prompts(ops):
     assert rows >= ops.PROMPT_TILE_ROWS[0]
     ctx = make_ctx(ops, torch.bfloat16, seqs)
     kv = make_kv("cuda", torch.bfloat16, 2, (rows + 64) // PAGE + 1, n_kv, hd, seed=2)
-    kv.k_pages.normal_(); kv.v_pages.normal_()
+    kv.plane("k").normal_(); kv.plane("v").normal_()
     q = rnd((ctx.n_tokens, n_heads * hd), torch.bfloat16, 5).cuda()
     outs = []
     for tiles in (0, 1, 2):

@@ -232,6 +232,73 @@ def test_toy_routed_feed_forward_and_position_encoding(ops, dtype):
     engine.cache.check()
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_mixer_with_a_plane_of_its_own_and_toy_input_layer(ops, dtype):
+    """A mixer that keeps one latent row a token in the cache's pages, in a plane of its own
+    width and element type instead of keys and values, and an input layer with learned positions:
+    both defined in tests/toy.py, chosen in the model's record, and stepped on the GPU (the input
+    layer inside the captured graphs, the mixer from the host between them) against their own
+    restatement.  Batches of unequal prompts, one after another, so that pages are used again."""
+    cfg_t = config_from_dict(dict(TINY_A, max_position_embeddings=256))
+    cfg = llama.PlainConfig(cfg_t.to_dict())
+    model = DecoderModel(toy.planes_spec(cfg_t))
+    t = random_tensors(model.declared(), 9, std=0.1, norm_std=0.2)
+    model.bind({k: v.to("cuda", torch.float32 if (dtype == torch.float32 or v.dim() == 1) else dtype)
+                for k, v in t.items()}, ops, dtype)
+    engine = Engine(model, ops, dtype, max_tokens=320)
+    engine.PROMPT_SEEN = 1
+    assert engine.use_graphs and [(safe, units) for safe, units in model.stretches()] == [
+        (True, [0]), (False, [1]), (True, [2, 3])]
+    g_latent, g_kv = engine.cache.groups
+    assert list(g_latent.planes) == ["z"] and g_latent.planes["z"].shape == (1, 6, 64, 8)
+    assert g_latent.planes["z"].dtype == torch.float32 and sorted(g_kv.planes) == ["k", "v"]
+    w = {k: v.double().numpy() for k, v in t.items()}
+    rng = np.random.default_rng(6)
+    reqs = {"a": rng.integers(0, 256, size=150).tolist(), "b": rng.integers(0, 256, size=70).tolist()}
+    steps = traces.batches([reqs, {"c": reqs["b"], "d": reqs["a"][:100]}], {"a": 12, "b": 8, "c": 3, "d": 40})
+    got = {}
+    for s in steps:
+        out = engine.step([StepEntry(e["id"], e["tokens"], e["want"]) for e in s["entries"]])
+        row = 0
+        for e in s["entries"]:
+            for _ in e["want"]:
+                got.setdefault(e["id"], []).append(out[row].double().cpu().numpy())
+                row += 1
+        engine.end(s["end"])
+        engine.cache.check()
+    for rid, toks in (("a", reqs["a"]), ("b", reqs["b"]), ("c", reqs["b"]), ("d", reqs["a"][:100])):
+        assert_logits_close(np.stack(got[rid]), toy.planes_oracle(cfg, w, toks), dtype, rid)
+    # a prompt of which only the last row is wanted goes through a captured prompt step
+    e = rng.integers(0, 256, size=90).tolist()
+    rows = [engine.step([StepEntry("e", e[:80], [79])]).double().cpu().numpy()]
+    rows += [engine.step([StepEntry("e", [x], [0])]).double().cpu().numpy() for x in e[80:]]
+    engine.end(["e"])
+    assert_logits_close(np.concatenate(rows), toy.planes_oracle(cfg, w, e)[79:], dtype, "e")
+    assert engine._graphs and engine._prompt_graphs
+    assert all(g.pool.n_free == g.pool.n_pages for g in engine.cache.groups)
+
+
+def test_attention_refuses_a_cache_entry_without_its_planes(ops):
+    """The attention kernels check what they are handed: a cache entry with other planes, or with
+    keys in another layout, is refused with an error that names what is there."""
+    from libllm_amd.errors import KernelError
+    from libllm_amd.parts import CacheNeed, CacheView, Plane, rows_plane
+    from libllm_amd.parts import kv_pages
+    ctx = make_ctx(ops, torch.bfloat16, [(0, 0, 3)])
+    q = torch.zeros((3, 2 * 16 * 3), dtype=torch.bfloat16, device="cuda")
+    table = torch.zeros((1, 1), dtype=torch.int32, device="cuda")
+    latent = CacheNeed("full", (rows_plane("z", (8,), 64),))
+    view = CacheView({"z": torch.zeros((2, 64, 8), device="cuda")}, table, 64, latent)
+    with pytest.raises(KernelError, match='planes "k" and "v"; this one has: z'):
+        ops.attention(q, 2, 2, 16, ctx, view, 0.25, 0)
+    good = kv_pages.kv_need(2, 16, 0, 64)
+    other = CacheNeed("full", (Plane("k", good.planes[0].page_shape, "rows"), good.planes[1]))
+    planes = {p.name: torch.zeros((2,) + p.page_shape, dtype=torch.bfloat16, device="cuda") for p in good.planes}
+    with pytest.raises(KernelError, match="laid out as 'rows'"):
+        ops.attention(q, 2, 2, 16, ctx, CacheView(planes, table, 64, other), 0.25, 0)
+    assert ops.attention(q, 2, 2, 16, ctx, CacheView(planes, table, 64, good), 0.25, 0).shape == (3, 32)
+
+
 def _halves_from_neighbours(w, n_heads, hd, rot):
     """Rows of a q or k projection (or bias) reordered so that the dims an interleaved encoding
     rotates together, (2j, 2j+1), become the pair (j, j + rot/2) of the rotate-half form."""

@@ -224,3 +224,114 @@ class CappedHead:
 
     def forward(self, ctx, h):
         return self.cap * torch.tanh(self.linear(ctx, h, out_dtype=torch.float32) / self.cap)
+
+
+# ---------------------------------------------------------------------------------------------
+# A mixer that keeps one latent row per token in the cache's pages, in a plane of its own (no
+# pair of keys and values, its own width and element type), and an input layer of another kind.
+from libllm_amd.config.spec import EmbeddingSpec  # noqa: E402
+from libllm_amd.parts import CacheNeed, Embedding, Stream, register_embedding, rows_plane  # noqa: E402
+
+
+@dataclass
+class LatentMixSpec(PartSpec):
+    width: int = 0
+    latent: int = 8
+
+
+@register_mixer("latent_mix")
+class LatentMix(Mixer):
+    """z_t = W_z x_t is cached (one row of ``latent`` numbers a token, in float32 whatever the
+    activations are); out_t = W_o sum_s softmax_s(q_t . z_s / sqrt(latent)) z_s over s <= t, with
+    q_t = W_q x_t: the cached rows are what is scored and what is summed."""
+    graph_safe = False               # walks the step's sequences on the host
+
+    def __init__(self, spec: LatentMixSpec):
+        self.width, self.latent = spec.width, spec.latent
+
+    def weights(self):
+        return {"z.weight": WeightDecl((self.latent, self.width)), "q.weight": WeightDecl((self.latent, self.width)),
+                "o.weight": WeightDecl((self.width, self.latent))}
+
+    def cache_need(self, page):
+        return CacheNeed("full", (rows_plane("z", (self.latent,), page, torch.float32),))
+
+    def bind(self, tensors, ops, dtype):
+        self.wz, self.wq, self.wo = (tensors[n + ".weight"].float() for n in "zqo")
+
+    def forward(self, ctx, x, entry):
+        view = ctx.kv(entry.cache)
+        pages, table, page = view.plane("z"), view.block_table, view.page_size
+        z_new, q = x.float() @ self.wz.t(), x.float() @ self.wq.t()
+        out = torch.empty_like(x)
+        row = 0
+        for slot, n, pos0 in zip(ctx.seq_slot_host, ctx.seq_lens, ctx.seq_pos0_host):
+            if n == 0:
+                continue
+            pos = torch.arange(pos0 + n, device=x.device)
+            where = table[slot].long()[pos // page]
+            if entry.writes:
+                pages[where[pos0:], pos[pos0:] % page] = z_new[row:row + n]
+            z = pages[where, pos % page]                              # [pos0 + n, latent], the new rows among them
+            s = q[row:row + n] @ z.t() / self.latent ** 0.5
+            s = s.masked_fill(pos[None, :] > pos[pos0:, None], float("-inf"))
+            out[row:row + n] = ((torch.softmax(s, dim=-1) @ z) @ self.wo.t()).to(x.dtype)
+            row += n
+        return out
+
+
+@dataclass
+class PositionedEmbeddingSpec(EmbeddingSpec):
+    max_position: int = 0
+    positions_tensor: str = "model.embed_positions.weight"
+
+
+@register_embedding("lookup_plus_positions")
+class PositionedEmbedding(Embedding):
+    """x_t = table[token_t] * scale + positions[position_t]: learned absolute positions."""
+    graph_safe = True                # index operations on device tensors only
+
+    def __init__(self, spec: PositionedEmbeddingSpec):
+        self.spec = spec
+
+    def weights(self):
+        s = self.spec
+        return {s.tensor: WeightDecl((s.vocab, s.width)), s.positions_tensor: WeightDecl((s.max_position, s.width))}
+
+    def bind(self, tensors, ops, dtype):
+        self.table, self.positions = tensors[self.spec.tensor], tensors[self.spec.positions_tensor]
+
+    def forward(self, ctx, then_norm=None):
+        rows = self.table[ctx.tokens.long()].float() * self.spec.scale + self.positions[ctx.tok_pos.long()].float()
+        return Stream(rows.contiguous())
+
+
+def planes_spec(base_config, latent=8):
+    """The Llama model as data with layer 0's mixer replaced by the latent mixer and the input
+    layer by the one with learned positions."""
+    spec = base_config.to_spec()
+    spec.layers[0].mixer = LatentMixSpec(kind="latent_mix", width=spec.width, latent=latent)
+    spec.layers[0].prefixes["mixer"] = "model.layers.0.latent."
+    e = spec.embedding
+    spec.embedding = PositionedEmbeddingSpec(e.vocab, e.width, e.tensor, e.scale, kind="lookup_plus_positions",
+                                             max_position=spec.max_position)
+    return spec
+
+
+def planes_oracle(cfg, weights, ids, latent=8):
+    """The same model through the plain functions, the two toys restated in numpy."""
+    import numpy as np
+
+    from plain import llama
+    t = len(ids)
+    x = llama.embedding(weights["model.embed_tokens.weight"], ids) + weights["model.embed_positions.weight"][:t]
+    positions = np.arange(t)
+    p = "model.layers.0."
+    h = llama.rms_norm(x, weights[p + "input_layernorm.weight"], cfg.eps)
+    z, q = h @ weights[p + "latent.z.weight"].T, h @ weights[p + "latent.q.weight"].T
+    s = q @ z.T / np.sqrt(latent) + llama.causal_mask(t)
+    x = x + (llama.softmax(s) @ z) @ weights[p + "latent.o.weight"].T
+    x = x + llama.mlp(cfg, weights, 0, llama.rms_norm(x, weights[p + "post_attention_layernorm.weight"], cfg.eps))
+    for layer in range(1, cfg.n_layers):
+        x = llama.decode_layer(cfg, weights, layer, x, positions)
+    return llama.lm_head(cfg, weights, llama.rms_norm(x, weights["model.norm.weight"], cfg.eps))
