@@ -13,6 +13,20 @@
 
 typedef uint16_t bf16_t;     // bfloat16 as raw bits: the upper half of an IEEE float
 
+// Activations of a gated feed-forward, out = act(gate) * up.  An entry point with a gated epilogue
+// takes the code in the upper bits of its `epilogue` argument (epilogue | act << 4); 0 is SiLU
+// (src/flint/cuda/swiglu.cu:44-49).
+#define LLM_ACT_SILU 0
+#define LLM_ACT_GELU_TANH 1      // 0.5 g (1 + tanh(sqrt(2 / pi) (g + 0.044715 g^3)))
+#define LLM_ACT_RELU 2
+#define LLM_ACT_COUNT 3
+__device__ __forceinline__ float llm_gated(int act, float g, float u) {
+  if (act == LLM_ACT_GELU_TANH)
+    return u * (0.5f * g * (1.0f + tanhf(0.7978845608028654f * (g + 0.044715f * g * g * g))));
+  if (act == LLM_ACT_RELU) return g > 0.f ? u * g : 0.f;
+  return u * g / (1.0f + expf(-g));
+}
+
 // Layout of the cache's pages.  A page holds 64 positions of every kv head; per (page, kv head):
 //   keys   [ceil(hd / 16)][64 positions][16 dims]   (blocks of 16 dims; a head size that is no
 //                                                    multiple of 16 pads its last block)

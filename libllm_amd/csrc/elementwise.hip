@@ -189,28 +189,28 @@ extern "C" int llm_add_rmsnorm(float* res, const void* delta, int delta_dtype, i
 
 // ---------------------------------------------------------------------------------- SiLU-mul
 // out[m, i] = gu[m, i] / (1 + exp(-gu[m, i])) * gu[m, I + i]: the gate is the first half
-// (src/flint/cuda/swiglu.cu:44-49).
+// (src/flint/cuda/swiglu.cu:44-49); `act` chooses another activation for the gate (common.h).
 template <typename T>
-__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I) {
+__global__ void silu_mul_kernel(const T* __restrict__ gu, T* __restrict__ out, int I, int act) {
   const int m = blockIdx.y;
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= I) return;
   const T* row = gu + (size_t)m * 2 * I;
   const float g = Conv<T>::load(row + i);
   const float u = Conv<T>::load(row + I + i);
-  Conv<T>::store(out + (size_t)m * I + i, u * g / (1.0f + expf(-g)));
+  Conv<T>::store(out + (size_t)m * I + i, llm_gated(act, g, u));
 }
 
 // The same for bfloat16 rows whose half width is a multiple of 8: 16 bytes of gate and of up per
 // thread, any number of rows through a grid-stride loop.
-__device__ __forceinline__ uint4 silu_mul_8(const uint4 g4, const uint4 u4) {
+__device__ __forceinline__ uint4 silu_mul_8(const uint4 g4, const uint4 u4, int act) {
   const uint32_t gw[4] = {g4.x, g4.y, g4.z, g4.w}, uw[4] = {u4.x, u4.y, u4.z, u4.w};
   uint32_t ow[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const float g0 = __uint_as_float(gw[j] << 16), g1 = __uint_as_float(gw[j] & 0xffff0000u);
     const float u0 = __uint_as_float(uw[j] << 16), u1 = __uint_as_float(uw[j] & 0xffff0000u);
-    const float r0 = u0 * g0 / (1.0f + expf(-g0)), r1 = u1 * g1 / (1.0f + expf(-g1));
+    const float r0 = llm_gated(act, g0, u0), r1 = llm_gated(act, g1, u1);
     ow[j] = (uint32_t)f32_to_bf16(r0) | ((uint32_t)f32_to_bf16(r1) << 16);
   }
   return make_uint4(ow[0], ow[1], ow[2], ow[3]);
@@ -219,7 +219,7 @@ __device__ __forceinline__ uint4 silu_mul_8(const uint4 g4, const uint4 u4) {
 // Two vectors a thread and round (the second half a grid apart), all four loads asked for before
 // the first is used.
 __global__ void silu_mul_vec_kernel(const bf16_t* __restrict__ gu, bf16_t* __restrict__ out, int I,
-                                    size_t total_vec) {
+                                    size_t total_vec, int act) {
   const int per_row = I / 8;
   const size_t span = (size_t)gridDim.x * blockDim.x;
   for (size_t v = (size_t)blockIdx.x * blockDim.x + threadIdx.x; v < total_vec; v += 2 * span) {
@@ -231,14 +231,14 @@ __global__ void silu_mul_vec_kernel(const bf16_t* __restrict__ gu, bf16_t* __res
     const uint4 ua = *reinterpret_cast<const uint4*>(gu + m * 2 * I + I + i);
     const uint4 gb = *reinterpret_cast<const uint4*>(gu + m2 * 2 * I + i2);
     const uint4 ub = *reinterpret_cast<const uint4*>(gu + m2 * 2 * I + I + i2);
-    *reinterpret_cast<uint4*>(out + m * I + i) = silu_mul_8(ga, ua);
-    if (two) *reinterpret_cast<uint4*>(out + m2 * I + i2) = silu_mul_8(gb, ub);
+    *reinterpret_cast<uint4*>(out + m * I + i) = silu_mul_8(ga, ua, act);
+    if (two) *reinterpret_cast<uint4*>(out + m2 * I + i2) = silu_mul_8(gb, ub, act);
   }
 }
 
-extern "C" int llm_silu_mul(const void* gu, void* out, int dtype, int M, int I, hipStream_t stream) {
+extern "C" int llm_silu_mul(const void* gu, void* out, int dtype, int M, int I, int act, hipStream_t stream) {
   if (M <= 0) return LLM_OK;
-  if (I <= 0 || M > 65535 * 32) return LLM_ERR_ARG;
+  if (I <= 0 || M > 65535 * 32 || act < 0 || act >= LLM_ACT_COUNT) return LLM_ERR_ARG;
   if (dtype == LLM_DTYPE_BF16 && I % 8 == 0 && ((((uintptr_t)gu) | ((uintptr_t)out)) & 15) == 0) {
     const size_t total_vec = (size_t)M * (I / 8);
     size_t blocks = (total_vec + 511) / 512;                      // two vectors a thread and round
@@ -248,7 +248,7 @@ extern "C" int llm_silu_mul(const void* gu, void* out, int dtype, int M, int I, 
     const size_t cap = (size_t)llm_compute_units() * 3;
     if (blocks > cap) blocks = cap;
     if (blocks == 0) blocks = 1;
-    silu_mul_vec_kernel<<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total_vec);
+    silu_mul_vec_kernel<<<(unsigned)blocks, 256, 0, stream>>>((const bf16_t*)gu, (bf16_t*)out, I, total_vec, act);
     return llm_launch_status();
   }
   // grid.y is limited to 65535: fold larger M into several launches
@@ -257,10 +257,10 @@ extern "C" int llm_silu_mul(const void* gu, void* out, int dtype, int M, int I, 
     dim3 grid((I + 255) / 256, mm);
     if (dtype == LLM_DTYPE_F32)
       silu_mul_kernel<float><<<grid, 256, 0, stream>>>((const float*)gu + (size_t)m0 * 2 * I,
-                                                        (float*)out + (size_t)m0 * I, I);
+                                                        (float*)out + (size_t)m0 * I, I, act);
     else if (dtype == LLM_DTYPE_BF16)
       silu_mul_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)gu + (size_t)m0 * 2 * I,
-                                                         (bf16_t*)out + (size_t)m0 * I, I);
+                                                         (bf16_t*)out + (size_t)m0 * I, I, act);
     else
       return LLM_ERR_ARG;
   }

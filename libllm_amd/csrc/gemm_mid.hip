@@ -26,6 +26,8 @@
 
 #define MID_EPI_NONE 0
 #define MID_EPI_SWIGLU 1
+#define MID_EPI_GATED 2      // as SwiGLU, the gate through the activation that the arguments name (common.h)
+#define MID_IS_GATED(E) ((E) == MID_EPI_SWIGLU || (E) == MID_EPI_GATED)
 #define MID_CK 128          // elements of K per chunk
 #define MID_STEPS 4         // steps of 32 per chunk
 #define MID_STAGES 4        // chunks of W in registers
@@ -56,7 +58,7 @@ template <int MT, int EPI, typename OutT>
 __global__ __launch_bounds__(MID_NT, 2) void gemm_mid_kernel(const bf16_t* __restrict__ X,
                                                              const bf16_t* __restrict__ W,
                                                              OutT* __restrict__ C, int M, int N, int K,
-                                                             int ldx, int w_steps, int n_out) {
+                                                             int ldx, int w_steps, int n_out, int act) {
   constexpr int ROW_B = MID_CK * 2;                  // bytes of a staged row: 16 pieces of 16 bytes, swizzled
   constexpr int BUF = 16 * MT * ROW_B;
   constexpr int PASSES = MT;                         // 256 threads carry 16 rows a pass
@@ -75,7 +77,7 @@ __global__ __launch_bounds__(MID_NT, 2) void gemm_mid_kernel(const bf16_t* __res
   const bf16_t* wp[MID_RT];
 #pragma unroll
   for (int rt = 0; rt < MID_RT; ++rt) {
-    if (EPI == MID_EPI_SWIGLU)
+    if (MID_IS_GATED(EPI))
       tile_row[rt] = rt * n_out + (blockIdx.x * 2 + wn) * 16;
     else
       tile_row[rt] = ((blockIdx.x * 2 + wn) * MID_RT + rt) * 16;
@@ -213,7 +215,7 @@ __global__ __launch_bounds__(MID_NT, 2) void gemm_mid_kernel(const bf16_t* __res
       acc[rt][mt] += f32x4{v.x, v.y, v.z, v.w};
     }
 
-  if (EPI == MID_EPI_SWIGLU) {
+  if (MID_IS_GATED(EPI)) {
     const int n = tile_row[0] + 4 * g;                 // output column: the gate tile's rows
     if (n >= n_out) return;
 #pragma unroll
@@ -224,7 +226,7 @@ __global__ __launch_bounds__(MID_NT, 2) void gemm_mid_kernel(const bf16_t* __res
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const float gt = bf16_to_f32(f32_to_bf16(acc[0][mt][e])), u = bf16_to_f32(f32_to_bf16(acc[1][mt][e]));
-        v[e] = u * gt / (1.0f + expf(-gt));
+        v[e] = (EPI == MID_EPI_SWIGLU) ? u * gt / (1.0f + expf(-gt)) : llm_gated(act, gt, u);
       }
       uint2 pk;
       pk.x = pack2_bf16(v[0], v[1]);
@@ -264,15 +266,15 @@ __global__ __launch_bounds__(MID_NT, 2) void gemm_mid_kernel(const bf16_t* __res
 
 template <int EPI, typename OutT>
 static int launch_mid(const bf16_t* X, const bf16_t* W, void* C, int M, int N, int K, int ldx,
-                      int k_split, hipStream_t stream) {
-  const int n_out = (EPI == MID_EPI_SWIGLU) ? N / 2 : N;
-  const int per_block = (EPI == MID_EPI_SWIGLU) ? 32 : 64;
+                      int k_split, int act, hipStream_t stream) {
+  const int n_out = (MID_IS_GATED(EPI)) ? N / 2 : N;
+  const int per_block = (MID_IS_GATED(EPI)) ? 32 : 64;
   const dim3 grid((n_out + per_block - 1) / per_block, k_split);
   const int w_steps = (K + 31) / 32;
 #define MID_CASE(T)                                                                                  \
   case T:                                                                                            \
     gemm_mid_kernel<T, EPI, OutT><<<grid, MID_NT, 0, stream>>>(X, W, (OutT*)C, M, N, K / k_split, ldx,  \
-                                                            w_steps, n_out);                         \
+                                                            w_steps, n_out, act);                    \
     break;
   switch ((M + 15) / 16) {
     MID_CASE(3)
@@ -289,10 +291,13 @@ static int launch_mid(const bf16_t* X, const bf16_t* W, void* C, int M, int N, i
 
 // X [M, K] bfloat16 with rows ldx apart, 33 <= M <= 128; W the tiled copy of a [N, K] matrix.
 // epilogue 0: C [M, N] bfloat16, or with k_split > 1 float32 [k_split, M, N], the products over
-// the slices of K; K is a multiple of 128 * k_split; epilogue 1: C [M, N/2] bfloat16, SwiGLU over
+// the slices of K; K is a multiple of 128 * k_split; epilogue 1 (1 | act << 4 for another activation of the gate, common.h): C [M, N/2] bfloat16, SwiGLU over
 // W = [Wg; Wu], N/2 a multiple of 16.
 extern "C" int llm_gemm_mid_bf16(const void* X, int ldx, const void* W_tiled, void* C, int epilogue,
                                  int out_dtype, int M, int N, int K, int k_split, hipStream_t stream) {
+  const int act = epilogue >> 4;                 // the gate's activation rides above the epilogue's code
+  epilogue &= 15;
+  if (act < 0 || act >= LLM_ACT_COUNT || (act != 0 && epilogue != MID_EPI_SWIGLU)) return LLM_ERR_ARG;
   if (M < 33 || M > 128 || N <= 0 || K <= 0 || (K & 7) || ldx < K || (ldx & 7) || k_split < 1)
     return LLM_ERR_ARG;
   if (X == nullptr || W_tiled == nullptr || C == nullptr) return LLM_ERR_ARG;
@@ -300,14 +305,16 @@ extern "C" int llm_gemm_mid_bf16(const void* X, int ldx, const void* W_tiled, vo
   if (k_split > 65535 || K % (k_split * MID_CK) != 0) return LLM_ERR_ARG;
   if (epilogue == MID_EPI_NONE) {
     if (k_split == 1 && out_dtype == LLM_DTYPE_BF16)
-      return launch_mid<MID_EPI_NONE, bf16_t>((const bf16_t*)X, (const bf16_t*)W_tiled, C, M, N, K, ldx, 1, stream);
+      return launch_mid<MID_EPI_NONE, bf16_t>((const bf16_t*)X, (const bf16_t*)W_tiled, C, M, N, K, ldx, 1, 0, stream);
     if (out_dtype == LLM_DTYPE_F32)
-      return launch_mid<MID_EPI_NONE, float>((const bf16_t*)X, (const bf16_t*)W_tiled, C, M, N, K, ldx, k_split, stream);
+      return launch_mid<MID_EPI_NONE, float>((const bf16_t*)X, (const bf16_t*)W_tiled, C, M, N, K, ldx, k_split, 0, stream);
     return LLM_ERR_ARG;
   }
   if (epilogue == MID_EPI_SWIGLU) {
     if ((N & 31) || out_dtype != LLM_DTYPE_BF16 || k_split != 1) return LLM_ERR_ARG;
-    return launch_mid<MID_EPI_SWIGLU, bf16_t>((const bf16_t*)X, (const bf16_t*)W_tiled, C, M, N, K, ldx, 1, stream);
+    if (act != LLM_ACT_SILU)      // SiLU keeps the kernel that knows nothing else
+      return launch_mid<MID_EPI_GATED, bf16_t>((const bf16_t*)X, (const bf16_t*)W_tiled, C, M, N, K, ldx, 1, act, stream);
+    return launch_mid<MID_EPI_SWIGLU, bf16_t>((const bf16_t*)X, (const bf16_t*)W_tiled, C, M, N, K, ldx, 1, 0, stream);
   }
   return LLM_ERR_ARG;
 }

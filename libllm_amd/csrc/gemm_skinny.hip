@@ -37,6 +37,8 @@
 #define SK_EPI_SWIGLU 1
 #define SK_EPI_ACCUM 2
 #define SK_EPI_ROPE 3
+#define SK_EPI_GATED 4       // as SwiGLU, the gate through the activation that the arguments name (common.h)
+#define SK_IS_GATED(E) ((E) == SK_EPI_SWIGLU || (E) == SK_EPI_GATED)
 
 // MT: 16-row tiles of X; RT: 16-row tiles of W per wave; WN: row groups per block; G: granules of
 // 2 steps that a wave takes per chunk (a chunk is 512*G elements of K).
@@ -60,6 +62,7 @@ struct SkinnyNorm {
   const float* ssq_in;     // [M, parts_in]: such sums for the rows of X, which still lack their scale; or null
   int parts_in;
   float eps;
+  int act;                 // gated epilogue: the gate's activation (common.h); 0 is SiLU
 };
 
 template <int MT, int RT, int WN, int G, int EPI, typename OutT>
@@ -73,7 +76,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   constexpr int CK = 512 * G;                    // elements of K per chunk
   constexpr int ROW_B = CK * 2;                  // bytes of a staged row; 16-byte pieces are swizzled
   constexpr int X_BYTES = 16 * MT * ROW_B;
-  constexpr int RED_BYTES = SK_WK * WN * ((EPI == SK_EPI_SWIGLU) ? 2 : 1) * MT * 1024;
+  constexpr int RED_BYTES = SK_WK * WN * ((SK_IS_GATED(EPI)) ? 2 : 1) * MT * 1024;
   constexpr int LDS_BYTES = X_BYTES > RED_BYTES ? X_BYTES : RED_BYTES;
   constexpr int XV = CK / 8;                     // 16-byte pieces of a staged row
   constexpr int ROWS_PASS = NT / XV;             // rows staged per pass of the block
@@ -98,7 +101,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   int tile_row[RT];
 #pragma unroll
   for (int rt = 0; rt < RT; ++rt) {
-    if (EPI == SK_EPI_SWIGLU)
+    if (SK_IS_GATED(EPI))
       tile_row[rt] = (rt & 1) * n_out + (group * (RT / 2) + (rt >> 1)) * 16;
     else
       tile_row[rt] = (group * RT + rt) * 16;
@@ -184,11 +187,11 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
   // a thread finishes at most one group of four outputs per round (ITEMS <= NT), and which one is
   // known from the start, so its position, cache page and rotation, or the values it adds to,
   // are in registers by the time the sums are (1 % of a decode step at up to 16 rows).
-  constexpr int RPR = (EPI == SK_EPI_SWIGLU) ? 2 : 1;    // W tiles of a row group per round
+  constexpr int RPR = (SK_IS_GATED(EPI)) ? 2 : 1;    // W tiles of a row group per round
   constexpr int OUT_RT = RT / RPR;
   constexpr int ITEMS = WN * MT * 64;
   static_assert(ITEMS <= NT, "one item a thread");
-  const int ldc = (EPI == SK_EPI_SWIGLU) ? n_out : N;
+  const int ldc = (SK_IS_GATED(EPI)) ? n_out : N;
   const int e_ln = tid & 63, e_mt = (tid >> 6) % MT, e_wn = tid / (64 * MT);
   const int e_m = e_mt * 16 + (e_ln & 15);
   const int e_n0 = (blockIdx.x * WN + e_wn) * OUT_RT * 16 + 4 * (e_ln >> 4);   // round ort adds 16 * ort
@@ -300,7 +303,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
     const int ln = e_ln, mt = e_mt, w_n = e_wn;
     float v[4];
     const int n = e_n0 + ort * 16;
-    if (EPI == SK_EPI_SWIGLU) {
+    if (SK_IS_GATED(EPI)) {
       float gsum[4] = {0.f, 0.f, 0.f, 0.f}, usum[4] = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
       for (int w = 0; w < SK_WK; ++w) {
@@ -322,7 +325,7 @@ __global__ __launch_bounds__(WN* SK_WK * 64) void gemm_skinny_kernel(const bf16_
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const float gt = bf16_to_f32(f32_to_bf16(gsum[e])), up = bf16_to_f32(f32_to_bf16(usum[e]));
-        v[e] = up * gt / (1.0f + expf(-gt));
+        v[e] = (EPI == SK_EPI_SWIGLU) ? up * gt / (1.0f + expf(-gt)) : llm_gated(norm.act, gt, up);
       }
     } else {
       float sum[4] = {0.f, 0.f, 0.f, 0.f};
@@ -436,9 +439,9 @@ struct SkinnyArgs {
 
 template <int MT, int RT, int WN, int G, int EPI, typename OutT>
 static int launch_skinny(const SkinnyArgs& a) {
-  const int rows = (EPI == SK_EPI_SWIGLU) ? a.n_out : a.N;
+  const int rows = (SK_IS_GATED(EPI)) ? a.n_out : a.N;
   const int tiles = (rows + 15) / 16;
-  constexpr int OUT_RT = (EPI == SK_EPI_SWIGLU) ? RT / 2 : RT;
+  constexpr int OUT_RT = (SK_IS_GATED(EPI)) ? RT / 2 : RT;
   const int blocks = (tiles + OUT_RT * WN - 1) / (OUT_RT * WN);
   const dim3 grid(blocks, a.k_split);
   gemm_skinny_kernel<MT, RT, WN, G, EPI, OutT><<<grid, WN * SK_WK * 64, 0, a.stream>>>(
@@ -450,7 +453,7 @@ static int launch_skinny(const SkinnyArgs& a) {
 template <int MT, int EPI, typename OutT>
 static int pick_rows(const SkinnyArgs& a) {
   const int units = llm_compute_units();
-  if constexpr (EPI == SK_EPI_SWIGLU) {
+  if constexpr (SK_IS_GATED(EPI)) {
     // four tiles a block (32 output columns) where that still leaves a block for every compute
     // unit; they pay from 33 rows of X on; at 17 to 32 rows two are 2 % of a decode step faster
     // (whole engines compared in one process; feed-forwards of 8,192 and 14,336 on 256 units)
@@ -469,7 +472,7 @@ static int pick_rows(const SkinnyArgs& a) {
 
 template <int EPI, typename OutT>
 static int pick_shape(const SkinnyArgs& a) {
-  constexpr int RT = (EPI == SK_EPI_SWIGLU) ? 2 : 1;
+  constexpr int RT = (SK_IS_GATED(EPI)) ? 2 : 1;
   const int mt = (a.M + 15) / 16;
   switch (mt) {
     case 1:
@@ -482,7 +485,7 @@ static int pick_shape(const SkinnyArgs& a) {
       // gate/up has more blocks than the chip has compute units: with the narrow chunk a block
       // needs few enough registers for two of them to share a unit, and the tail of one overlaps
       // the head of the next (3 % of a decode step at the 1B and 8B shapes, whole engines compared)
-      if constexpr (EPI == SK_EPI_SWIGLU) return launch_skinny<1, RT, 1, 1, EPI, OutT>(a);
+      if constexpr (SK_IS_GATED(EPI)) return launch_skinny<1, RT, 1, 1, EPI, OutT>(a);
       // likewise any weight with more tiles than units whose K gives fewer than three chunks of
       // 1,024: with the narrow chunk a block still has loads ahead of its arithmetic (the head of
       // the 1B shape, K = 2,048: 0.829 against 0.838 ms a decode step at batch 1, 0.977 against
@@ -502,12 +505,16 @@ static int pick_shape(const SkinnyArgs& a) {
 // tiled copy that llm_pack_weight makes.
 // With k_split > 1 (more than 16 rows, epilogue 0, float32) C is [k_split, M, N]: the products over
 // the k_split slices of K, for the caller to add in order.
-// C[M, N] (epilogue 0: stored as out_dtype; 2: added into the float32 C) or C[M, N/2] (epilogue 1,
+// C[M, N] (epilogue 0: stored as out_dtype; 2: added into the float32 C) or C[M, N/2] (epilogue 1, or 1 | act << 4 for another activation of the gate, common.h:
 // SwiGLU over W = [Wg; Wu], N/2 a multiple of 16) from X[M, K] and W[N, K].  X is bfloat16.
 static int skinny_product(const void* X, const void* W, void* C, int epilogue, int out_dtype, int M,
-                          int N, int K, int ldw, int k_split, const SkinnyNorm& norm,
+                          int N, int K, int ldw, int k_split, SkinnyNorm norm,
                           hipStream_t stream) {
   if (M <= 0 || N <= 0) return LLM_OK;
+  norm.act = epilogue >> 4;                    // the gate's activation rides above the epilogue's code
+  epilogue &= 15;
+  if (norm.act < 0 || norm.act >= LLM_ACT_COUNT || (norm.act != 0 && epilogue != SK_EPI_SWIGLU)) return LLM_ERR_ARG;
+  if (norm.act != LLM_ACT_SILU) epilogue = SK_EPI_GATED;       // SiLU keeps the kernel that knows nothing else
   // slices of K: more than 16 rows, plain epilogue, float32 results [k_split, M, N]
   if (k_split < 1 || (k_split > 1 && (M <= 16 || epilogue != SK_EPI_NONE || out_dtype != LLM_DTYPE_F32 ||
                                       K % (k_split * 32) != 0)))
@@ -531,10 +538,10 @@ static int skinny_product(const void* X, const void* W, void* C, int epilogue, i
   if (epilogue == SK_EPI_NONE) {
     if (out_dtype == LLM_DTYPE_BF16) return pick_shape<SK_EPI_NONE, bf16_t>(a);
     if (out_dtype == LLM_DTYPE_F32) return pick_shape<SK_EPI_NONE, float>(a);
-  } else if (epilogue == SK_EPI_SWIGLU) {
+  } else if (SK_IS_GATED(epilogue)) {
     if ((N & 31) || out_dtype != LLM_DTYPE_BF16) return LLM_ERR_ARG;
     a.n_out = N / 2;
-    return pick_shape<SK_EPI_SWIGLU, bf16_t>(a);
+    return epilogue == SK_EPI_SWIGLU ? pick_shape<SK_EPI_SWIGLU, bf16_t>(a) : pick_shape<SK_EPI_GATED, bf16_t>(a);
   } else if (epilogue == SK_EPI_ACCUM) {
     if (out_dtype != LLM_DTYPE_F32) return LLM_ERR_ARG;
     return pick_shape<SK_EPI_ACCUM, float>(a);
@@ -569,7 +576,7 @@ extern "C" int llm_gemm_skinny_norm_bf16(const void* X, const void* W, void* C, 
     norm.ssq_out = ssq_out;
   }
   if (ssq_in != nullptr) {
-    if (epilogue == SK_EPI_ACCUM || parts_in <= 0 || !(eps >= 0.f)) return LLM_ERR_ARG;
+    if ((epilogue & 15) == SK_EPI_ACCUM || parts_in <= 0 || !(eps >= 0.f)) return LLM_ERR_ARG;
     norm.ssq_in = ssq_in;
     norm.parts_in = parts_in;
     norm.eps = eps;

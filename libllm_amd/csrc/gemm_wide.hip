@@ -29,12 +29,14 @@
 #define WD_NT 512          // threads of a block
 #define WD_EPI_NONE 0
 #define WD_EPI_SWIGLU 1
+#define WD_EPI_GATED 2       // as SwiGLU, the gate through the activation that the arguments name (common.h)
+#define WD_IS_GATED(E) ((E) == WD_EPI_SWIGLU || (E) == WD_EPI_GATED)
 
 template <int EPI, int BM>
 __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restrict__ X, int ldx,
                                                           const bf16_t* __restrict__ W, int ldw,
                                                           bf16_t* __restrict__ C, int M, int N, int K,
-                                                          int n_out, int m_tiles, int n_tiles) {
+                                                          int n_out, int m_tiles, int n_tiles, int act) {
   extern __shared__ __attribute__((aligned(16))) unsigned char lds[];
   static_assert(BM == 256 || BM == 128, "rows of X a block");
   constexpr int OPER = 256 * 128;                 // bytes of W's tile; X's follows it
@@ -73,7 +75,7 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
   for (int p = 0; p < 4; ++p) {
     const int row = row0 + 64 * p;
     int n;
-    if (EPI == WD_EPI_SWIGLU) {
+    if (WD_IS_GATED(EPI)) {
       n = nt_blk * 128 + (row & 127);
       if (n > n_out - 1) n = n_out - 1;
       n += (row >> 7) * n_out;
@@ -114,7 +116,7 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
   int a_row[NTW], b_row[4];
 #pragma unroll
   for (int nt = 0; nt < NTW; ++nt)
-    a_row[nt] = (EPI == WD_EPI_SWIGLU) ? ((nt / (NTW / 2)) * 128 + wn * (NTW / 2) * 16 + (nt % (NTW / 2)) * 16 + r)
+    a_row[nt] = (WD_IS_GATED(EPI)) ? ((nt / (NTW / 2)) * 128 + wn * (NTW / 2) * 16 + (nt % (NTW / 2)) * 16 + r)
                                        : (wn * NTW * 16 + nt * 16 + r);
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt) b_row[mt] = wm * 64 + mt * 16 + r;
@@ -199,7 +201,7 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
   // bytes longer than they are so that the 16 rows of a store fall into different banks, and then
   // stores whole rows, 16 bytes a lane.
   __syncthreads();                                   // every wave has read the last tile
-  constexpr int OUT_T = (EPI == WD_EPI_SWIGLU) ? NTW / 2 : NTW;   // tiles of 16 outputs of a wave
+  constexpr int OUT_T = (WD_IS_GATED(EPI)) ? NTW / 2 : NTW;   // tiles of 16 outputs of a wave
   constexpr int OUT_COLS = OUT_T * 16;
   constexpr int ROW_B = OUT_COLS * 2 + 16;
   unsigned char* mine = lds + wave * (64 * ROW_B);
@@ -208,7 +210,7 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
 #pragma unroll
     for (int nt = 0; nt < OUT_COLS / 16; ++nt) {
       uint2 pk;
-      if (EPI == WD_EPI_SWIGLU) {
+      if (WD_IS_GATED(EPI)) {
         // gate and up rounded to bfloat16 first, as the unfused path stores them; the exponential
         // and the reciprocal by the hardware's instructions (their error is far below the rounding
         // of the result)
@@ -219,7 +221,8 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e)
-          v[e] = up[e] * gt[e] * __builtin_amdgcn_rcpf(1.0f + fast_exp2(-1.4426950408889634f * gt[e]));
+          v[e] = (EPI == WD_EPI_SWIGLU) ? up[e] * gt[e] * __builtin_amdgcn_rcpf(1.0f + fast_exp2(-1.4426950408889634f * gt[e]))
+                                        : llm_gated(act, gt[e], up[e]);
         pk.x = pack2_bf16(v[0], v[1]);
         pk.y = pack2_bf16(v[2], v[3]);
       } else {
@@ -231,8 +234,8 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
   // (a wave reads only what it wrote itself: the compiler's wait for its stores is enough)
   constexpr int LPR = OUT_COLS / 8;                  // lanes a row
   constexpr int RPP = 64 / LPR;                      // rows a pass
-  const int ldc = (EPI == WD_EPI_SWIGLU) ? n_out : N;
-  const int n_wave = (EPI == WD_EPI_SWIGLU) ? nt_blk * 128 + wn * OUT_COLS : nt_blk * WD_BN + wn * OUT_COLS;
+  const int ldc = (WD_IS_GATED(EPI)) ? n_out : N;
+  const int n_wave = (WD_IS_GATED(EPI)) ? nt_blk * 128 + wn * OUT_COLS : nt_blk * WD_BN + wn * OUT_COLS;
   const int col = (lane % LPR) * 8;
 #pragma unroll
   for (int pass = 0; pass < 64 / RPP; ++pass) {
@@ -255,9 +258,9 @@ __global__ __launch_bounds__(WD_NT) void gemm_wide_kernel(const bf16_t* __restri
 
 template <int EPI, int BM>
 static int launch_wide(const void* X, int ldx, const void* W, int ldw, void* C, int M, int N, int K,
-                       int n_out, hipStream_t stream) {
+                       int n_out, int act, hipStream_t stream) {
   const int m_tiles = (M + BM - 1) / BM;
-  const int per = (EPI == WD_EPI_SWIGLU) ? 128 : WD_BN;
+  const int per = (WD_IS_GATED(EPI)) ? 128 : WD_BN;
   const int n_tiles = (n_out + per - 1) / per;
   const long long blocks = 8LL * ((m_tiles + 7) / 8) * 8 * ((n_tiles + 7) / 8);   // bands of 8 tiles of X rows; surplus blocks leave at once
   if (blocks > 0x7fffffffLL) return LLM_ERR_ARG;
@@ -274,16 +277,20 @@ static int launch_wide(const void* X, int ldx, const void* W, int ldw, void* C, 
     asked[dev] = true;
   }
   gemm_wide_kernel<EPI, BM><<<(unsigned)blocks, WD_NT, lds_bytes, stream>>>(
-      (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (bf16_t*)C, M, N, K, n_out, m_tiles, n_tiles);
+      (const bf16_t*)X, ldx, (const bf16_t*)W, ldw, (bf16_t*)C, M, N, K, n_out, m_tiles, n_tiles, act);
   return llm_launch_status();
 }
 
 // X [M, K] rows ldx apart, W [N, K] rows ldw apart (both bfloat16, K a multiple of 64, 16-byte aligned rows);
-// epilogue 0: C [M, N]; 1: C [M, N/2], SwiGLU over W = [Wg; Wu], N/2 a multiple of 16.
+// epilogue 0: C [M, N]; 1: C [M, N/2], SwiGLU over W = [Wg; Wu], N/2 a multiple of 16 (1 | act << 4:
+// the gate through another activation of common.h).
 // block_rows: rows of X a block takes, 256 or 128 (half the arithmetic per byte a unit reads, twice
 // the blocks: for steps whose tiles of 256 rows would leave units idle).
 extern "C" int llm_gemm_wide_bf16(const void* X, int ldx, const void* W, int ldw, void* C, int epilogue,
                                   int block_rows, int M, int N, int K, hipStream_t stream) {
+  const int act = epilogue >> 4;                 // the gate's activation rides above the epilogue's code
+  epilogue &= 15;
+  if (act < 0 || act >= LLM_ACT_COUNT || (act != 0 && epilogue != WD_EPI_SWIGLU)) return LLM_ERR_ARG;
   if (M <= 0 || N <= 0 || K < WD_BK || (K % WD_BK) || ldx < K || ldw < K || (ldx & 7) || (ldw & 7)) return LLM_ERR_ARG;
   if ((((uintptr_t)X) | ((uintptr_t)W) | ((uintptr_t)C)) & 15) return LLM_ERR_ARG;
   if (epilogue != WD_EPI_NONE && epilogue != WD_EPI_SWIGLU) return LLM_ERR_ARG;
@@ -292,9 +299,12 @@ extern "C" int llm_gemm_wide_bf16(const void* X, int ldx, const void* W, int ldw
   const int n_out = (epilogue == WD_EPI_SWIGLU) ? N / 2 : N;
   if (epilogue == WD_EPI_SWIGLU && (N & 31)) return LLM_ERR_ARG;
   if (n_out & 3) return LLM_ERR_ARG;
+  if (epilogue == WD_EPI_SWIGLU && act != LLM_ACT_SILU)       // SiLU keeps the kernel that knows nothing else
+    return block_rows == 256 ? launch_wide<WD_EPI_GATED, 256>(X, ldx, W, ldw, C, M, N, K, n_out, act, stream)
+                             : launch_wide<WD_EPI_GATED, 128>(X, ldx, W, ldw, C, M, N, K, n_out, act, stream);
   if (epilogue == WD_EPI_SWIGLU)
-    return block_rows == 256 ? launch_wide<WD_EPI_SWIGLU, 256>(X, ldx, W, ldw, C, M, N, K, n_out, stream)
-                             : launch_wide<WD_EPI_SWIGLU, 128>(X, ldx, W, ldw, C, M, N, K, n_out, stream);
-  return block_rows == 256 ? launch_wide<WD_EPI_NONE, 256>(X, ldx, W, ldw, C, M, N, K, n_out, stream)
-                           : launch_wide<WD_EPI_NONE, 128>(X, ldx, W, ldw, C, M, N, K, n_out, stream);
+    return block_rows == 256 ? launch_wide<WD_EPI_SWIGLU, 256>(X, ldx, W, ldw, C, M, N, K, n_out, 0, stream)
+                             : launch_wide<WD_EPI_SWIGLU, 128>(X, ldx, W, ldw, C, M, N, K, n_out, 0, stream);
+  return block_rows == 256 ? launch_wide<WD_EPI_NONE, 256>(X, ldx, W, ldw, C, M, N, K, n_out, 0, stream)
+                           : launch_wide<WD_EPI_NONE, 128>(X, ldx, W, ldw, C, M, N, K, n_out, 0, stream);
 }

@@ -35,7 +35,7 @@ _SIGNATURES = {
     "llm_embed": [_vp, _i, _vp, _vp, _i, _i, _i, _f, _vp],
     "llm_embed_norm": [_vp, _i, _vp, _vp, _i, _i, _i, _f, _vp, _vp, _vp, _vp],
     "llm_add_rmsnorm": [_vp, _vp, _i, _i, ctypes.c_size_t, _vp, _f, _vp, _i, _vp, _i, _i, _vp],
-    "llm_silu_mul": [_vp, _vp, _i, _i, _i, _vp],
+    "llm_silu_mul": [_vp, _vp, _i, _i, _i, _i, _vp],
     "llm_add_bias": [_vp, _i, _vp, _i, _i, _vp],
     "llm_rope_kv_write": [_vp, _i, _i, _vp, _i, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp,
                           _vp, _i, _i, _i, _i, _vp],
@@ -149,6 +149,9 @@ class HipOps:
     # lengths do not move the crossing (4 x 1,024 rows: 39.1 against 43.0).
     PROMPT_TILE_ROWS = (3584, 2560)
     _EPI_NONE, _EPI_SWIGLU, _EPI_ACCUM = 0, 1, 2
+    # activations of the gate in a gated feed-forward (csrc/common.h); a gated epilogue takes the
+    # code above its own: epilogue | act << 4
+    ACTIVATIONS = {"silu": 0, "gelu_tanh": 1, "relu": 2}
 
     def __init__(self, device: Optional[str] = None):
         if not torch.cuda.is_available():
@@ -460,7 +463,7 @@ class HipOps:
         """Launches the skinny kernel on rows m0 .. m0+mm of the bfloat16 matrix x; with ``k_split``
         the products over that many slices of K go to ``out[k_split, mm, n]``."""
         n, k = w.shape
-        width = n // 2 if epilogue == self._EPI_SWIGLU else n
+        width = n // 2 if (epilogue & 15) == self._EPI_SWIGLU else n
         wptr, ldw = self._streamed(w)
         if isinstance(x, NormedRows):           # rows that lack their norm's scale: see Prenormed
             pre = x.pre
@@ -562,10 +565,17 @@ class HipOps:
                                               self._stream()), "add_bias")
         return out if out.dtype == out_dtype else out.to(out_dtype)
 
-    def linear_swiglu(self, x, w, dtype=None):
-        """silu(x Wg^T) * (x Wu^T) for the stacked weight ``w = [Wg; Wu]``: one kernel for few
-        rows in bfloat16, else the product followed by the SiLU-mul kernel.  ``x`` is a matrix or
-        a ``normed`` record; ``dtype`` is the activation dtype (needed for a record)."""
+    def _act(self, activation):
+        if activation not in self.ACTIVATIONS:
+            raise KernelError("unknown activation %r (known: %s)" % (activation, ", ".join(sorted(self.ACTIVATIONS))))
+        return self.ACTIVATIONS[activation]
+
+    def linear_swiglu(self, x, w, dtype=None, activation="silu"):
+        """act(x Wg^T) * (x Wu^T) for the stacked weight ``w = [Wg; Wu]``, ``act`` being SiLU or
+        another of ``ACTIVATIONS``: one kernel where a product of ours takes the rows, else the
+        library's product followed by the kernel that gates.  ``x`` is a matrix or a ``normed``
+        record; ``dtype`` is the activation dtype (needed for a record)."""
+        gated = self._EPI_SWIGLU | (self._act(activation) << 4)
         lazy = isinstance(x, NormedRows)
         m, k = (x.n_rows, x.res.shape[1]) if lazy else x.shape
         dtype = dtype or (x.dtype if not lazy else None)
@@ -579,31 +589,31 @@ class HipOps:
                 and dtype == torch.bfloat16 and not self._mid_ok(x, w, m, k)):
             self._weight(self._plain(w), "linear weight")
             out = torch.empty((m, inter), dtype=torch.bfloat16, device=self.device)
-            self._skinny(x, w, out, self._EPI_SWIGLU, 0, m)
+            self._skinny(x, w, out, gated, 0, m)
             return out
         if lazy:
             if dtype is None:
                 raise KernelError("linear_swiglu: a normed record needs the activation dtype")
             x = self._materialise(x, dtype)
-            return self.linear_swiglu(x, w, dtype)
+            return self.linear_swiglu(x, w, dtype, activation)
         if self._mid_ok(x, w, m, k) and inter % 16 == 0 and dtype == torch.bfloat16:
             self._weight(self._plain(w), "linear weight")
-            return self._mid(x, w, torch.empty((m, inter), dtype=torch.bfloat16, device=self.device),
-                             self._EPI_SWIGLU)
+            return self._mid(x, w, torch.empty((m, inter), dtype=torch.bfloat16, device=self.device), gated)
         if dtype == torch.bfloat16 and (block_rows := self._wide_ok(x, w, m, k, inter)):
             self._weight(self._plain(w), "linear weight")
             self._dev(x, "linear input")
             return self._wide(x, w, torch.empty((m, inter), dtype=torch.bfloat16, device=self.device),
-                              self._EPI_SWIGLU, block_rows)
-        return self.silu_mul(self.linear(x, w, None, x.dtype))
+                              gated, block_rows)
+        return self.silu_mul(self.linear(x, w, None, x.dtype), activation)
 
-    def silu_mul(self, gu):
+    def silu_mul(self, gu, activation="silu"):
+        """act(first half of each row) * second half; ``act`` is SiLU unless said otherwise."""
         m, two_i = gu.shape
         if two_i % 2:
             raise KernelError("silu_mul: the input width %d is odd" % two_i)
         out = torch.empty((m, two_i // 2), dtype=gu.dtype, device=self.device)
         self._check(self.lib.llm_silu_mul(self._dev(gu, "gate_up"), out.data_ptr(), _code(gu.dtype),
-                                          m, two_i // 2, self._stream()), "silu_mul")
+                                          m, two_i // 2, self._act(activation), self._stream()), "silu_mul")
         return out
 
     # rotating pairs side by side (2j, 2j+1) let the projection's epilogue rotate them: a mixer

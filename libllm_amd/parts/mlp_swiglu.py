@@ -1,6 +1,8 @@
 """SwiGLU feed-forward: down(silu(gate(x)) * up(x)); gate and up are one matrix product over the
 stacked weight, gate rows first (src/libllm/llama.cc:81-98, tools/llama_exporter.py:73-78,
-src/flint/cuda/swiglu.cu:44-49)."""
+src/flint/cuda/swiglu.cu:44-49).  The record may name another activation for the gate, of those
+the operations know (``ops.ACTIVATIONS``); the Llama configuration asks for SiLU only, as the
+reference does (tools/llama_exporter.py:87-88)."""
 from dataclasses import dataclass
 
 import torch
@@ -21,6 +23,9 @@ class SwiGLUSpec(PartSpec):
     down_name: str = "down_proj"
 
 
+ACTIVATIONS = ("silu", "gelu_tanh", "relu")
+
+
 @register_feed_forward("swiglu")
 class SwiGLU(FeedForward):
     graph_safe = True      # reads nothing from the host during a step
@@ -28,9 +33,9 @@ class SwiGLU(FeedForward):
     adds_to_stream = True  # the output product can add into the residual stream
 
     def __init__(self, spec: SwiGLUSpec):
-        if spec.activation != "silu":
-            raise ConfigError("feed-forward activation %r is not supported (silu only)"
-                              % (spec.activation,))
+        if spec.activation not in ACTIVATIONS:
+            raise ConfigError("feed-forward activation %r is not supported (known: %s)"
+                              % (spec.activation, ", ".join(ACTIVATIONS)))
         if spec.width <= 0 or spec.intermediate <= 0:
             raise ConfigError("feed-forward sizes must be positive")
         self.spec = spec
@@ -54,5 +59,8 @@ class SwiGLU(FeedForward):
         self.down.bind(tensors[s.down_name + ".weight"], ops=ops)
 
     def forward(self, ctx: StepContext, x, residual=None):
-        h = ctx.ops.linear_swiglu(x, self.gate_up.prepared, ctx.dtype)
+        if self.spec.activation == "silu":
+            h = ctx.ops.linear_swiglu(x, self.gate_up.prepared, ctx.dtype)
+        else:
+            h = ctx.ops.linear_swiglu(x, self.gate_up.prepared, ctx.dtype, self.spec.activation)
         return self.down(ctx, h, residual=residual)

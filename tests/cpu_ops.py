@@ -36,13 +36,15 @@ class CpuOps:
             return y.to(torch.bfloat16)
         return y.to(out_dtype)
 
-    def linear_swiglu(self, x, w, dtype=None):
-        return self.silu_mul(self.linear(x, w, None, x.dtype))
+    def linear_swiglu(self, x, w, dtype=None, activation="silu"):
+        return self.silu_mul(self.linear(x, w, None, x.dtype), activation)
 
-    def silu_mul(self, gu):
+    def silu_mul(self, gu, activation="silu"):
         i = gu.shape[1] // 2
         g, u = gu[:, :i].float(), gu[:, i:].float()
-        return (u * g / (1.0 + torch.exp(-g))).to(gu.dtype)
+        act = {"silu": lambda t: t / (1.0 + torch.exp(-t)), "relu": torch.relu,
+               "gelu_tanh": lambda t: torch.nn.functional.gelu(t, approximate="tanh")}[activation]
+        return (u * act(g)).to(gu.dtype)
 
     def rope_kv_write(self, qkv, bias, n_heads, n_kv, hd, cos, sin, rot_dim, ctx, kv, write):
         m = qkv.shape[0]

@@ -529,6 +529,60 @@ def test_gemm_mid_refuses(ops):
         ops._mid(rnd((100, 200), torch.bfloat16, 2).cuda(), w2, torch.empty((100, 64), dtype=torch.bfloat16, device="cuda"), ops._EPI_NONE)
 
 
+# ---------------------------------------------------------------- other activations of the gate
+def gate_act(name, g):
+    """The gate's activation in float64: SiLU (src/flint/cuda/swiglu.cu:44-49), GELU in its tanh
+    form, ReLU."""
+    if name == "silu":
+        return g / (1 + torch.exp(-g))
+    if name == "relu":
+        return torch.relu(g)
+    return 0.5 * g * (1 + torch.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g ** 3)))
+
+
+@pytest.mark.parametrize("activation", ["gelu_tanh", "relu", "silu"])
+def test_gated_products_with_other_activations(ops, activation):
+    """act(gate) * up with another activation than SiLU, through every kernel that gates: the
+    product for few rows (1, 16, 40 rows), the one for 33 to 128 rows, the one for many rows in
+    both sizes of block, and the gating kernel behind the library's product, in both dtypes."""
+    inter, k = 512, 256
+    w = rnd((2 * inter, k), torch.bfloat16, 6, scale=0.08).cuda()
+    pw = ops.prepare_weight(w)
+
+    def want(x):
+        gu = (x.double() @ w.double().t()).bfloat16().double()
+        return gu[:, inter:] * gate_act(activation, gu[:, :inter])
+
+    def err(out, ref):
+        return ((out.double().cpu() - ref.cpu()).abs() / (ref.cpu().abs() + ref.cpu().abs().mean())).max().item()
+    code = ops._EPI_SWIGLU | (ops.ACTIVATIONS[activation] << 4)
+    for m in (1, 16, 40, 64):
+        x = rnd((m, k), torch.bfloat16, m).cuda()
+        out = torch.empty((m, inter), dtype=torch.bfloat16, device="cuda")
+        ops._skinny(x, pw, out, code, 0, m)
+        assert err(out, want(x)) < 0.02, ("few rows", m)
+    for m in (33, 128):
+        x = rnd((m, k), torch.bfloat16, m).cuda()
+        out = ops._mid(x, pw, torch.empty((m, inter), dtype=torch.bfloat16, device="cuda"), code)
+        assert err(out, want(x)) < 0.02, ("33 to 128 rows", m)
+    for block_rows in (256, 128):
+        x = rnd((300, k), torch.bfloat16, 9).cuda()
+        out = ops._wide(x, pw, torch.empty((300, inter), dtype=torch.bfloat16, device="cuda"), code, block_rows)
+        assert err(out, want(x)) < 0.02, ("many rows", block_rows)
+    for m in (5, 200):                                            # whatever form the launcher picks
+        x = rnd((m, k), torch.bfloat16, m + 1).cuda()
+        assert err(ops.linear_swiglu(x, pw, torch.bfloat16, activation), want(x)) < 0.02
+    for dtype in DTYPES:
+        gu = rnd((9, 152), dtype, 15, 2.0).cuda()
+        ref = gu[:, 76:].double() * gate_act(activation, gu[:, :76].double())
+        assert close(ops.silu_mul(gu, activation), ref, dtype, f32=2e-6)
+    gu = rnd((70, 1024), torch.bfloat16, 16, 2.0).cuda()        # the vector form
+    assert close(ops.silu_mul(gu, activation), gu[:, 512:].double() * gate_act(activation, gu[:, :512].double()), torch.bfloat16)
+    from libllm_amd.errors import KernelError
+    with pytest.raises(KernelError, match="unknown activation"):
+        ops.silu_mul(gu, "swish9")
+
+
 # ---------------------------------------------------------------- the product for many rows
 @pytest.mark.parametrize("block_rows", [256, 128])
 @pytest.mark.parametrize("mnk", [(129, 64, 64), (300, 520, 128), (2048, 512, 256), (257, 1000, 192), (600, 264, 4096),

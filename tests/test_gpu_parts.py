@@ -278,6 +278,29 @@ def test_toy_mixer_with_a_plane_of_its_own_and_toy_input_layer(ops, dtype):
     assert all(g.pool.n_free == g.pool.n_pages for g in engine.cache.groups)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("activation", ["gelu_tanh", "relu"])
+def test_feed_forward_with_another_activation(ops, dtype, activation):
+    """The gated feed-forward with another activation of the gate, chosen in the part's record:
+    steps of 3, 20, 50, 100 and 200 rows go through each form of the gated product (few rows,
+    33 to 128 rows, the library's with the gating kernel behind it)."""
+    from test_gpu_kernels import gate_act
+    spec = SwiGLUSpec(kind="swiglu", width=128, intermediate=384, activation=activation)
+    ff = build_feed_forward(spec)
+    dev, host = weights_for(ff, "ff.", 5, dtype)
+    ff.bind(dev, ops, dtype)
+    for m in (3, 20, 50, 100, 200):
+        ctx = make_ctx(ops, dtype, [(0, 0, m)])
+        x = rows(m, 128, dtype, m)
+        out = ff.forward(ctx, x.cuda())
+        xd = x.double().numpy()
+        gate, up = xd @ host["ff.gate_proj.weight"].T, xd @ host["ff.up_proj.weight"].T
+        ref = (up * gate_act(activation, torch.from_numpy(gate)).numpy()) @ host["ff.down_proj.weight"].T
+        assert rel_err(out.double().cpu().numpy(), ref) < tol(dtype), (m, activation)
+    with pytest.raises(Exception, match="not supported"):
+        build_feed_forward(SwiGLUSpec(kind="swiglu", width=128, intermediate=384, activation="swish9"))
+
+
 def test_attention_refuses_a_cache_entry_without_its_planes(ops):
     """The attention kernels check what they are handed: a cache entry with other planes, or with
     keys in another layout, is refused with an error that names what is there."""
