@@ -39,8 +39,12 @@ class Engine:
     # Queued from the host a prompt of up to some hundred tokens waits for the host, not the device.
     # Up to 128 rows the steps are 16 apart, as the products' forms are: a prompt of 70 tokens in
     # a graph of 80 or 96 rows takes 1.47 ms where one of 128 rows takes 1.58 (1B shape; 5.34
-    # against 5.85 at 8B).
-    PROMPT_ROWS = (16, 32, 48, 64, 80, 96, 112, 128, 192, 256, 384, 512, 768, 1024, 1536, 2048)
+    # against 5.85 at 8B).  Beyond, the vendor library's products run, whose time grows evenly with
+    # the rows but for a few row counts at which its choice of kernel is poor: at exactly 192 rows
+    # the four products of a layer take 153 us where they take 108 at 184 rows and 111 at 200 (3B
+    # shape; 237 against 177 and 182 at 8B; 1B the same everywhere), and likewise at 160 rows of
+    # the 8B shape.  Hence 176 and 224 between 128 and 256, and no 192.
+    PROMPT_ROWS = (16, 32, 48, 64, 80, 96, 112, 128, 176, 224, 256, 384, 512, 768, 1024, 1536, 2048)
     PROMPT_SEQS = (2, 3, 5, 9, 17)
     PROMPT_SEEN = 2
     PROMPT_GRAPHS = 24      # prompt graphs kept; the one unused for longest goes first (each holds its activations)
