@@ -711,7 +711,7 @@ def test_captures_with_an_eager_collector(models):
         gc.set_threshold(*old)
 
 
-@pytest.mark.parametrize("rows", [512, 2048])
+@pytest.mark.parametrize("rows", [176, 224, 512, 2048])
 def test_library_products_inside_prompt_graphs(rows):
     """A prompt of real width fills its graph exactly, so that the graph and an engine without
     graphs run the same kernels, the library's for large products among them: six replays with
