@@ -526,6 +526,41 @@ def test_padding_changes_nothing(models):
     assert np.array_equal(a, b[:, :5])
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("use_graphs", [False, True])
+def test_steps_seen_before_ask_the_device_for_no_memory(models, use_graphs, dtype):
+    """Once steps of some shapes have run, steps of those shapes ask the device for no memory:
+    what the operations allocate is cut from blocks that the process holds already (a captured
+    graph's own pool; for steps queued kernel by kernel the pool that hands a step's blocks
+    back as its tensors die, as the reference's stream-ordered pool does,
+    src/flint/cuda/common.h:116-142).  Counted by the pool's requests to the device and by the
+    bytes it holds."""
+    import torch
+    from libllm_amd.engine import StepEntry
+    from libllm_amd.runtime import load_engine
+    path, cfg, _ = models["A"]
+    engine = load_engine(path, dtype=dtype, max_tokens=1024, use_graphs=use_graphs)
+    lengths = [9, 70, 31]
+
+    def batch(seed):
+        requests = make_requests(cfg, lengths, seed=seed)
+        engine.step([StepEntry(r, t, [len(t) - 1]) for r, t in requests.items()])
+        for k in range(6):
+            out = engine.step([StepEntry(r, [(seed + k) % cfg.vocab], [0]) for r in requests])
+        engine.end(list(requests))
+        return out.float().sum().item()                      # waits for the device
+
+    for seed in range(3):                                    # a prompt's graph is captured when its shape comes again
+        batch(seed)
+    stats = torch.cuda.memory_stats()
+    asked, held = stats["num_device_alloc"], stats["reserved_bytes.all.current"]
+    for seed in range(3, 7):
+        batch(seed)
+    stats = torch.cuda.memory_stats()
+    assert stats["num_device_alloc"] == asked and stats["reserved_bytes.all.current"] == held
+    assert bool(engine._graphs) == use_graphs and bool(engine._prompt_graphs) == use_graphs
+
+
 @pytest.mark.parametrize("name", list(CONFIGS))
 def test_norms_between_products_get_no_kernel(models, name):
     """Decoding up to 16 rows in bfloat16, the product that adds into the stream prepares the RMS
