@@ -53,8 +53,19 @@ SHAPES = {
            "intermediate_size": 14336, "tie_word_embeddings": False,
            "rope_scaling": {"rope_type": "llama3", "factor": 8.0, "low_freq_factor": 1.0,
                             "high_freq_factor": 4.0, "original_max_position_embeddings": 8192}},
+    # further sizes of the same architecture (layer sizes and vocabulary only; the position encoding
+    # stays the default's, which does not change a step's time): every head with keys of its own,
+    # a feed-forward that is no multiple of 256, and the widest layers of the family, of which
+    # ``--layers`` runs as many as fit beside their tiled copies
+    "7b": {"num_hidden_layers": 32, "hidden_size": 4096, "num_attention_heads": 32, "num_key_value_heads": 32,
+           "head_dim": 128, "intermediate_size": 11008, "vocab_size": 32000, "tie_word_embeddings": False},
+    "13b": {"num_hidden_layers": 40, "hidden_size": 5120, "num_attention_heads": 40, "num_key_value_heads": 40,
+            "head_dim": 128, "intermediate_size": 13824, "vocab_size": 32000, "tie_word_embeddings": False},
+    "70b": {"num_hidden_layers": 80, "hidden_size": 8192, "num_attention_heads": 64, "num_key_value_heads": 8,
+            "head_dim": 128, "intermediate_size": 28672, "tie_word_embeddings": False},
 }
-NAMES = {"1b": "Llama-3.2-1B shape", "3b": "Llama-3.2-3B shape", "8b": "Llama-3.1-8B shape"}
+NAMES = {"1b": "Llama-3.2-1B shape", "3b": "Llama-3.2-3B shape", "8b": "Llama-3.1-8B shape",
+         "7b": "Llama-2-7B sizes", "13b": "Llama-2-13B sizes", "70b": "Llama-3.1-70B sizes"}
 
 
 def log(msg):

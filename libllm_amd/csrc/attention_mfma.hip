@@ -661,7 +661,7 @@ __global__ void attn_decode_combine_loop_kernel(const float* __restrict__ part_o
 }
 
 // ---------------------------------------------------------------------------------- entry points
-#define FOR_HEAD_DIMS(X) X(16) X(32) X(48) X(64) X(80) X(96) X(112) X(128) X(160) X(192) X(256)
+#define FOR_HEAD_DIMS(X) X(16) X(32) X(48) X(64) X(80) X(96) X(112) X(128) X(144) X(160) X(176) X(192) X(208) X(224) X(240) X(256)
 
 extern "C" int llm_attention_mfma_supported(int hd) {
 #define CASE(D) if (hd == D) return 1;
@@ -733,7 +733,7 @@ extern "C" int llm_attention_decode_bf16(const void* q, int q_stride, const void
   const bool ahead = hd <= 128 && (long long)n_blocks * n_kv * n_seqs <= 2LL * llm_compute_units();
 #define CASE(D)                                                                                   \
   if (hd == D) {                                                                                  \
-    constexpr int WAVES = (D > 128) ? 2 : 4;                                                      \
+    constexpr int WAVES = (D > 192) ? 2 : 4;                                                      \
     if (ahead)                                                                                    \
       attn_decode_kernel<D, WAVES, true><<<grid, WAVES * 64, 0, stream>>>(                        \
           (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, table,      \
@@ -770,5 +770,7 @@ extern "C" int llm_attention_decode_bf16(const void* q, int q_stride, const void
   return LLM_ERR_ARG;
 }
 
-// Waves per block of the decode kernel for a head size (the host sizes its grid with it).
-extern "C" int llm_attention_decode_waves(int hd) { return hd > 128 ? 2 : 4; }
+// Waves per block of the decode kernel for a head size (the host sizes its grid with it): four
+// while their partial results fit the 64 KiB of shared memory a block may declare (with two,
+// head sizes 160 and 192 read 3.3 and 2.7 TB/s at batch 64 and 4,096 keys; with four 4.7 and 4.1).
+extern "C" int llm_attention_decode_waves(int hd) { return hd > 192 ? 2 : 4; }

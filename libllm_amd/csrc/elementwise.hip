@@ -164,16 +164,19 @@ extern "C" int llm_add_rmsnorm(float* res, const void* delta, int delta_dtype, i
   if (n_out <= 0) return LLM_OK;
   if (H <= 0 || (delta != nullptr && n_delta < 1)) return LLM_ERR_ARG;
   constexpr int NT = 256;
-  const bool reg = (H % 4 == 0) && H <= NT * 4 * 4 && delta_stride % 4 == 0 &&
+  // rows of up to 16,384 elements stay in registers: 8 or 16 elements a thread, and for rows
+  // beyond 4,096 elements more threads rather than more registers, so that a row's loads are all
+  // asked for at once (a block is all that reads a row, and a compute unit reads slowly alone)
+  const bool reg = (H % 4 == 0) && H <= 1024 * 4 * 4 && delta_stride % 4 == 0 &&
                    ((((uintptr_t)res) | ((uintptr_t)w) | ((uintptr_t)delta) | ((uintptr_t)out)) & 15) == 0;
-  const bool reg2 = reg && H <= NT * 4 * 2;
+#define REG(TD, TO, THREADS, NV)                                                                            \
+    add_rmsnorm_reg_kernel<TD, TO, THREADS, NV><<<n_out, THREADS, 0, stream>>>(                       \
+        res, (const TD*)delta, n_delta, delta_stride, w, eps, (TO*)out, rows, H)
 #define LAUNCH(TD, TO) do {                                                                         \
-  if (reg2)                                                                                         \
-    add_rmsnorm_reg_kernel<TD, TO, NT, 2><<<n_out, NT, 0, stream>>>(res, (const TD*)delta, n_delta, delta_stride, w, eps,  \
-                                                                    (TO*)out, rows, H);             \
-  else if (reg)                                                                                     \
-    add_rmsnorm_reg_kernel<TD, TO, NT, 4><<<n_out, NT, 0, stream>>>(res, (const TD*)delta, n_delta, delta_stride, w, eps,  \
-                                                                    (TO*)out, rows, H);             \
+  if (reg && H <= NT * 4 * 2) REG(TD, TO, NT, 2);                                                           \
+  else if (reg && H <= NT * 4 * 4) REG(TD, TO, NT, 4);                                                      \
+  else if (reg && H <= 512 * 4 * 4) REG(TD, TO, 512, 4);                                                    \
+  else if (reg) REG(TD, TO, 1024, 4);                                                                       \
   else                                                                                              \
     add_rmsnorm_kernel<TD, TO, NT><<<n_out, NT, 0, stream>>>(res, (const TD*)delta, n_delta, delta_stride, w, eps, (TO*)out, rows, H); \
   } while (0)
@@ -184,6 +187,7 @@ extern "C" int llm_add_rmsnorm(float* res, const void* delta, int delta_dtype, i
   else if (delta_dtype == LLM_DTYPE_BF16 && out_dtype == LLM_DTYPE_F32) LAUNCH(bf16_t, float);
   else return LLM_ERR_ARG;
 #undef LAUNCH
+#undef REG
   return llm_launch_status();
 }
 

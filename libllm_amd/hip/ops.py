@@ -129,9 +129,12 @@ class HipOps:
     # against 315, 1,195 against 1,269, and 52 against 55 at 512; 8B: 95 against 112 at 512, 191
     # against 207 at 1,024, the same from 2,048 on).  With half-empty rounds the library's stays
     # (1B, 256 rows: a tile of 128 rows fills half a round, 31 against 33; some such steps would
-    # gain, others lose 10 %).  K beyond WIDE_MAX_K has not been measured.
+    # gain, others lose 10 %).  It gains up to WIDE_MAX_K elements of K (width 5,120, feed-forward
+    # 13,824, whole prompt steps: 10.07 against 10.31 ms at 2,048 rows, 19.65 against 20.85 at 4,096)
+    # and loses beyond (width 8,192, feed-forward 28,672: 16.97 against 16.59 ms and 34.6 against
+    # 33.4), so there the library's stays.
     WIDE_FILL = 0.75
-    WIDE_MAX_K = 4096
+    WIDE_MAX_K = 5120
     # Launch sizes below are in blocks per compute unit; ``__init__`` multiplies them by the
     # device's number of units (the figures in the comments were measured on 256 units).
     MID_BLOCKS_PER_UNIT = 1.0       # blocks that the slices of K of the product for 33 to 128 rows aim at (half and twice as many lose 8 to 10 % of a prompt step of 128 tokens at the 3B and 8B shapes: fewer blocks, or more matrices for the norm to add)

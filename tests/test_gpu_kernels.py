@@ -60,7 +60,9 @@ def test_embed_reference_vector(ops):
 
 # ------------------------------------------------------------------------------- norm
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("width", [10, 11, 192, 2050, 9000])     # 10/11: src/flint/cuda/test.cc:243-248
+# 10/11: src/flint/cuda/test.cc:243-248; rows of up to 2,048, 4,096, 8,192 and 16,384 elements that are a
+# multiple of 4 have a kernel form each, the others the plain one
+@pytest.mark.parametrize("width", [10, 11, 192, 2050, 4096, 5120, 8192, 9000, 16384, 16388, 20002])
 def test_add_rmsnorm(ops, dtype, width):
     m, eps = 7, 1e-5
     res = rnd((m, width), torch.float32, 2, 3.0).cuda()
@@ -78,6 +80,23 @@ def test_add_rmsnorm(ops, dtype, width):
     out = ops.add_rmsnorm(res, None, w, eps, dtype, rows)
     assert torch.equal(res, before)
     assert close(out, ref[rows.long()], dtype)
+
+
+@pytest.mark.parametrize("width", [2048, 5120, 8192, 12000])
+@pytest.mark.parametrize("n_delta", [1, 3, 11])
+def test_add_rmsnorm_of_several_matrices(ops, width, n_delta):
+    """Several float32 matrices are added into the stream in their order, at every form of the kernel."""
+    m = 5
+    res = rnd((m, width), torch.float32, 5, 3.0).cuda()
+    parts = rnd((n_delta, m, width), torch.float32, 6).cuda()
+    w = (1.0 + rnd((width,), torch.float32, 7, 0.3)).cuda()
+    want = res.clone()
+    for j in range(n_delta):
+        want += parts[j]
+    out = ops.add_rmsnorm(res, parts, w, 1e-5, torch.bfloat16)
+    assert torch.equal(res, want)
+    x = want.double()
+    assert close(out, x * w.double() / torch.sqrt((x * x).mean(-1, keepdim=True) + 1e-5), torch.bfloat16)
 
 
 def test_rmsnorm_zero_and_eps(ops):
@@ -585,7 +604,7 @@ def test_gated_products_with_other_activations(ops, activation):
 
 # ---------------------------------------------------------------- the product for many rows
 @pytest.mark.parametrize("block_rows", [256, 128])
-@pytest.mark.parametrize("mnk", [(129, 64, 64), (300, 520, 128), (2048, 512, 256), (257, 1000, 192), (600, 264, 4096),
+@pytest.mark.parametrize("mnk", [(129, 64, 64), (300, 520, 128), (2048, 512, 256), (257, 1000, 192), (600, 264, 4096), (260, 384, 5120),
                                  (300, 268, 128), (129, 100, 64), (513, 4, 64)])
 def test_gemm_wide(ops, mnk, block_rows):
     """Plain, against float64, both sizes of block: rows and weight rows that are no multiples of
@@ -941,7 +960,7 @@ def test_attention_reference_cases(ops, dtype, case):
 
 
 @pytest.mark.parametrize("fast", [True, False])
-@pytest.mark.parametrize("hd", [16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 256, 144])
+@pytest.mark.parametrize("hd", list(range(16, 257, 16)))
 def test_attention_head_sizes_bf16(ops, hd, fast):
     # unequal batch: a fresh prompt, a continued one crossing pages, a single token with a long past
     seqs = [(1, 0, 70), (0, 100, 37), (2, 300, 1)]
@@ -978,7 +997,8 @@ def test_attention_far_key_stands_out(ops, dtype, far):
 
 
 @pytest.mark.parametrize("tiles", [1, 2])
-@pytest.mark.parametrize("hd,window", [(16, 0), (64, 0), (64, 70), (80, 5), (128, 0), (128, 130), (256, 64)])
+@pytest.mark.parametrize("hd,window", [(16, 0), (64, 0), (64, 70), (80, 5), (128, 0), (128, 130), (144, 0), (176, 90),
+                                       (208, 0), (240, 0), (256, 64)])
 def test_prompt_attention_tiles_of_rows(ops, hd, window, tiles):
     """A wave of the prompt kernel takes one or two tiles of 16 rows (blocks of 64 or 128 rows),
     by the number of blocks; here both are forced on small cases: prompts that end inside the first
@@ -1062,10 +1082,11 @@ def test_a_build_whose_product_for_33_to_128_rows_spills_does_not_use_it(monkeyp
     assert not other._mid_ok(x, other.prepare_weight(w), 100, 256)
 
 
-@pytest.mark.parametrize("hd", [160, 192, 256])
+@pytest.mark.parametrize("hd", [144, 160, 176, 192, 208, 224, 240, 256])
 @pytest.mark.parametrize("ctx_len,far", [(600, 3), (2100, 1999), (9000, 77)])
 def test_attention_decode_of_wide_heads_over_many_pages(ops, hd, ctx_len, far):
-    """Heads wider than 128: the decode kernel's form of two waves a block, and each form of the
+    """Heads wider than 128: the decode kernel without its overlap of pages (four waves a block
+    up to head size 192, two beyond), and each form of the
     merge (up to 8 partials, up to 32, and the loop, whose block must stay within 1,024 threads:
     four groups of 192 or 256 threads, not eight).  One far key dominates."""
     out, ref = run_attention(ops, torch.bfloat16, 4, 2, hd, [(0, ctx_len, 1)], seed=hd, boost=(far, 12.0))
