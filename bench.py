@@ -4,7 +4,7 @@ random weights at batch 8 and a context of 4,096 tokens, plus the prefill of 2,0
 decoding at batch 1 and 64.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
-    python bench.py --sweep            # decode at batch 1..128 x context 4,096..131,072, as a table
+    python bench.py --sweep            # decode at batch 1..256 x context 4,096..131,072, as a table
 
 A step is one decode step inside the generation loop (``Generator.stream``, the loop that serves
 requests): the step function over the cache as a captured graph, arg-max sampling on the device,
@@ -227,12 +227,12 @@ def run_workload(args, torch):
     return 0
 
 
-SWEEP_BATCHES = (1, 8, 16, 32, 64, 128)
+SWEEP_BATCHES = (1, 8, 16, 32, 64, 128, 256)
 SWEEP_CONTEXTS = (4096, 16384, 32768, 131072)
 
 
 def run_sweep(args, torch):
-    """Decode steps at batch 1 to 128 and contexts of 4,096 to 131,072 tokens (where the cache fits
+    """Decode steps at batch 1 to 256 and contexts of 4,096 to 131,072 tokens (where the cache fits
     the device), each with its bytes / time against 8 TB/s.  The cache is not filled by prompts
     (at 131,072 tokens a batch that alone would take minutes): the requests are given their pages
     and lengths in the cache's books, the pages hold random values, and the step function decodes
@@ -312,7 +312,7 @@ def main() -> int:
     ap.add_argument("--workload", choices=["unequal16", "batch64"],
                     help="run a generation workload through the generation loop instead")
     ap.add_argument("--sweep", action="store_true",
-                    help="decode steps at batch 1 to 128 and contexts of 4,096 to 131,072 tokens, as a table")
+                    help="decode steps at batch 1 to 256 and contexts of 4,096 to 131,072 tokens, as a table")
     ap.add_argument("--no-workloads", action="store_true",
                     help="skip the generation workloads of the 3B and 8B shapes")
     args = ap.parse_args()

@@ -172,7 +172,8 @@ class Generator:
                     cand = [st for st in live if len(st.output) + 1 < max_new_tokens
                             and st.prompt_len + len(st.output) + 1 < self.max_position]
                     if cand:
-                        rows = pending.rows([live.index(st) for st in cand])
+                        place = {id(st): i for i, st in enumerate(live)}     # (a search per sequence would compare records field by field)
+                        rows = pending.rows([place[id(st)] for st in cand])
                         logits = self.engine.step([StepEntry(name[st.index], [0], [0]) for st in cand],
                                                   tokens_device=rows)
                         queued = (cand, self._draw(logits, params, cand, 1, True))
@@ -192,7 +193,8 @@ class Generator:
                     break
                 if queued is not None:
                     cand, drawn = queued
-                    pending = _Rows(drawn, [cand.index(st) for st in live])
+                    place = {id(st): i for i, st in enumerate(cand)}
+                    pending = _Rows(drawn, [place[id(st)] for st in live])
                 else:
                     logits = self.engine.step([StepEntry(name[st.index], [st.output[-1]], [0])
                                                for st in live])

@@ -30,8 +30,10 @@ class Engine:
 
     # batch sizes the decode graphs are captured for; a step runs in the smallest that holds it, its
     # spare rows pointing at the sink.  With powers of two alone a batch of 40 paid for 64 rows
-    # (2.73 ms a step at the 1B shape against 2.43 in a graph of 48).
-    GRAPH_BATCHES = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64, 80, 96, 112, 128)
+    # (2.73 ms a step at the 1B shape against 2.43 in a graph of 48).  Beyond 256 rows a step is
+    # queued kernel by kernel, which takes the host 4 to 5 ms at the 1B shape: less than the
+    # device needs for that many rows unless the contexts are short.
+    GRAPH_BATCHES = (1, 2, 3, 4, 6, 8, 12, 16, 24, 32, 48, 64, 80, 96, 112, 128, 160, 192, 224, 256)
     GRAPH_MIN_CTX = 1024
     # Steps that bring whole prompts are captured too, padded to one of these numbers of rows and
     # of sequences (one sequence is always spare: it takes the padding rows, in the sink slot).  A

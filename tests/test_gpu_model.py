@@ -779,12 +779,12 @@ def test_library_products_inside_prompt_graphs(rows):
     assert list(engines[0]._prompt_graphs) == [(rows, 2)] and not engines[1]._prompt_graphs
 
 
-@pytest.mark.parametrize("n_prompts", [40, 96])
+@pytest.mark.parametrize("n_prompts", [40, 96, 224])    # 224: a graph of exactly as many rows, so that the library chooses the same product for both engines
 @pytest.mark.parametrize("widths", [(2048, 32, 64, 8192), (4096, 32, 128, 14336)])
 def test_decode_graphs_of_many_rows(widths, n_prompts):
     """From 17 rows on the products that add into the stream are computed over slices of K, which
     the next norm kernel adds; from 33 rows on by the product for 33 to 128 rows where its
-    slices fill the device, beyond 128 by the library's.  Layers of real width: a graph of 48 or 96 rows replayed twelve times, an engine
+    slices fill the device, beyond 128 by the library's.  Layers of real width: a graph of 48, 96 or 224 rows replayed twelve times, an engine
     without graphs stepping beside it, other work and a synchronisation between the replays;
     every replay gives the bits of the eager step."""
     import torch
@@ -813,7 +813,7 @@ def test_decode_graphs_of_many_rows(widths, n_prompts):
             scratch = (scratch @ scratch).clamp_(-1, 1)         # the program's own eager work
             torch.cuda.synchronize()
         assert torch.equal(outs[0], outs[1]), "replay %d differs from the eager step" % k
-    assert [key[0] for key in engines[0]._graphs] == [48 if n_prompts == 40 else 96] and not engines[1]._graphs
+    assert [key[0] for key in engines[0]._graphs] == [{40: 48, 96: 96, 224: 224}[n_prompts]] and not engines[1]._graphs
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
