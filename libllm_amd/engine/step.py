@@ -6,6 +6,7 @@ requests are packed one after another; no padding enters the model.  The referen
 points for one sequence, prefill and decode (src/libllm/llama.cc:349-368); this is their
 generalisation to unequal batches.
 """
+import warnings
 from dataclasses import dataclass, field
 from typing import Dict, Hashable, List, Optional, Sequence
 
@@ -13,7 +14,7 @@ import numpy as np
 import torch
 
 from ..cache import PAGE, SequenceCache
-from ..errors import CacheError, RequestError
+from ..errors import CacheError, ReplayMismatch, RequestError
 from ..parts import StepContext
 from .model import DecoderModel
 
@@ -66,6 +67,7 @@ class Engine:
         self._graphs: Dict[tuple, "_DecodeGraph"] = {}     # (batch bucket, context bucket) -> graph
         self._prompt_graphs: Dict[tuple, "_PromptGraph"] = {}   # (rows, sequences) -> graph
         self._prompt_seen: Dict[tuple, int] = {}
+        self._no_graph = set()         # shapes whose replays did not give the eager step's bits
         self.steps_run = 0
 
     # ---- requests
@@ -145,8 +147,9 @@ class Engine:
         pos0 = [cache.length(s) for s in slots]
         want_all_single = all(n == 1 for n in lens) and all(list(e.want) == [0] for e in entries)
         graph = None
-        if self.use_graphs and want_all_single and len(entries) <= self.GRAPH_BATCHES[-1]:
-            logits = self._graph_step(entries, slots, pos0, tokens_device)
+        if self.use_graphs and want_all_single and len(entries) <= self.GRAPH_BATCHES[-1] \
+                and (graph := self._decode_graph(len(entries), pos0)) is not None:
+            logits = graph.run([e.tokens[0] for e in entries], slots, pos0, tokens_device)
         elif self.use_graphs and tokens_device is None and not all(n == 1 for n in lens) \
                 and (graph := self._prompt_graph(entries, lens)) is not None:
             logits = graph.run(entries, slots, lens, pos0)
@@ -217,6 +220,8 @@ class Engine:
         if rows > min(self.cache.pages_per_seq * PAGE, self.cache.max_position) or wanted > seqs:
             return None
         key = (rows, seqs)
+        if ("prompt",) + key in self._no_graph:
+            return None
         graph = self._prompt_graphs.pop(key, None)
         if graph is None:
             seen = self._prompt_seen.get(key, 0) + 1
@@ -225,13 +230,26 @@ class Engine:
                 return None
             while len(self._prompt_graphs) >= max(1, self.PROMPT_GRAPHS):
                 del self._prompt_graphs[next(iter(self._prompt_graphs))]     # dicts keep the order of insertion
-            graph = _PromptGraph(self, rows, seqs)
+            graph = self._checked(("prompt",) + key, lambda: _PromptGraph(self, rows, seqs))
+            if graph is None:
+                return None
         self._prompt_graphs[key] = graph                                      # the last used lies last
         return graph
 
+    def _checked(self, key, make):
+        """The graph that ``make`` captures, or None if its replays do not give what the same
+        step gives queued kernel by kernel: steps of that shape then run from the host, and a
+        warning says so once."""
+        try:
+            return make()
+        except ReplayMismatch as e:
+            self._no_graph.add(key)
+            warnings.warn("libllm_amd: %s; steps of this shape run without a captured graph" % e)
+            return None
+
     # ---- decoding one token per sequence through a captured graph
-    def _graph_step(self, entries, slots, pos0, tokens_device=None):
-        b = len(entries)
+    def _decode_graph(self, b, pos0):
+        """The captured graph for a decode step of ``b`` sequences, or None if there is none."""
         bucket = next(g for g in self.GRAPH_BATCHES if g >= b)
         # the longest context a graph serves is part of its key: kernels size their grids by it
         limit = self.cache.pages_per_seq * PAGE
@@ -239,11 +257,13 @@ class Engine:
         while ctx_bucket < max(pos0) + 1:
             ctx_bucket *= 2
         ctx_bucket = min(ctx_bucket, limit)
-        graph = self._graphs.get((bucket, ctx_bucket))
-        if graph is None:
-            graph = _DecodeGraph(self, bucket, ctx_bucket)
-            self._graphs[(bucket, ctx_bucket)] = graph
-        return graph.run([e.tokens[0] for e in entries], slots, pos0, tokens_device)
+        key = (bucket, ctx_bucket)
+        graph = self._graphs.get(key)
+        if graph is None and ("decode",) + key not in self._no_graph:
+            graph = self._checked(("decode",) + key, lambda: _DecodeGraph(self, bucket, ctx_bucket))
+            if graph is not None:
+                self._graphs[key] = graph
+        return graph
 
 
 class _CapturedForward:
@@ -256,10 +276,33 @@ class _CapturedForward:
     fixed addresses; what a host-run unit returns lies somewhere new each time and is copied to
     a buffer that the next captured stretch was captured with (a prepared norm that such a unit
     may leave is dropped: the next norm then works from the sum itself).  The state of the stream
-    object at every border is kept from set-up, since a replayed graph runs no Python."""
+    object at every border is kept from set-up, since a replayed graph runs no Python.
 
-    def __init__(self, model, ops, ctx, want_rows):
+    With ``check``, the captured step is replayed ``CHECK_REPLAYS`` times over the buffers it was
+    captured with before it serves, and must give, every time, the logits that the same step gave
+    queued kernel by kernel, or ReplayMismatch is raised: work may be recorded into a graph that
+    does not replay (see ``HipOps.capture``).  This asks for a step that gives the same bits
+    whenever it runs: a decode step of padding alone does (every row is the same token at
+    position 0 of the sink slot), a prompt step of padding alone does not (its rows a page apart
+    write to the same places of the sink page), and a model whose parts keep state of their own
+    per sequence does not either, since running a step again moves that state on."""
+
+    CHECK_REPLAYS = 2
+
+    def __init__(self, model, ops, ctx, want_rows, check=False):
         self.model, self.ctx, self.want_rows = model, ctx, want_rows
+        self.stream = self.logits = None
+        reference = None
+        check = check and self.CHECK_REPLAYS > 0 and all(need is None for need in model.state_needs())
+        if check:
+            # the same step from the host, cut where the captured one is cut: after a stretch
+            # that runs from the host the next norm works from the sum itself, here too
+            for safe, units in model.stretches():
+                self._run(units)
+                if not safe:
+                    self.stream.pre = None
+            reference = None if self.logits is None else self.logits.clone()
+            self.stream = self.logits = None
         self.pieces = []                 # (graph or None, units, border state after the piece)
         self.stream = None
         self.logits = None
@@ -282,6 +325,18 @@ class _CapturedForward:
         self.n_graphs = sum(1 for g, _, _ in self.pieces if g is not None)
         self.n_host_pieces = len(self.pieces) - self.n_graphs
         self.last_unit = last
+        if check and self.n_graphs:
+            for replay in range(self.CHECK_REPLAYS):
+                if not self._same(self.run(), reference):
+                    raise ReplayMismatch("replay %d of a captured step of %d rows differs from the step queued "
+                                         "kernel by kernel" % (replay + 1, ctx.n_tokens))
+
+    @staticmethod
+    def _same(out, reference) -> bool:
+        if out is None or reference is None:
+            return out is None and reference is None
+        # bit for bit, so that a NaN equals itself
+        return out.shape == reference.shape and torch.equal(out.view(torch.int32), reference.view(torch.int32))
 
     def _run(self, units, before=None):
         if before is not None:
@@ -353,7 +408,7 @@ class _DecodeGraph:
         engine._attach_cache(ctx)
         self.ctx = ctx
         self._fill([0] * b, [engine.cache.sink_slot] * b, [0] * b)
-        self.forward = _CapturedForward(self.model, ops, ctx, self.want_rows)
+        self.forward = _CapturedForward(self.model, ops, ctx, self.want_rows, check=True)
 
     def _fill(self, tokens, slots, pos0):
         b = self.bucket

@@ -23,3 +23,7 @@ class KernelError(LlmError):
 
 class RequestError(LlmError):
     """A step or generation request that the engine cannot run (bad token id, empty prompt)."""
+
+
+class ReplayMismatch(LlmError):
+    """Work recorded into a graph did not, replayed, give the bits it gives when queued directly."""

@@ -15,7 +15,7 @@ import numpy as np
 import torch
 
 from ..parts.kv_pages import K_LAYOUT, V_LAYOUT, key_pages_shape, value_pages_shape
-from ..errors import KernelError
+from ..errors import KernelError, ReplayMismatch
 from . import build
 
 _F32, _BF16 = 0, 1
@@ -188,6 +188,7 @@ class HipOps:
         self.fold_norms = True          # up to ACCUM_ROWS rows, a norm between two products gets no kernel of its own
         self.prompt_tiles = 0           # tiles of rows a wave of prompt attention takes (1 or 2; 0: by the number of blocks)
         self.timing = False
+        self._warming = False           # inside the run that precedes a capture
         if os.environ.get("LIBLLM_AMD_TIME", "") not in ("", "0"):
             self.start_timing()
 
@@ -270,7 +271,9 @@ class HipOps:
         return host.to(self.device, non_blocking=True)
 
     def capture(self, body):
-        """Runs ``body`` once to warm up, then captures it into a HIP graph.
+        """Runs ``body`` once to warm up, then captures it into a HIP graph.  A product of the
+        vendor library that ``body`` holds is first tried alone (``_library_product``); if it
+        does not replay, ReplayMismatch is raised and nothing is captured.
 
         The capture is in global mode: runtime calls that free or query device resources are
         errors anywhere in the process while it lasts, and a finaliser that makes one (of a graph,
@@ -278,8 +281,12 @@ class HipOps:
         collector goes before the capture begins, and the collector does not run during it."""
         side = torch.cuda.Stream(self.device)
         side.wait_stream(torch.cuda.current_stream(self.device))
-        with torch.cuda.stream(side):
-            body()
+        warming, self._warming = self._warming, True
+        try:
+            with torch.cuda.stream(side):
+                body()
+        finally:
+            self._warming = warming
         torch.cuda.current_stream(self.device).wait_stream(side)
         torch.cuda.synchronize(self.device)
         gc.collect()
@@ -559,7 +566,7 @@ class HipOps:
             self._check(self.lib.llm_gemm_f32(xf.data_ptr(), w.data_ptr(), out.data_ptr(), m, n, k,
                                               self._stream()), "gemm_f32")
         elif w.dtype == torch.bfloat16 and x.dtype == torch.bfloat16:
-            out = torch.matmul(x, w.t())
+            out = self._library_product(x, w)
         else:
             raise KernelError("linear: input %s with weight %s is not supported" % (x.dtype, w.dtype))
         if bias is not None:
@@ -567,6 +574,45 @@ class HipOps:
             self._check(self.lib.llm_add_bias(out.data_ptr(), _code(out.dtype), bias.data_ptr(), m, n,
                                               self._stream()), "add_bias")
         return out if out.dtype == out_dtype else out.to(out_dtype)
+
+    REPLAY_TRIALS = 3
+    _replayable = {}                # (device, shape of a library product) -> whether it replays from a graph; one for the process
+
+    def _library_product(self, x, w):
+        """x W^T by the vendor library.  The library chooses a kernel by the shape, and some of
+        its kernels clear a scratch buffer first by a fill that, recorded into a graph, has been
+        seen here to take effect on the first replay only.  So the first time a shape is about
+        to be captured (in the run that precedes the capture) the product alone is recorded
+        into a graph of its own and replayed ``REPLAY_TRIALS`` times over new rows, with the
+        same product queued directly beside it; a shape whose replays differ by one bit raises
+        ReplayMismatch, now and whenever it is about to be captured again."""
+        if self._warming and not torch.cuda.is_current_stream_capturing():
+            key = (x.shape[0], w.shape[0], w.shape[1], x.stride(0), w.stride(0), self.device.index or 0)
+            if key not in self._replayable:
+                self._replayable[key] = self._product_replays(x, w)
+            if not self._replayable[key]:
+                raise ReplayMismatch("the library's product of %d x %d rows over %d elements does not replay from a "
+                                     "captured graph" % key[:3])
+        return torch.matmul(x, w.t())
+
+    def _product_replays(self, x, w) -> bool:
+        rows = torch.empty_strided(x.shape, x.stride(), dtype=x.dtype, device=self.device).normal_()
+        held = {}
+
+        def body():
+            held["out"] = torch.matmul(rows, w.t())
+        warming, self._warming = self._warming, False        # (the capture below warms up too)
+        try:
+            graph = self.capture(body)
+        finally:
+            self._warming = warming
+        same = True
+        for trial in range(self.REPLAY_TRIALS):
+            rows.normal_()
+            direct = torch.matmul(rows, w.t())
+            graph.replay()
+            same = same and torch.equal(held["out"].view(torch.int16), direct.view(torch.int16))
+        return same
 
     def _act(self, activation):
         if activation not in self.ACTIVATIONS:

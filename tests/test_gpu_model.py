@@ -561,6 +561,64 @@ def test_steps_seen_before_ask_the_device_for_no_memory(models, use_graphs, dtyp
     assert bool(engine._graphs) == use_graphs and bool(engine._prompt_graphs) == use_graphs
 
 
+def test_a_captured_step_whose_replay_differs_is_not_used(models, monkeypatch):
+    """A captured decode step is replayed twice before it serves and compared, bit for bit, with
+    the same step queued kernel by kernel (work may be recorded that does not replay).  Here the
+    comparison is made to fail: the engine warns, keeps no graph for that shape, and its steps
+    give what an engine without graphs gives."""
+    from libllm_amd.engine import step as step_mod
+    from libllm_amd.runtime import load_engine
+    path, cfg, _ = models["A"]
+    requests = make_requests(cfg, [9, 70, 31], seed=5)
+    plain_path = load_engine(path, dtype="bfloat16", max_tokens=1024, use_graphs=False)
+    want = _decode_rows(plain_path, requests, 4)
+    checked = load_engine(path, dtype="bfloat16", max_tokens=1024)
+    assert np.array_equal(_decode_rows(checked, requests, 4), want) and checked._graphs and not checked._no_graph
+    calls = []
+    monkeypatch.setattr(step_mod._CapturedForward, "_same", staticmethod(lambda out, ref: bool(calls.append(1))))
+    engine = load_engine(path, dtype="bfloat16", max_tokens=1024)
+    with pytest.warns(UserWarning, match="run without a captured graph"):
+        got = _decode_rows(engine, requests, 4)
+    assert len(calls) == 1 and not engine._graphs
+    assert engine._no_graph == {("decode", 3, 128)}         # (the position limit of this configuration is 128)
+    assert np.array_equal(got, want)
+
+
+def test_a_library_product_that_does_not_replay_is_not_captured(models, monkeypatch):
+    """Before a product of the vendor library is recorded into a graph, its shape is tried alone:
+    recorded, replayed over new rows and compared with the product queued directly.  Shapes that
+    pass are remembered; here the trial is then made to fail, and the prompt step that holds such
+    a product runs without a graph, with a warning, and gives the same logits."""
+    from libllm_amd.engine import StepEntry
+    from libllm_amd.hip.ops import HipOps
+    from libllm_amd.runtime import load_engine
+    path, cfg, _ = models["C"]
+    prompt = make_requests(cfg, [150], seed=8)["r0"]
+
+    def logits(engine):
+        engine.PROMPT_SEEN = 1
+        out = []
+        for k in range(3):
+            out.append(engine.step([StepEntry("p", prompt, [len(prompt) - 1])]).cpu().numpy().copy())
+            engine.end(["p"])
+        assert all(np.array_equal(o, out[0]) for o in out)
+        return out[0]
+
+    engine = load_engine(path, dtype="bfloat16", max_tokens=1024)
+    monkeypatch.setattr(HipOps, "_replayable", {})
+    want = logits(engine)
+    assert list(engine._prompt_graphs) == [(176, 2)]
+    tried = engine.ops._replayable
+    assert tried and all(tried.values()) and all(key[0] == 176 for key in tried)
+    monkeypatch.setattr(HipOps, "_replayable", {})
+    monkeypatch.setattr(HipOps, "_product_replays", lambda self, x, w: False)
+    other = load_engine(path, dtype="bfloat16", max_tokens=1024)
+    with pytest.warns(UserWarning, match="does not replay from a captured graph"):
+        got = logits(other)
+    assert not other._prompt_graphs and other._no_graph == {("prompt", 176, 2)}
+    assert np.array_equal(got, want)
+
+
 @pytest.mark.parametrize("name", list(CONFIGS))
 def test_norms_between_products_get_no_kernel(models, name):
     """Decoding up to 16 rows in bfloat16, the product that adds into the stream prepares the RMS
