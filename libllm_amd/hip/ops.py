@@ -510,11 +510,18 @@ class HipOps:
             return self._mid(x, w, torch.empty((ks, m, n), dtype=torch.float32, device=self.device),
                              self._EPI_NONE, ks)
         if (self.MID_HEAD and out_dtype == torch.float32 and residual is None and bias is None
-                and self.SKINNY_ROWS < m and self._mid_ok(x, w, m, k)):
+                and self.SKINNY_ROWS < m and not lazy):
             # float32 results (logits) for 65 to 128 rows in one pass over the weight, where the
-            # product for few rows would take two
-            return self._mid(x, w, torch.empty((1, m, n), dtype=torch.float32, device=self.device),
-                             self._EPI_NONE, 1)[0]
+            # product for few rows would take two, and for more rows in passes of up to 128
+            passes = -(-m // self.MID_ROWS)
+            # the rows dealt out evenly, each pass starting at a multiple of 16 rows (which keeps
+            # its rows of the result aligned): passes of 49 to 128 rows
+            cuts = [min(m, -(-(i * m) // (passes * 16)) * 16) for i in range(passes)] + [m]
+            if self._mid_ok(x[:cuts[1]], w, cuts[1], k):
+                out = torch.empty((m, n), dtype=torch.float32, device=self.device)
+                for m0, m1 in zip(cuts, cuts[1:]):
+                    self._mid(x[m0:m1], w, out[m0:m1].view(1, m1 - m0, n), self._EPI_NONE, 1)
+                return out
         if (self._skinny_ok(x, w, m, k) and bias is None and residual is not None
                 and self.ACCUM_ROWS < m <= self.SPLIT_ROWS and (ks := self._k_split(n, k)) > 1):
             # K in slices, one block for 64 rows of the weight and a slice: each slice of X is staged

@@ -534,6 +534,32 @@ def test_logits_of_65_to_128_rows_take_one_pass(ops):
     assert torch.equal(ops.linear(lazy, w, None, torch.float32), ops.linear(rows, w, None, torch.float32))
 
 
+@pytest.mark.parametrize("n", [1000, 517])
+def test_float32_results_of_many_rows_in_passes(ops, n):
+    """Logits (float32, no residual) of 65 rows and more go through the product for 33 to 128
+    rows, in one pass up to 128 rows and in even passes beyond; a row's bits do not depend on
+    how many rows there are, nor on the pass it falls into.  A vocabulary that is no multiple of
+    4 has rows that are not 16 bytes apart: every pass still starts at an aligned row."""
+    k = 256
+    x = rnd((1100, k), torch.bfloat16, 21).cuda()
+    w = ops.prepare_weight(rnd((n, k), torch.bfloat16, 22, scale=0.05).cuda())
+    ref = x.double() @ w.w.double().t()
+    calls = []
+    real = ops._mid
+    ops._mid = lambda *a, **kw: calls.append(a[0].shape[0]) or real(*a, **kw)
+    try:
+        full = ops.linear(x, w, None, torch.float32)
+        assert sum(calls) == 1100 and len(calls) == 9 and all(49 <= c <= 128 for c in calls)
+        assert full.dtype == torch.float32 and close(full, ref, torch.float32)
+        for m in (65, 128, 129, 255, 257, 1000):
+            del calls[:]
+            part = ops.linear(x[:m], w, None, torch.float32)
+            assert sum(calls) == m and len(calls) == -(-m // 128)
+            assert torch.equal(part, full[:m])
+    finally:
+        ops._mid = real
+
+
 def test_gemm_mid_refuses(ops):
     from libllm_amd.errors import KernelError
     w = ops.prepare_weight(rnd((64, 256), torch.bfloat16, 1).cuda())
