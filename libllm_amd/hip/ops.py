@@ -119,7 +119,7 @@ class HipOps:
     # 48 and 64: 2.04 against 2.09 and 2.38 against 2.46 ms at the 1B shape, 4.02 against 4.11 and
     # 4.69 against 4.83 at 3B, 5.58 against 5.74 and 6.17 against 6.45 at 8B).
     MID_FROM = 33
-    MID_HEAD = True         # logits of 65 to 128 rows by it too
+    MID_HEAD = True         # logits of 65 rows and more by it too (beyond 128 rows in passes)
     # Beyond MID_ROWS rows the gate/up product with its SwiGLU is a kernel of ours where its tiles
     # (256 or 128 rows by 128 outputs) would be filled, over whole rounds of the compute units, to
     # at least WIDE_FILL: there it beats the library's product followed by the SiLU-mul kernel, which reads
