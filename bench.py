@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Serving benchmark on one MI355X: decoded tokens a second of a Llama-3.2-1B-shaped model with
 random weights at batch 8 and a context of 4,096 tokens, plus the prefill of 2,048 tokens and
-decoding at batch 1 and 64.
+decoding at batch 1, 64 and 256.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
     python bench.py --sweep            # decode at batch 1..256 x context 4,096..131,072, as a table
@@ -306,7 +306,7 @@ def main() -> int:
     ap.add_argument("--context", type=int, default=4096)
     ap.add_argument("--prefill", type=int, default=2048)
     ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
-    ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1 and 64")
+    ap.add_argument("--no-points", action="store_true", help="skip decoding at batch 1, 64 and 256")
     ap.add_argument("--sampling", default="greedy", choices=["greedy", "default"],
                     help="greedy, or the command line's default (temperature 1, top-k 50, top-p 0.8)")
     ap.add_argument("--workload", choices=["unequal16", "batch64"],
@@ -342,7 +342,10 @@ def main() -> int:
     cfg = config_from_dict(d)
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     itemsize = 2 if short == "bf16" else 4
-    biggest = max(args.batch, 1 if args.no_points else 64)
+    # decoding is also measured at batch 1 and 64, and at 256 (the largest captured graph) where
+    # the cache for that is small beside the device's memory
+    point_batches = () if args.no_points else ((1, 64, 256) if args.shape == "1b" else (1, 64))
+    biggest = max((args.batch,) + point_batches)
     max_tokens = biggest * (args.context + 64) + 4096
     log("building %d layers of %d with random weights, cache for %d tokens" %
         (args.layers, layers_full, max_tokens))
@@ -369,8 +372,8 @@ def main() -> int:
 
     flops_measured = (peaks["bf16_TFs"] if short == "bf16" else peaks["fp32_TFs"]) * 1e12
     points = {}
-    if not args.no_points:
-        for b in (1, 64):
+    if point_batches:
+        for b in point_batches:
             dtb = time_decode(gen, params, torch, b, args.context, args.steps, args.warmup, vocab)
             points["decode_b%d" % b] = round(b * args.steps / dtb, 1)
             bytes_b = weight_bytes(cfg, itemsize) + b * mean_ctx * kv_bytes_per_token(cfg, itemsize)
