@@ -96,16 +96,29 @@ class Stream:
 
     def __init__(self, res: torch.Tensor):
         self.res = res            # [tokens, width] float32
-        self.delta = None         # [tokens, width] in the activation dtype, or None
+        self.delta = None         # what is still to be added: [tokens, width], or [n, tokens, width] float32, or None
         self.pre = None           # what a product that added into ``res`` has left for the next norm
 
     def put(self, out) -> None:
-        """Takes what a mixer or feed-forward returned: rows still to be added (a matrix), None
-        (it added them itself), or the record ``ops.linear(..., then_norm=)`` returned when it
-        added them and prepared the norm that comes next."""
+        """Takes what a mixer or feed-forward returned: rows still to be added (a matrix in the
+        activation dtype, or a stack ``[n, tokens, width]`` of float32 matrices that are added
+        one after another, in their order: the slices of K of a product, or the results of two
+        parts that read the same rows), None (it added them itself), or the record
+        ``ops.linear(..., then_norm=)`` returned when it added them and prepared the norm that
+        comes next."""
         is_rows = out is None or isinstance(out, torch.Tensor)
         self.delta = out if is_rows else None
         self.pre = None if is_rows else out
+
+    def settle(self) -> torch.Tensor:
+        """Adds what is still to be added into the 32-bit sum, in the order the norm kernel
+        adds it, and returns the sum: for a norm that has no kernel which adds and normalises
+        in one pass (the RMS norm's does)."""
+        delta, self.delta, self.pre = self.delta, None, None
+        if delta is not None:
+            for part in (delta if delta.dim() == 3 else [delta]):
+                self.res.add_(part)
+        return self.res
 
 
 class StepContext:

@@ -23,7 +23,8 @@ class CpuOps:
 
     def add_rmsnorm(self, res, delta, weight, eps, out_dtype, rows=None):
         if delta is not None:
-            res += delta.float()
+            for part in (delta if delta.dim() == 3 else [delta]):      # a stack is added in its order
+                res += part.float()
         x = res if rows is None else res[rows.long()]
         inv = torch.rsqrt((x * x).mean(dim=-1, keepdim=True) + eps)
         return (x * weight * inv).to(out_dtype)

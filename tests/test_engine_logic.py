@@ -199,6 +199,25 @@ def test_toy_mixer_with_a_plane_of_its_own_and_toy_input_layer():
     assert all(g.pool.n_free == g.pool.n_pages for g in engine.cache.groups)
 
 
+def test_toy_norm_and_toy_block_arrangement():
+    """A norm of another kind and another arrangement of a block (one norm, mixer and
+    feed-forward side by side), both defined in tests/toy.py and chosen in the model's record:
+    whole prompts and cut ones agree with their restatement."""
+    cfg_t = config_from_dict(TINY_A)
+    cfg = llama.PlainConfig(TINY_A)
+    engine, w = build(toy.arrangement_spec(cfg_t), 13, CpuOps())
+    declared = engine.model.declared()
+    assert "model.layers.1.ln_a.bias" in declared and "model.layers.0.post_attention_layernorm.weight" not in declared
+    ids = np.random.default_rng(3).integers(0, 256, size=100).tolist()
+    ref = toy.arrangement_oracle(cfg, w, ids)
+    whole = engine.step([StepEntry("a", ids, list(range(100)))])
+    engine.end(["a"])
+    cut = torch.cat([engine.step([StepEntry("b", ids[:70], list(range(70)))])] +
+                    [engine.step([StepEntry("b", [t], [0])]) for t in ids[70:]])
+    engine.end(["b"])
+    assert err(whole.double().numpy(), ref) < 1e-4 and err(cut.double().numpy(), ref) < 1e-4
+
+
 def test_a_dropped_engine_goes_at_once(models):
     """Nothing an engine owns refers back to it, so dropping it frees it there and then, without
     the collector of cycles (which may run at any later time, for instance while a graph is being

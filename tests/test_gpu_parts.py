@@ -233,6 +233,47 @@ def test_toy_routed_feed_forward_and_position_encoding(ops, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+def test_toy_norm_and_toy_block_arrangement(ops, dtype):
+    """A norm of another kind (mean taken out, a bias) and another arrangement of a block (one
+    norm whose rows the mixer and the feed-forward both read, their results handed to the stream
+    as two float32 matrices), both defined in tests/toy.py and chosen in the model's record.  The
+    layer arranged in parallel is captured with its neighbours; the layer with the toy norm,
+    which works through library calls, runs from the host between the graphs.  Whole prompts,
+    cut ones, and batches of unequal lengths agree with the restatement."""
+    cfg = llama.PlainConfig(TINY_A)
+    model = DecoderModel(toy.arrangement_spec(config_from_dict(TINY_A)))
+    t = random_tensors(model.declared(), 13, std=0.1, norm_std=0.2)
+    model.bind({k: v.to("cuda", torch.float32 if (dtype == torch.float32 or v.dim() == 1) else dtype)
+                for k, v in t.items()}, ops, dtype)
+    engine = Engine(model, ops, dtype, max_tokens=512)
+    engine.PROMPT_SEEN = 1
+    assert engine.use_graphs and [(safe, units) for safe, units in model.stretches()] == [
+        (True, [0, 1]), (False, [2]), (True, [3])]
+    w = {k: v.double().numpy() for k, v in t.items()}
+    ids = np.random.default_rng(3).integers(0, 256, size=100).tolist()
+    ref = toy.arrangement_oracle(cfg, w, ids)
+    whole = engine.step([StepEntry("a", ids, list(range(100)))]).double().cpu().numpy()
+    engine.end(["a"])
+    cut = torch.cat([engine.step([StepEntry("b", ids[:70], list(range(70)))]).clone()] +
+                    [engine.step([StepEntry("b", [x], [0])]).clone() for x in ids[70:]]).double().cpu().numpy()
+    engine.end(["b"])
+    assert_logits_close(whole, ref, dtype, "whole")
+    assert_logits_close(cut, ref, dtype, "cut")
+    # two requests of unequal lengths in one batch, their last rows through a captured prompt step
+    short = ids[:23]
+    out = engine.step([StepEntry("c", ids[:60], [59]), StepEntry("d", short, [22])]).double().cpu().numpy()
+    assert_logits_close(out[:1], ref[59:60], dtype, "c")
+    assert_logits_close(out[1:], toy.arrangement_oracle(cfg, w, short)[22:], dtype, "d")
+    nxt = engine.step([StepEntry("c", [ids[60]], [0]), StepEntry("d", [ids[23]], [0])]).double().cpu().numpy()
+    assert_logits_close(nxt[:1], ref[60:61], dtype, "c next")
+    engine.end(["c", "d"])
+    engine.cache.check()
+    assert engine._graphs and engine._prompt_graphs
+    graphs = list(engine._graphs.values()) + list(engine._prompt_graphs.values())
+    assert all(g.forward.n_graphs == 2 and g.forward.n_host_pieces == 1 for g in graphs)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 def test_toy_mixer_with_a_plane_of_its_own_and_toy_input_layer(ops, dtype):
     """A mixer that keeps one latent row a token in the cache's pages, in a plane of its own
     width and element type instead of keys and values, and an input layer with learned positions:

@@ -335,3 +335,88 @@ def planes_oracle(cfg, weights, ids, latent=8):
     for layer in range(1, cfg.n_layers):
         x = llama.decode_layer(cfg, weights, layer, x, positions)
     return llama.lm_head(cfg, weights, llama.rms_norm(x, weights["model.norm.weight"], cfg.eps))
+
+
+# ---------------------------------------------------------------------------------------------
+# A norm of another kind (mean taken out, a bias added) and another arrangement of a block (the
+# mixer and the feed-forward read the same normalised rows, one norm a block).
+from libllm_amd.parts import Block, Norm, register_block, register_norm  # noqa: E402
+
+
+@dataclass
+class CenteredNormSpec(PartSpec):
+    width: int = 0
+    eps: float = 0.0
+
+
+@register_norm("centered")
+class CenteredNorm(Norm):
+    """y = (x - mean(x)) * rsqrt(var(x) + eps) * weight + bias, in 32-bit, by library calls: it
+    runs from the host, between the captured stretches of its neighbours."""
+    graph_safe = False
+
+    def __init__(self, spec: CenteredNormSpec):
+        self.width, self.eps = spec.width, float(spec.eps)
+
+    def weights(self):
+        return {"weight": WeightDecl((self.width,), role="vector", init="ones"),
+                "bias": WeightDecl((self.width,), role="vector", init="normal")}
+
+    def bind(self, tensors, ops, dtype):
+        self.weight, self.bias = tensors["weight"].float(), tensors["bias"].float()
+
+    def add_norm(self, ctx, stream, rows=None, lazy=False):
+        x = stream.settle()
+        if rows is not None:
+            x = x[rows.long()]
+        x = x - x.mean(-1, keepdim=True)
+        return (x * torch.rsqrt((x * x).mean(-1, keepdim=True) + self.eps) * self.weight + self.bias).to(ctx.dtype)
+
+
+@register_block("parallel")
+class ParallelBlock(Block):
+    """x += mixer(norm(x)) + feed_forward(norm(x)): one norm, both parts read its rows, and their
+    results go to the stream as two float32 matrices that the next norm adds in 32-bit."""
+
+    def __init__(self, mixer, feed_forward, norms):
+        assert len(norms) == 1
+        super().__init__(mixer, feed_forward, norms)
+
+    def entry_norm(self):
+        return self.norms[0]
+
+    def forward(self, ctx, stream, entry):
+        h = self.norms[0].add_norm(ctx, stream)
+        mixed = self.mixer.forward(ctx, h, entry)
+        fed = self.feed_forward.forward(ctx, h)
+        stream.put(torch.stack([mixed.float(), fed.float()]))
+
+
+def arrangement_spec(base_config, eps=1e-3):
+    """The Llama model as data with layer 0 arranged in parallel around its first RMS norm, and
+    layer 1's two norms replaced by the centered one."""
+    spec = base_config.to_spec()
+    first, second = spec.layers[0], spec.layers[1]
+    first.block, first.norms = "parallel", first.norms[:1]
+    del first.prefixes["norm1"]
+    second.norms = [CenteredNormSpec(kind="centered", width=spec.width, eps=eps) for _ in range(2)]
+    second.prefixes["norm0"], second.prefixes["norm1"] = "model.layers.1.ln_a.", "model.layers.1.ln_b."
+    return spec
+
+
+def arrangement_oracle(cfg, weights, ids, eps=1e-3):
+    """The same model through the plain functions, the two toys restated in numpy."""
+    import numpy as np
+
+    from plain import llama
+    positions = np.arange(len(ids))
+    x = llama.embedding(weights["model.embed_tokens.weight"], ids)
+    h = llama.rms_norm(x, weights["model.layers.0.input_layernorm.weight"], cfg.eps)
+    x = x + llama.attention_block(cfg, weights, 0, h, positions) + llama.mlp(cfg, weights, 0, h)
+
+    def centered(x, name):
+        c = x - x.mean(-1, keepdims=True)
+        return c / np.sqrt((c * c).mean(-1, keepdims=True) + eps) * weights[name + "weight"] + weights[name + "bias"]
+    x = x + llama.attention_block(cfg, weights, 1, centered(x, "model.layers.1.ln_a."), positions)
+    x = x + llama.mlp(cfg, weights, 1, centered(x, "model.layers.1.ln_b."))
+    return llama.lm_head(cfg, weights, llama.rms_norm(x, weights["model.norm.weight"], cfg.eps))
