@@ -278,6 +278,25 @@ def test_random_traces(long_models, tmp_path, case):
     check("long" + name, cfg, weights, requests, traces.collect(steps, str(tmp_path), cfg.vocab), dtype)
 
 
+@pytest.mark.parametrize("case", range(6))
+def test_batches_of_more_than_128_requests(long_models, tmp_path, case):
+    """160 to 250 short requests start together and decode a few tokens each, the shorter ones
+    ending earlier: the decode graphs of 160 to 256 rows and those below as the batch thins out
+    (the last two cases without graphs), every position against the plain implementation."""
+    name, dtype, use_graphs = "ABC"[case % 3], DTYPES[case % 2], case < 4
+    path, cfg, weights = long_models[name]
+    rng = np.random.default_rng(5000 + case)
+    n = [250, 170, 200, 161, 250, 160][case]
+    group = {"q%d" % i: rng.integers(0, cfg.vocab, size=int(rng.integers(1, 40))).tolist() for i in range(n)}
+    tails = {r: int(rng.integers(1, 12)) if len(t) > 12 else int(rng.integers(0, len(t))) for r, t in group.items()}
+    steps = traces.batches([group], tails)
+    for i, s in enumerate(steps):
+        s["step"] = i
+    engine = run_replay(path, dtype, steps, tmp_path, max_tokens=traces.max_tokens_needed(steps), use_graphs=use_graphs)
+    assert (max(k[0] for k in engine._graphs) > 128) if use_graphs else not engine._graphs
+    check("long" + name, cfg, weights, group, traces.collect(steps, str(tmp_path), cfg.vocab), dtype)
+
+
 BENCH_SHAPES = {
     "1b": dict(hidden_size=2048, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
                intermediate_size=8192, tie_word_embeddings=True, factor=32.0),
