@@ -74,6 +74,28 @@ def test_greedy_generation_of_a_wide_batch(model_b):
     assert model.engine.cache.slots.n_free == model.engine.cache.slots.n_slots
 
 
+def test_greedy_generation_of_two_hundred_requests_with_stop_tokens(model_b):
+    """Two hundred requests at once, in 32-bit, a tenth of the vocabulary being stop tokens: the
+    sequences end at all times, so that the batch thins from a graph of 224 rows down, and the
+    step that is queued ahead carries other rows than the tokens drawn before it.  Every seventh
+    request as the plain implementation generates it alone."""
+    from libllm_amd import Device, Model
+    path, cfg, weights = model_b
+    rng = np.random.default_rng(19)
+    prompts = [rng.integers(10, cfg.vocab, size=int(n)).tolist() for n in rng.integers(1, 12, size=200)]
+    stop = sorted(set(rng.integers(0, cfg.vocab, size=cfg.vocab // 10).tolist()))
+    model = Model(path, Device.AUTO, dtype="float32", max_tokens=200 * 64, max_batch=200)
+    got = model.generate(prompts, max_new_tokens=16, temperature=0.0, stop_tokens=stop)
+    buckets = sorted(k[0] for k in model.engine._graphs)
+    assert buckets[-1] == 224 and len(buckets) >= 4
+    lengths = sorted(len(g) for g in got)
+    assert lengths[0] < 4 and lengths[-1] == 16            # some end early, some run to the limit
+    for p, g in zip(prompts[::7], got[::7]):
+        assert g == sampling.generate(cfg, weights, p, 16, stop=stop)
+    model.engine.cache.check()
+    assert model.engine.cache.slots.n_free == model.engine.cache.slots.n_slots
+
+
 def test_sampled_generation_and_stop_tokens(model_b):
     from libllm_amd import Model
     path, cfg, weights = model_b
