@@ -121,6 +121,25 @@ def test_gemm_f32(ops, mnk):
     assert max_err(out, ref) < 2e-6
 
 
+@pytest.mark.parametrize("nk", [(1000, 2050), (37, 8200), (2048, 4096), (70, 17), (16, 64), (17, 65), (5, 3)])
+def test_gemm_f32_of_few_rows_gives_the_same_bits(ops, nk):
+    """Up to 16 rows go through a kernel of their own (16 rows of the weight a block, 64 elements
+    of K between barriers, 16 bytes a load where K and the addresses allow): it adds the terms in
+    the order of the kernel for many rows, so a row's bits do not depend on how many rows a step
+    has.  K that is no multiple of 4, of 16 or of 64; weights of fewer than 16 rows; a view whose
+    rows do not start at 16 bytes."""
+    n, k = nk
+    x = rnd((40, k), torch.float32, 15).cuda()
+    w = rnd((n, k), torch.float32, 16).cuda()
+    many = ops.linear(x, w, None, torch.float32)                 # 40 rows: the kernel for many rows
+    assert max_err(many, x.double() @ w.double().t()) < 2e-6
+    for m in (1, 7, 16):
+        few = ops.linear(x[:m].contiguous(), w, None, torch.float32)
+        assert torch.equal(few, many[:m])
+    shifted = torch.cat([x.new_zeros(1), x[:3].reshape(-1)])[1:].view(3, k)     # rows that start 4 bytes off
+    assert shifted.data_ptr() % 16 == 4 and torch.equal(ops.linear(shifted, w, None, torch.float32), many[:3])
+
+
 def test_linear_bias_and_mixed_dtypes(ops):
     x = rnd((5, 40), torch.bfloat16, 7).cuda()
     w32 = rnd((24, 40), torch.float32, 8).cuda()        # a matrix stored in 32-bit stays so
