@@ -483,7 +483,7 @@ __device__ __forceinline__ void page_values(const PageFrags<HD>& f, const f32x4 
 }
 
 template <int HD, int WAVES, bool AHEAD>
-__global__ __launch_bounds__(WAVES * 64, (HD <= 128) ? 2 : 1) void attn_decode_kernel(
+__global__ __launch_bounds__(WAVES * 64, (HD <= 128) ? 2 : ((HD <= 192) ? 3 : 1)) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ v_pages, const int* __restrict__ table, int table_stride,
     const int* __restrict__ seq_slot, const int* __restrict__ seq_pos0, float* __restrict__ part_o,
@@ -772,5 +772,7 @@ extern "C" int llm_attention_decode_bf16(const void* q, int q_stride, const void
 
 // Waves per block of the decode kernel for a head size (the host sizes its grid with it): four
 // while their partial results fit the 64 KiB of shared memory a block may declare (with two,
-// head sizes 160 and 192 read 3.3 and 2.7 TB/s at batch 64 and 4,096 keys; with four 4.7 and 4.1).
+// head sizes 160 and 192 read 3.3 and 2.7 TB/s at batch 64 and 4,096 keys; with four 4.7 and 4.1;
+// the kernel's launch bounds ask for three such blocks a compute unit, without which head size
+// 176 took 170 registers, two too many for that, and read 2.7 TB/s instead of 4.3).
 extern "C" int llm_attention_decode_waves(int hd) { return hd > 192 ? 2 : 4; }
