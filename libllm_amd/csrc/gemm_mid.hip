@@ -1,6 +1,7 @@
-// C[M,N] = X[M,K] * W[N,K]^T for 33 to 128 rows: still bound by the one pass over W, but with too
+// C[M,N] = X[M,K] * W[N,K]^T for 33 to 256 rows: still bound by the one pass over W, but with too
 // many rows for a block to stage all of them per 16 rows of W, as the product for few rows does.
-// bfloat16 inputs, float32 accumulation on the matrix cores.
+// bfloat16 inputs, float32 accumulation on the matrix cores.  (Up to 128 rows a block takes all
+// the rows; beyond, two blocks take a slab of rows each, see the kernel's first lines.)
 //
 // A block owns 64 rows of W over all of K or one slice of it.  Four of its eight waves compute:
 // two pairs of waves with two tiles of 16 rows each (what a wave reads of X from shared memory
@@ -58,7 +59,8 @@ template <int MT, int EPI, typename OutT>
 __global__ __launch_bounds__(MID_NT, 2) void gemm_mid_kernel(const bf16_t* __restrict__ X,
                                                              const bf16_t* __restrict__ W,
                                                              OutT* __restrict__ C, int M, int N, int K,
-                                                             int ldx, int w_steps, int n_out, int act) {
+                                                             int ldx, int w_steps, int n_out, int act,
+                                                             int slab_rows, int n_tiles) {
   constexpr int ROW_B = MID_CK * 2;                  // bytes of a staged row: 16 pieces of 16 bytes, swizzled
   constexpr int BUF = 16 * MT * ROW_B;
   constexpr int PASSES = MT;                         // 256 threads carry 16 rows a pass
@@ -68,8 +70,20 @@ __global__ __launch_bounds__(MID_NT, 2) void gemm_mid_kernel(const bf16_t* __res
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int wn = wave >> 1, wk = wave & 1;
   const int r = lane & 15, g = lane >> 4;
+  // More than 128 rows go in two slabs of slab_rows rows, a block each.  The two blocks of a tile
+  // of W are neighbours among the blocks that one chiplet gets (block b goes to chiplet b % 8),
+  // so they run side by side and the second finds the tile in the chiplet's cache.
+  int bx = blockIdx.x, m0 = 0;
+  if (slab_rows < M) {
+    const int i = bx >> 3;
+    bx = (i >> 1) * 8 + (bx & 7);
+    m0 = (i & 1) * slab_rows;
+  }
+  if (bx >= n_tiles) return;                         // (the grid is rounded up to whole rounds of the chiplets)
+  const int m_total = M;
+  M = (M - m0 < slab_rows) ? M - m0 : slab_rows;     // this block's rows
   const int k0 = blockIdx.y * K;                     // this block's slice of K (K elements, a multiple of 32 if sliced)
-  X += k0;
+  X += k0 + (size_t)m0 * ldx;
   const int n_chunks = K / MID_CK;                   // K is a multiple of the chunk
 
   // first rows of W of this wave's tiles
@@ -78,9 +92,9 @@ __global__ __launch_bounds__(MID_NT, 2) void gemm_mid_kernel(const bf16_t* __res
 #pragma unroll
   for (int rt = 0; rt < MID_RT; ++rt) {
     if (MID_IS_GATED(EPI))
-      tile_row[rt] = rt * n_out + (blockIdx.x * 2 + wn) * 16;
+      tile_row[rt] = rt * n_out + (bx * 2 + wn) * 16;
     else
-      tile_row[rt] = ((blockIdx.x * 2 + wn) * MID_RT + rt) * 16;
+      tile_row[rt] = ((bx * 2 + wn) * MID_RT + rt) * 16;
     int t = tile_row[rt] / 16;
     if (t > (N - 1) / 16) t = (N - 1) / 16;          // tiles past the end read the last one; not stored
     wp[rt] = W + ((size_t)t * w_steps * 64 + lane) * 8 + (size_t)(k0 / 32) * 512;
@@ -231,7 +245,7 @@ __global__ __launch_bounds__(MID_NT, 2) void gemm_mid_kernel(const bf16_t* __res
       uint2 pk;
       pk.x = pack2_bf16(v[0], v[1]);
       pk.y = pack2_bf16(v[2], v[3]);
-      *reinterpret_cast<uint2*>(C + (size_t)m * n_out + n) = pk;       // n_out is a multiple of 16
+      *reinterpret_cast<uint2*>(C + (size_t)(m0 + m) * n_out + n) = pk;       // n_out is a multiple of 16
     }
     return;
   }
@@ -245,7 +259,7 @@ __global__ __launch_bounds__(MID_NT, 2) void gemm_mid_kernel(const bf16_t* __res
       const int m = mt * 16 + r;
       if (m >= M) continue;
       const f32x4 sum = acc[rt][mt];
-      OutT* dst = C + ((size_t)blockIdx.y * M + m) * N + n;
+      OutT* dst = C + ((size_t)blockIdx.y * m_total + m0 + m) * N + n;
       if (n + 3 < N && (N & 3) == 0) {
         if (sizeof(OutT) == 2) {
           uint2 pk;
@@ -269,14 +283,17 @@ static int launch_mid(const bf16_t* X, const bf16_t* W, void* C, int M, int N, i
                       int k_split, int act, hipStream_t stream) {
   const int n_out = (MID_IS_GATED(EPI)) ? N / 2 : N;
   const int per_block = (MID_IS_GATED(EPI)) ? 32 : 64;
-  const dim3 grid((n_out + per_block - 1) / per_block, k_split);
+  const int n_tiles = (n_out + per_block - 1) / per_block;
+  // up to 128 rows: a block a tile of W; beyond: two slabs of rows, evenly, in whole tiles of 16
+  const int slab_rows = (M <= 128) ? M : ((M + 31) / 32) * 16;
+  const dim3 grid((M <= 128) ? n_tiles : 2 * ((n_tiles + 7) / 8) * 8, k_split);
   const int w_steps = (K + 31) / 32;
 #define MID_CASE(T)                                                                                  \
   case T:                                                                                            \
     gemm_mid_kernel<T, EPI, OutT><<<grid, MID_NT, 0, stream>>>(X, W, (OutT*)C, M, N, K / k_split, ldx,  \
-                                                            w_steps, n_out, act);                    \
+                                                            w_steps, n_out, act, slab_rows, n_tiles); \
     break;
-  switch ((M + 15) / 16) {
+  switch ((slab_rows + 15) / 16) {
     MID_CASE(3)
     MID_CASE(4)
     MID_CASE(5)
@@ -289,7 +306,8 @@ static int launch_mid(const bf16_t* X, const bf16_t* W, void* C, int M, int N, i
   return llm_launch_status();
 }
 
-// X [M, K] bfloat16 with rows ldx apart, 33 <= M <= 128; W the tiled copy of a [N, K] matrix.
+// X [M, K] bfloat16 with rows ldx apart, 33 <= M <= 256 (beyond 128 in two slabs of rows that
+// share every tile of W through the chiplet's cache); W the tiled copy of a [N, K] matrix.
 // epilogue 0: C [M, N] bfloat16, or with k_split > 1 float32 [k_split, M, N], the products over
 // the slices of K; K is a multiple of 128 * k_split; epilogue 1 (1 | act << 4 for another activation of the gate, common.h): C [M, N/2] bfloat16, SwiGLU over
 // W = [Wg; Wu], N/2 a multiple of 16.
@@ -298,7 +316,7 @@ extern "C" int llm_gemm_mid_bf16(const void* X, int ldx, const void* W_tiled, vo
   const int act = epilogue >> 4;                 // the gate's activation rides above the epilogue's code
   epilogue &= 15;
   if (act < 0 || act >= LLM_ACT_COUNT || (act != 0 && epilogue != MID_EPI_SWIGLU)) return LLM_ERR_ARG;
-  if (M < 33 || M > 128 || N <= 0 || K <= 0 || (K & 7) || ldx < K || (ldx & 7) || k_split < 1)
+  if (M < 33 || M > 256 || N <= 0 || K <= 0 || (K & 7) || ldx < K || (ldx & 7) || k_split < 1)
     return LLM_ERR_ARG;
   if (X == nullptr || W_tiled == nullptr || C == nullptr) return LLM_ERR_ARG;
   if ((((uintptr_t)X) | ((uintptr_t)W_tiled) | ((uintptr_t)C)) & 15) return LLM_ERR_ARG;

@@ -119,7 +119,19 @@ class HipOps:
     # 48 and 64: 2.04 against 2.09 and 2.38 against 2.46 ms at the 1B shape, 4.02 against 4.11 and
     # 4.69 against 4.83 at 3B, 5.58 against 5.74 and 6.17 against 6.45 at 8B).
     MID_FROM = 33
-    MID_HEAD = True         # logits of 65 rows and more by it too (beyond 128 rows in passes)
+    MID_HEAD = True         # logits of 65 rows and more by it too (beyond its most rows in passes)
+    # With ``mid_two``, 129 to MID_TWO_ROWS rows go to the same product in two slabs of rows, a
+    # block each for every tile of W, neighbours on one chiplet, so that W still comes from memory
+    # once.  Where it is taken, by the product (us a product with the norm that follows, at 160 / 256
+    # rows, against the library's): down 1B 20.8 / 24.5 against 30.1 / 32.5, 3B 30.0 / 33.9 against
+    # 33.6 / 39.7, 8B 49.7 / 56.8 against 89.1 / 70.2, a 8,192 x 28,672 weight 172 / 197 against 221 /
+    # 323; output 3B 18.5 / 20.6 against 21.2 / 22.9, 8B 22.1 / 25.8 against 33.0 / 28.9 (1B 13.7 /
+    # 16.0 against 13.3 / 14.2: a tie at best); half as many slices of K as up to 128 rows, for as
+    # many blocks.  Whole engines, 1B: decode at batch 160 / 192 / 256 2.61 / 2.93 / 3.19 against 2.81 /
+    # 3.11 / 3.30 ms a step (context 1,024), prompts of 140 to 256 tokens 1.74 to 1.89 against 1.92 to
+    # 1.98 ms.
+    MID_TWO_ROWS = 256
+    MID_PLAIN_FILL = 0.6    # a product that does not add into the stream goes to it in two slabs if its blocks fill this share of one round of the units
     # Beyond MID_ROWS rows the gate/up product with its SwiGLU is a kernel of ours where its tiles
     # (256 or 128 rows by 128 outputs) would be filled, over whole rounds of the compute units, to
     # at least WIDE_FILL: there it beats the library's product followed by the SiLU-mul kernel, which reads
@@ -181,6 +193,7 @@ class HipOps:
         self.fast_gemm = True           # the skinny product for few rows (else the library's for every product)
         self.wide_gemm = True           # the gate/up product with SwiGLU for many rows (else the library's and the SiLU-mul kernel)
         self.mid_gemm = True            # the product for 33 to 128 rows (else the one for few rows and the library's)
+        self.mid_two = True             # the same for 129 to 256 rows, in two slabs (else the library's)
         if not build.trusted("gemm_mid.hip"):
             # its loads are invisible to the compiler: with a spilled register it would be wrong
             self.mid_gemm = False
@@ -420,9 +433,12 @@ class HipOps:
             ks -= 1
         return ks
 
+    def _mid_rows(self):
+        return self.MID_TWO_ROWS if self.mid_two else self.MID_ROWS
+
     def _mid_ok(self, x, w, m, k):
         return (self.fast_gemm and self.mid_gemm and isinstance(w, PreparedWeight)
-                and self.MID_FROM <= m <= self.MID_ROWS and not isinstance(x, NormedRows)
+                and self.MID_FROM <= m <= self._mid_rows() and not isinstance(x, NormedRows)
                 and x.dtype == torch.bfloat16 and x.dim() == 2 and x.stride(1) == 1 and x.stride(0) >= k
                 and x.stride(0) % 8 == 0 and x.data_ptr() % 16 == 0 and k % 128 == 0)
 
@@ -453,11 +469,11 @@ class HipOps:
             x.shape[0], n, k, self._stream()), "gemm_wide_bf16")
         return out
 
-    def _k_split_mid(self, n, k):
-        """Slices of K for a product of 33 to 128 rows whose result the next norm adds: enough for
-        about MID_BLOCKS blocks at 64 weight rows a block, each at least MID_MIN_SLICE long and a
-        multiple of 128."""
-        ks = max(1, min(16, self.MID_BLOCKS // max(1, -(-n // 64))))
+    def _k_split_mid(self, n, k, slabs=1):
+        """Slices of K for a product of 33 to 256 rows whose result the next norm adds: enough for
+        about MID_BLOCKS blocks at 64 weight rows a block and slab of rows, each at least
+        MID_MIN_SLICE long and a multiple of 128."""
+        ks = max(1, min(16, self.MID_BLOCKS // max(1, -(-n // 64) * slabs)))
         while ks > 1 and (k % (ks * 128) or k // ks < self.MID_MIN_SLICE):
             ks -= 1
         return ks
@@ -513,9 +529,9 @@ class HipOps:
                 and self.SKINNY_ROWS < m and not lazy):
             # float32 results (logits) for 65 to 128 rows in one pass over the weight, where the
             # product for few rows would take two, and for more rows in passes of up to 128
-            passes = -(-m // self.MID_ROWS)
+            passes = -(-m // self._mid_rows())
             # the rows dealt out evenly, each pass starting at a multiple of 16 rows (which keeps
-            # its rows of the result aligned): passes of 49 to 128 rows
+            # its rows of the result aligned): passes of at least 49 rows
             cuts = [min(m, -(-(i * m) // (passes * 16)) * 16) for i in range(passes)] + [m]
             if self._mid_ok(x[:cuts[1]], w, cuts[1], k):
                 out = torch.empty((m, n), dtype=torch.float32, device=self.device)
@@ -558,12 +574,22 @@ class HipOps:
             if self._skinny_ok(x, w, m, k) and bias is None:
                 return self.linear(x, w, None, out_dtype, residual)
         if self._mid_ok(x, w, m, k) and bias is None and out_dtype != torch.float32:
-            # (without slices of K, for a product that does not add into the stream, it has too few
-            # blocks for the q|k|v weights and loses to the library: 16.7 against 13.0 us at 128 rows)
-            if residual is not None and (ks := self._k_split_mid(n, k)) * -(-n // 64) >= self.MID_FILL * self.units:
+            slabs = 2 if m > self.MID_ROWS else 1
+            tiles = -(-n // 64) * slabs
+            if residual is not None and (ks := self._k_split_mid(n, k, slabs)) * tiles >= self.MID_FILL * self.units:
                 # K in slices for enough blocks; the norm kernel that follows adds them, in order
                 return self._mid(x, w, torch.empty((ks, m, n), dtype=torch.float32, device=self.device),
                                  self._EPI_NONE, ks)
+            # Without slices of K, for a product that does not add into the stream (q|k|v), it has
+            # too few blocks up to 128 rows and loses to the library (16.7 against 13.0 us at 128
+            # rows of the 1B shape).  In two slabs it has twice as many and wins where they make
+            # one round of the units that is well filled (us at 160 / 256 rows: 3B, 160 blocks,
+            # 19.3 / 21.6 against 24.0 / 32.3; 8B, 192 blocks, 24.7 / 28.0 against 29.2 / 41.3; but
+            # 1B, 96 blocks, 13.5 / 15.3 against 9.5 / 10.9, and a weight of 10,240 x 8,192, 320
+            # blocks, 85 / 99 against 72 / 94).
+            if (residual is None and slabs == 2
+                    and self.MID_PLAIN_FILL * self.units <= tiles <= self.units):
+                return self._mid(x, w, torch.empty((m, n), dtype=torch.bfloat16, device=self.device), self._EPI_NONE)
         w = self._plain(w)
         if w.dtype == torch.float32:
             if w.stride(0) != k:
@@ -652,7 +678,11 @@ class HipOps:
                 raise KernelError("linear_swiglu: a normed record needs the activation dtype")
             x = self._materialise(x, dtype)
             return self.linear_swiglu(x, w, dtype, activation)
-        if self._mid_ok(x, w, m, k) and inter % 16 == 0 and dtype == torch.bfloat16:
+        # (in two slabs of rows only where all its blocks run at once: us at 160 / 256 rows against
+        # the library's product and the gating kernel: 1B 30.0 / 36.3 against 32.7 / 36.5, 3B 41.3 /
+        # 48.1 against 40.8 / 50.3, but 8B, 1,792 blocks, 93 / 105 against 67 / 80)
+        if (self._mid_ok(x, w, m, k) and inter % 16 == 0 and dtype == torch.bfloat16
+                and (m <= self.MID_ROWS or -(-inter // 32) <= self.units)):
             self._weight(self._plain(w), "linear weight")
             return self._mid(x, w, torch.empty((m, inter), dtype=torch.bfloat16, device=self.device), gated)
         if dtype == torch.bfloat16 and (block_rows := self._wide_ok(x, w, m, k, inter)):

@@ -562,8 +562,8 @@ def test_logits_of_65_to_128_rows_take_one_pass(ops):
 
 @pytest.mark.parametrize("n", [1000, 517])
 def test_float32_results_of_many_rows_in_passes(ops, n):
-    """Logits (float32, no residual) of 65 rows and more go through the product for 33 to 128
-    rows, in one pass up to 128 rows and in even passes beyond; a row's bits do not depend on
+    """Logits (float32, no residual) of 65 rows and more go through the product for 33 to 256
+    rows, in one pass up to 256 rows and in even passes beyond; a row's bits do not depend on
     how many rows there are, nor on the pass it falls into.  A vocabulary that is no multiple of
     4 has rows that are not 16 bytes apart: every pass still starts at an aligned row."""
     k = 256
@@ -575,24 +575,58 @@ def test_float32_results_of_many_rows_in_passes(ops, n):
     ops._mid = lambda *a, **kw: calls.append(a[0].shape[0]) or real(*a, **kw)
     try:
         full = ops.linear(x, w, None, torch.float32)
-        assert sum(calls) == 1100 and len(calls) == 9 and all(49 <= c <= 128 for c in calls)
+        top = ops._mid_rows()                                 # most rows of a pass: 256, in two slabs beyond 128
+        assert sum(calls) == 1100 and len(calls) == -(-1100 // top) and all(49 <= c <= top for c in calls)
         assert full.dtype == torch.float32 and close(full, ref, torch.float32)
         for m in (65, 128, 129, 255, 257, 1000):
             del calls[:]
             part = ops.linear(x[:m], w, None, torch.float32)
-            assert sum(calls) == m and len(calls) == -(-m // 128)
+            assert sum(calls) == m and len(calls) == -(-m // top)
             assert torch.equal(part, full[:m])
     finally:
         ops._mid = real
+
+
+@pytest.mark.parametrize("m", [129, 130, 160, 161, 200, 255, 256])
+@pytest.mark.parametrize("nk", [(64, 128), (1000, 256), (2048, 2048), (520, 1024), (4, 128)])
+def test_gemm_mid_in_two_slabs(ops, m, nk):
+    """129 to 256 rows go in two slabs of rows, a block each for every tile of W: plain as
+    bfloat16, in slices of K as float32 matrices, and gated, against float64; a row's bits are
+    those of the same row among up to 128 (the slabs split at other rows than the passes do);
+    weights whose tiles are no multiple of 8 (the grid is rounded up to whole rounds of the
+    chiplets), a sentinel behind the result."""
+    n, k = nk
+    x = rnd((m, k), torch.bfloat16, 31).cuda()
+    w = ops.prepare_weight(rnd((n, k), torch.bfloat16, 32, scale=0.05).cuda())
+    ref = x.double() @ w.w.double().t()
+    buf = torch.full((m * n + 64,), 7.0, dtype=torch.bfloat16, device="cuda")
+    out = ops._mid(x, w, buf[:m * n].view(m, n), ops._EPI_NONE)
+    assert close(out, ref, torch.bfloat16) and (buf[m * n:] == 7.0).all()
+    first = ops._mid(x[:128], w, torch.empty((128, n), dtype=torch.bfloat16, device="cuda"), ops._EPI_NONE)
+    rest = ops._mid(x[m - 100:], w, torch.empty((100, n), dtype=torch.bfloat16, device="cuda"), ops._EPI_NONE)
+    assert torch.equal(out[:128], first) and torch.equal(out[m - 100:], rest)
+    ks = 2 if (k // 128) % 2 == 0 else 1
+    parts = ops._mid(x, w, torch.empty((ks, m, n), dtype=torch.float32, device="cuda"), ops._EPI_NONE, ks)
+    total = parts[0].clone()
+    for j in range(1, ks):
+        total += parts[j]
+    assert close(total, ref, torch.float32)
+    if n % 32 == 0:
+        inter = n // 2
+        got = ops._mid(x, w, torch.empty((m, inter), dtype=torch.bfloat16, device="cuda"), ops._EPI_SWIGLU)
+        one = torch.cat([ops._mid(x[:128], w, torch.empty((128, inter), dtype=torch.bfloat16, device="cuda"), ops._EPI_SWIGLU),
+                         ops._mid(x[128:] if m - 128 >= 33 else x[m - 33:], w,
+                                  torch.empty((max(m - 128, 33), inter), dtype=torch.bfloat16, device="cuda"), ops._EPI_SWIGLU)[-(m - 128):]])
+        assert torch.equal(got, one)
 
 
 def test_gemm_mid_refuses(ops):
     from libllm_amd.errors import KernelError
     w = ops.prepare_weight(rnd((64, 256), torch.bfloat16, 1).cuda())
     x = rnd((128, 256), torch.bfloat16, 2).cuda()
-    for rows, ks in ((32, 1), (129, 1), (100, 3)):                     # too few rows, too many, slices that do not divide K
+    for rows, ks in ((32, 1), (257, 1), (100, 3)):                     # too few rows, too many, slices that do not divide K
         with pytest.raises(KernelError):
-            xs = torch.cat([x, x])[:rows].contiguous()
+            xs = torch.cat([x, x, x])[:rows].contiguous()
             ops._mid(xs, w, torch.empty((ks, rows, 64), dtype=torch.float32, device="cuda"), ops._EPI_NONE, ks)
     w2 = ops.prepare_weight(rnd((64, 200), torch.bfloat16, 1).cuda())    # K no multiple of the chunk
     assert not ops._mid_ok(rnd((100, 200), torch.bfloat16, 2).cuda(), w2, 100, 200)

@@ -315,7 +315,8 @@ def test_layers_of_the_measured_shapes(tmp_path, shape):
     by the sizes and by the rows of a step, so the tiny configurations do not reach every form:
     batches of 1, 8, 20, 48 and 64 decode through each form of the skinny product and, from 33
     rows on, the product for 33 to 128 rows, as do batches of 96 and 128 and a prompt of 100
-    tokens; the three prompts of 670 tokens (a step of some 2,030 rows) go through the library's
+    tokens; a batch of 200, a prompt of 230 tokens and two of 75 (a step of some 160 rows) go through
+    the same product in two slabs of rows; the three prompts of 670 tokens (a step of some 2,030 rows) go through the library's
     products and, for the gate and up weights of the 1B and 3B shapes, the product for many rows
     (test_the_gate_and_up_product_of_a_long_prompt_is_ours sees that it runs)."""
     sh = dict(BENCH_SHAPES[shape])
@@ -330,7 +331,8 @@ def test_layers_of_the_measured_shapes(tmp_path, shape):
     rng = np.random.default_rng(1)
     for batch, prompt, decode, dtypes in ((1, 40, 5, DTYPES), (8, 30, 5, DTYPES), (20, 20, 3, DTYPES),
                                           (48, 10, 3, ["bfloat16"]), (64, 8, 3, DTYPES), (3, 670, 2, ["bfloat16"]),
-                                          (96, 6, 3, ["bfloat16"]), (1, 100, 2, ["bfloat16"]), (128, 1, 2, ["bfloat16"])):
+                                          (96, 6, 3, ["bfloat16"]), (1, 100, 2, ["bfloat16"]), (128, 1, 2, ["bfloat16"]),
+                                          (200, 1, 2, ["bfloat16"]), (1, 230, 2, ["bfloat16"]), (2, 75, 2, ["bfloat16"])):
         group = {"s%d_%d" % (batch, i): rng.integers(0, cfg.vocab, size=prompt + int(rng.integers(0, 9)) + decode).tolist()
                  for i in range(batch)}
         steps = traces.batches([group], {r: decode for r in group})
