@@ -127,9 +127,10 @@ class HipOps:
     # 33.6 / 39.7, 8B 49.7 / 56.8 against 89.1 / 70.2, a 8,192 x 28,672 weight 172 / 197 against 221 /
     # 323; output 3B 18.5 / 20.6 against 21.2 / 22.9, 8B 22.1 / 25.8 against 33.0 / 28.9 (1B 13.7 /
     # 16.0 against 13.3 / 14.2: a tie at best); half as many slices of K as up to 128 rows, for as
-    # many blocks.  Whole engines, 1B: decode at batch 160 / 192 / 256 2.61 / 2.93 / 3.19 against 2.81 /
-    # 3.11 / 3.30 ms a step (context 1,024), prompts of 140 to 256 tokens 1.74 to 1.89 against 1.92 to
-    # 1.98 ms.
+    # many blocks.  Whole engines with the rules below (ms): decode at batch 160 / 256, context 1,024:
+    # 1B 2.48 / 3.08 against 2.81 / 3.29, 3B 6.38 / 8.30 against 6.79 / 9.02, 8B 9.06 / 11.8 against
+    # 10.9 / 12.9; prompts of 170 / 256 tokens: 1B 1.58 / 1.74 against 1.93 / 1.96, 3B 3.71 / 4.01
+    # against 4.05 / 4.70, 8B 6.20 / 6.89 against 7.00 / 7.87.
     MID_TWO_ROWS = 256
     MID_PLAIN_FILL = 0.6    # a product that does not add into the stream goes to it in two slabs if its blocks fill this share of one round of the units
     # Beyond MID_ROWS rows the gate/up product with its SwiGLU is a kernel of ours where its tiles
