@@ -541,6 +541,46 @@ def test_steps_of_33_to_64_rows_use_it_where_it_fills_the_device(ops):
     assert torch.equal(ops.linear_swiglu(xs[:40].contiguous(), gate_up), act[:40])
 
 
+def test_steps_of_129_to_256_rows_take_it_by_the_product(ops):
+    """Which products of a step of 129 to 256 rows go to the product for 33 to 128 rows in two
+    slabs, and which stay with the library or the product for many rows: by the weight's shape,
+    as measured (the down and output products in slices of K, half as many as up to 128 rows;
+    q|k|v where its blocks fill most of one round of the units; gate|up where all its blocks run
+    at once).  Every result against float64."""
+    took = []
+    real_mid, real_lib, real_wide = ops._mid, ops._library_product, ops._wide
+    ops._mid = lambda *a, **kw: took.append(("mid", a[4] if len(a) > 4 else kw.get("k_split", 1))) or real_mid(*a, **kw)
+    ops._library_product = lambda *a, **kw: took.append(("library", 1)) or real_lib(*a, **kw)
+    ops._wide = lambda *a, **kw: took.append(("wide", 1)) or real_wide(*a, **kw)
+    try:
+        m = 200
+        for what, (n, k), adds, want in (("down 1B", (2048, 8192), True, ("mid", 4)), ("down 8B", (4096, 14336), True, ("mid", 2)),
+                                         ("q|k|v 1B", (3072, 2048), False, ("library", 1)), ("q|k|v 3B", (5120, 3072), False, ("mid", 1)),
+                                         ("q|k|v 8B", (6144, 4096), False, ("mid", 1)), ("q|k|v wide", (10240, 8192), False, ("library", 1))):
+            x = rnd((m, k), torch.bfloat16, 41).cuda()
+            w = ops.prepare_weight(rnd((n, k), torch.bfloat16, 42, scale=0.02).cuda())
+            res = torch.zeros((m, n), dtype=torch.float32, device="cuda")
+            del took[:]
+            out = ops.linear(x, w, None, torch.bfloat16, residual=res if adds else None)
+            assert took == [want], (what, took)
+            ref = x.double() @ w.w.double().t()
+            if adds:
+                assert tuple(out.shape) == (want[1], m, n) and close(out.sum(0), ref, torch.float32, f32=3e-5)
+            else:
+                assert close(out, ref, torch.bfloat16)
+        for what, (inter, k), want in (("gate|up 1B", (8192, 2048), "mid"), ("gate|up 8B", (14336, 4096), "library")):      # (at 256 rows the product for many rows, whose tiles it then fills)
+            x = rnd((m, k), torch.bfloat16, 43).cuda()
+            w = ops.prepare_weight(rnd((2 * inter, k), torch.bfloat16, 44, scale=0.02).cuda())
+            del took[:]
+            out = ops.linear_swiglu(x, w)
+            assert [t[0] for t in took] == [want], (what, took)
+            gu = (x.double() @ w.w.double().t()).bfloat16().double()
+            ref = gu[:, inter:] * gu[:, :inter] / (1 + torch.exp(-gu[:, :inter]))
+            assert ((out.double() - ref).abs() / (ref.abs() + ref.abs().mean())).max().item() < 0.02
+    finally:
+        ops._mid, ops._library_product, ops._wide = real_mid, real_lib, real_wide
+
+
 def test_logits_of_65_to_128_rows_take_one_pass(ops):
     """Float32 results without a stream to add to (the head) go through the product for 33 to 128
     rows from 65 rows on, where the product for few rows would read the weight twice; a normed
