@@ -15,6 +15,7 @@ from typing import Iterable, List, Optional, Sequence, Union
 from .cache import PAGE
 from .engine import Generator, StepEntry
 from .errors import ConfigError, RequestError
+from .prompt import ControlToken, plain_prompt
 from .config import config_from_dir
 from .runtime import load_engine, random_engine
 from .sampling import Sampler, SamplingParams
@@ -36,13 +37,6 @@ def parse_device(device) -> Device:
             raise ConfigError("invalid device name: must be one of \"cpu\", \"cuda\" or \"auto\"")
         return names[device.lower()]
     return Device(int(device))
-
-
-class ControlToken:
-    """A control token in a prompt, by name, for example <|eot_id|>."""
-
-    def __init__(self, token_name: str) -> None:
-        self._name = token_name
 
 
 class Chunk:
@@ -67,6 +61,9 @@ class _ByteTokenizer:
     def control(self, name: str) -> int:
         raise RequestError("control token %r needs a tokenizer.json beside the model" % name)
 
+    def knows(self, name: str) -> bool:
+        return False
+
     def piece(self, token: int) -> bytes:
         return bytes([token]) if token < 256 else ("<%d>" % token).encode()
 
@@ -84,6 +81,9 @@ class _FileTokenizer:
         if tid is None:
             raise RequestError("unknown control token %r" % name)
         return tid
+
+    def knows(self, name: str) -> bool:
+        return self.tok.token_to_id(name) is not None
 
     def piece(self, token: int) -> bytes:
         return self.tok.decode([token], skip_special_tokens=False).encode("utf-8")
@@ -159,6 +159,19 @@ class Model:
             spec = self.engine.model.spec
             self._tok = _FileTokenizer(path) if os.path.isfile(path) else _ByteTokenizer(spec.vocab, spec.bos_token)
         return self._tok
+
+    def build_prompt(self, messages):
+        """The prompt of a conversation (``[{"role", "content"}, ...]``, the last message the
+        user's, or the assistant's to be continued): in the architecture's chat format, as the
+        reference's model class builds it (src/libllm/llama.cc:406-442), where the tokenizer
+        beside the model knows the format's control tokens; else the messages as lines of text."""
+        build = getattr(self.config, "build_prompt", None)
+        if build is not None:
+            blocks = build(messages)
+            tok = self._tokenizer()
+            if all(tok.knows(b._name) for b in blocks if isinstance(b, ControlToken)):
+                return blocks
+        return plain_prompt(messages)
 
     def _prepare_prompt(self, prompt) -> List[int]:
         if isinstance(prompt, str):

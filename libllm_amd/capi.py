@@ -50,8 +50,8 @@ def info(model) -> str:
 
 def complete(model, kwargs_json: str) -> Iterator:
     """Starts a completion.  ``messages`` is a list of ``{"role", "content"}`` as in the reference
-    (src/libllm/llm.cc:98-123); since tokenisation lies outside this library the contents are
-    joined as the command line joins them.  Ours: ``token_ids`` in place of ``messages``,
+    (src/libllm/llm.cc:98-123), put into the architecture's chat format where the tokenizer beside
+    the model knows its control tokens (``Model.build_prompt``).  Ours: ``token_ids`` in place of ``messages``,
     ``max_new_tokens``, ``seed``, ``stop_ids`` (beside the model's own).  Defaults: temperature 1.0, top_k 50, top_p 0.8
     (src/libllm/llm.cc:125-132)."""
     kw = json.loads(kwargs_json)
@@ -65,12 +65,7 @@ def complete(model, kwargs_json: str) -> Iterator:
     if "token_ids" in kw:
         prompt = [int(t) for t in kw["token_ids"]]
     else:
-        parts = []
-        for m in kw["messages"]:
-            if not isinstance(m, dict) or "role" not in m or "content" not in m:
-                raise RequestError("a message needs \"role\" and \"content\"")
-            parts.append("%s: %s\n" % (m["role"], m["content"]))
-        prompt = "".join(parts) + "assistant: "
+        prompt = model.build_prompt(kw["messages"])
     completion = model.complete(prompt, top_k=int(kw.get("top_k", 50)), top_p=float(kw.get("top_p", 0.8)),
                                 temperature=float(kw.get("temperature", 1.0)),
                                 max_new_tokens=int(kw.get("max_new_tokens", 256)), seed=int(kw.get("seed", 0)),

@@ -6,7 +6,9 @@ empty lines ignored and end of input leaving; after each reply it prints
 counterpart of the reference's llm_benchmark (src/libllm/benchmark_main.cc:98-134).
 
 Tokenisation is outside this library: with ``-ids`` a line is a list of token ids and the reply is
-printed as ids; otherwise a tokenizer.json beside the model, or bytes as token ids, are used.
+printed as ids; otherwise a tokenizer.json beside the model, or bytes as token ids, are used.  The
+session's messages go into the architecture's chat format (``Model.build_prompt``,
+src/libllm/llama.cc:406-442) where that tokenizer knows its control tokens, else as lines of text.
 """
 import argparse
 import sys
@@ -104,7 +106,7 @@ def chat_main(argv) -> int:
             if not history and system_prompt:
                 history.append(("system", system_prompt))
             history.append(("user", question))
-            prompt = "".join("%s: %s\n" % h for h in history) + "assistant: "
+            prompt = model.build_prompt([{"role": role, "content": text} for role, text in history])
         t0 = time.time()
         n, reply_ids, reply_text = 0, [], ""
         for chunk in model.complete(prompt, top_k=args.top_k, top_p=args.top_p, temperature=args.temperature,

@@ -141,6 +141,12 @@ class LlamaConfig:
         }
         return d
 
+    def build_prompt(self, messages):
+        """The messages of a chat in this architecture's format, as blocks of text and control
+        tokens (src/libllm/llama.cc:406-442)."""
+        from ..prompt import llama3_prompt
+        return llama3_prompt(messages)
+
     def to_spec(self) -> ModelSpec:
         """The decoder as data: every layer a prenorm block of grouped-query attention with
         rotary positions and a SwiGLU feed-forward (src/libllm/llama.cc:231-312); tensor names

@@ -90,6 +90,56 @@ def test_generation_matches_plain(models):
     assert [c.token_id for c in chunks if c.token_id is not None] == sampling.generate(cfg, weights, prompts[1], 3)
 
 
+def test_messages_become_the_architectures_chat_format(models, tmp_path):
+    """The messages of a chat, block by block as the reference's model class appends them
+    (src/libllm/llama.cc:406-442), where the tokenizer beside the model knows the control tokens;
+    lines of text where there is no tokenizer file; the last message the user's or the
+    assistant's."""
+    import shutil
+    from libllm_amd import ControlToken
+    from libllm_amd.prompt import llama3_prompt, plain_prompt
+    tokenizers = pytest.importorskip("tokenizers")
+    path, cfg, _ = models["B"]
+    chat = [{"role": "system", "content": "be brief"}, {"role": "user", "content": "hello there"},
+            {"role": "assistant", "content": "hi"}, {"role": "user", "content": "hello hi"}]
+    c = ControlToken
+    head = lambda role: [c("<|start_header_id|>"), role, c("<|end_header_id|>")]          # noqa: E731
+    assert llama3_prompt(chat) == (
+        [c("<|begin_of_text|>")] + head("system") + ["\n\nbe brief", c("<|eot_id|>")]
+        + head("user") + ["\n\nhello there", c("<|eot_id|>")] + head("assistant") + ["\n\nhi", c("<|eot_id|>")]
+        + head("user") + ["\n\nhello hi", c("<|eot_id|>")] + head("assistant") + ["\n\n"])
+    assert llama3_prompt(chat[:3])[-4:] == head("assistant") + ["\n\nhi"]                # left open: the reply continues it
+    for bad in ([], chat[:1], [{"role": "user"}]):
+        with pytest.raises(RequestError):
+            llama3_prompt(bad)
+    # no tokenizer file beside the model: bytes are the tokens, the messages lines of text
+    plain = Model(path, dtype="float32", max_tokens=512, ops=CpuOps())
+    assert plain.build_prompt(chat) == plain_prompt(chat) == (
+        "system: be brief\nuser: hello there\nassistant: hi\nuser: hello hi\nassistant: ")
+    # a tokenizer that knows the control tokens
+    folder = tmp_path / "with_tokenizer"
+    shutil.copytree(path, folder)
+    words = ["<|begin_of_text|>", "<|start_header_id|>", "<|end_header_id|>", "<|eot_id|>", "[UNK]", "system", "user",
+             "assistant", "be", "brief", "hello", "there", "hi"]
+    tok = tokenizers.Tokenizer(tokenizers.models.WordLevel({w: i for i, w in enumerate(words)}, unk_token="[UNK]"))
+    tok.pre_tokenizer = tokenizers.pre_tokenizers.Whitespace()
+    tok.add_special_tokens(words[:4])
+    tok.save(str(folder / "tokenizer.json"))
+    model = Model(str(folder), dtype="float32", max_tokens=512, ops=CpuOps())
+    blocks = model.build_prompt(chat)
+    assert blocks == llama3_prompt(chat)
+    bot, sh, eh, eot = 0, 1, 2, 3
+    assert model._prepare_prompt(blocks) == [bot, sh, 5, eh, 8, 9, eot, sh, 6, eh, 10, 11, eot, sh, 7, eh, 12, eot,
+                                             sh, 6, eh, 10, 12, eot, sh, 7, eh]
+    reply = [ch.token_id for ch in model.complete(blocks, top_k=1, max_new_tokens=3) if ch.token_id is not None]
+    assert len(reply) <= 3
+    # a tokenizer without them: lines of text again
+    tok2 = tokenizers.Tokenizer(tokenizers.models.WordLevel({w: i for i, w in enumerate(words[4:])}, unk_token="[UNK]"))
+    tok2.pre_tokenizer = tokenizers.pre_tokenizers.Whitespace()
+    tok2.save(str(folder / "tokenizer.json"))
+    assert Model(str(folder), dtype="float32", max_tokens=512, ops=CpuOps()).build_prompt(chat) == plain_prompt(chat)
+
+
 def build(spec, seed, ops, max_tokens=512):
     model = DecoderModel(spec)
     tensors = random_tensors(model.declared(), seed, std=0.1, norm_std=0.2, dtype=torch.float32)
