@@ -173,6 +173,13 @@ class Model:
                 return blocks
         return plain_prompt(messages)
 
+    def chat_stop_ids(self) -> List[int]:
+        """The ids of the control tokens that end a turn in the architecture's chat format, as
+        far as the tokenizer beside the model knows them: stop tokens of a chat's replies, beside
+        the model's own."""
+        tok = self._tokenizer()
+        return [tok.control(name) for name in getattr(self.config, "chat_stop_tokens", ()) if tok.knows(name)]
+
     def _prepare_prompt(self, prompt) -> List[int]:
         if isinstance(prompt, str):
             return self._tokenizer().encode(prompt)

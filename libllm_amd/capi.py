@@ -66,6 +66,7 @@ def complete(model, kwargs_json: str) -> Iterator:
         prompt = [int(t) for t in kw["token_ids"]]
     else:
         prompt = model.build_prompt(kw["messages"])
+        kw["stop_ids"] = list(kw.get("stop_ids") or []) + model.chat_stop_ids()
     completion = model.complete(prompt, top_k=int(kw.get("top_k", 50)), top_p=float(kw.get("top_p", 0.8)),
                                 temperature=float(kw.get("temperature", 1.0)),
                                 max_new_tokens=int(kw.get("max_new_tokens", 256)), seed=int(kw.get("seed", 0)),

@@ -111,7 +111,7 @@ def chat_main(argv) -> int:
         n, reply_ids, reply_text = 0, [], ""
         for chunk in model.complete(prompt, top_k=args.top_k, top_p=args.top_p, temperature=args.temperature,
                                     max_new_tokens=args.max_new_tokens, seed=args.seed + turn,
-                                    stop_ids=args.stop_id):
+                                    stop_ids=(args.stop_id or []) + ([] if args.ids else model.chat_stop_ids())):
             if chunk.token_id is not None:
                 n += 1
                 reply_ids.append(chunk.token_id)

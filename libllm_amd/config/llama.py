@@ -147,6 +147,11 @@ class LlamaConfig:
         from ..prompt import llama3_prompt
         return llama3_prompt(messages)
 
+    # the control token that ends a turn in that format: a reply stops there, beside the stop
+    # tokens that config.json names (the reference reads its id from the exported model,
+    # src/libllm/llama.cc:342,390-392)
+    chat_stop_tokens = ("<|eot_id|>",)
+
     def to_spec(self) -> ModelSpec:
         """The decoder as data: every layer a prenorm block of grouped-query attention with
         rotary positions and a SwiGLU feed-forward (src/libllm/llama.cc:231-312); tensor names

@@ -131,6 +131,7 @@ def test_messages_become_the_architectures_chat_format(models, tmp_path):
     bot, sh, eh, eot = 0, 1, 2, 3
     assert model._prepare_prompt(blocks) == [bot, sh, 5, eh, 8, 9, eot, sh, 6, eh, 10, 11, eot, sh, 7, eh, 12, eot,
                                              sh, 6, eh, 10, 12, eot, sh, 7, eh]
+    assert model.chat_stop_ids() == [eot] and plain.chat_stop_ids() == []
     reply = [ch.token_id for ch in model.complete(blocks, top_k=1, max_new_tokens=3) if ch.token_id is not None]
     assert len(reply) <= 3
     # a tokenizer without them: lines of text again
