@@ -51,6 +51,7 @@ class Engine:
     PROMPT_SEQS = (2, 3, 5, 9, 17)
     PROMPT_SEEN = 2
     PROMPT_GRAPHS = 24      # prompt graphs kept; the one unused for longest goes first (each holds its activations)
+    DECODE_GRAPHS = 64      # decode graphs kept, likewise (all twenty of one context length hold 2.8 GB at the 1B shape)
 
     def __init__(self, model: DecoderModel, ops, dtype: torch.dtype, max_tokens: int,
                  max_slots: Optional[int] = None, use_graphs: bool = True):
@@ -258,11 +259,13 @@ class Engine:
             ctx_bucket *= 2
         ctx_bucket = min(ctx_bucket, limit)
         key = (bucket, ctx_bucket)
-        graph = self._graphs.get(key)
+        graph = self._graphs.pop(key, None)
         if graph is None and ("decode",) + key not in self._no_graph:
+            while len(self._graphs) >= max(1, self.DECODE_GRAPHS):
+                del self._graphs[next(iter(self._graphs))]                  # dicts keep the order of insertion
             graph = self._checked(("decode",) + key, lambda: _DecodeGraph(self, bucket, ctx_bucket))
-            if graph is not None:
-                self._graphs[key] = graph
+        if graph is not None:
+            self._graphs[key] = graph                                       # the last used lies last
         return graph
 
 

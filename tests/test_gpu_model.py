@@ -792,6 +792,30 @@ def test_prompt_graphs_are_bounded(models):
     assert seen == [[16], [16, 32], [32, 48], [48, 16], [16, 80], [80, 32]]
 
 
+def test_decode_graphs_are_bounded(models):
+    """At most ``DECODE_GRAPHS`` decode graphs are kept, the one unused for longest goes first, and
+    a batch size that comes again after its graph went is captured again and gives the same
+    logits."""
+    import torch
+    from libllm_amd.engine import StepEntry
+    from libllm_amd.runtime import load_engine
+    path, cfg, _ = models["A"]
+    engine = load_engine(path, dtype="float32", max_tokens=2048)
+    engine.DECODE_GRAPHS = 2
+    ref = load_engine(path, dtype="float32", max_tokens=2048, use_graphs=False)
+    seen = []
+    for n in (1, 3, 5, 1, 8, 3):                         # graphs of 1, 3, 6, 1, 8 and 3 rows
+        names = ["r%d" % i for i in range(n)]
+        for e in (engine, ref):
+            e.step([StepEntry(r, [7 + i, 9], []) for i, r in enumerate(names)])
+        a = engine.step([StepEntry(r, [11 + i], [0]) for i, r in enumerate(names)]).clone()
+        b = ref.step([StepEntry(r, [11 + i], [0]) for i, r in enumerate(names)])
+        assert torch.equal(a, b)
+        engine.end(names); ref.end(names)
+        seen.append([k[0] for k in engine._graphs])
+    assert seen == [[1], [1, 3], [3, 6], [6, 1], [1, 8], [8, 3]]
+
+
 def test_captures_with_an_eager_collector(models):
     """The collector of cycles set to run at almost every allocation, engines built and dropped one
     after another, each capturing graphs of both kinds, some cyclic garbage that owns device
