@@ -482,25 +482,118 @@ __device__ __forceinline__ void page_values(const PageFrags<HD>& f, const f32x4 
   }
 }
 
+// ---- work dealt out by length.  With sequences of very unequal lengths in one step, the same
+// number of blocks for every (sequence, kv head) leaves the longest to a few blocks (64 sequences,
+// one of 131,072 tokens among 63 of 2,048: one block a pair, 512 pages a wave, 13.4 ms a step
+// where 3 would do).  Here the grid is flat, `budget` blocks and one more for every pair at most;
+// every block works out its share from the lengths in device memory, so the same captured graph
+// serves any lengths: the pages of all pairs are cut into chunks of C pages, C the least number
+// that keeps the chunks within the budget; pair (b, kvh) has c_b = ceil(pages_b / C) chunks, in
+// the order b, kvh, chunk.  A pair of one chunk writes its output itself; the others leave
+// partials [chunk, head of the group] that the merge kernel below finds by the same sums.
+__device__ __forceinline__ int attn_pages_of(int pos, int window, int& pg_first) {
+  const int kmin = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+  pg_first = kmin / PAGE;
+  return pos / PAGE - pg_first + 1;
+}
+
+__device__ __forceinline__ int wave_sum_int(int v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+// Pages of a chunk: from the lengths of all sequences.  Every lane returns the same.
+__device__ __forceinline__ int attn_chunk_pages(const int* __restrict__ seq_pos0, int n_seqs, int n_kv,
+                                                int window, int budget, int waves) {
+  const int lane = threadIdx.x & 63;
+  int total = 0, first;
+  for (int i = lane; i < n_seqs; i += 64) total += attn_pages_of(seq_pos0[i], window, first);
+  total = wave_sum_int(total);
+  const long long units = (long long)total * n_kv;
+  const int c = (int)((units + budget - 1) / budget);
+  return c > waves ? c : waves;
+}
+
+// Chunks (per kv head) of the sequences before sequence b, and of b itself.
+__device__ __forceinline__ void attn_chunks_before(const int* __restrict__ seq_pos0, int n_seqs, int window,
+                                                   int chunk, int b, int& before, int& mine) {
+  const int lane = threadIdx.x & 63;
+  int sum = 0, first;
+  for (int i = lane; i < b; i += 64) sum += (attn_pages_of(seq_pos0[i], window, first) + chunk - 1) / chunk;
+  before = wave_sum_int(sum);
+  mine = (attn_pages_of(seq_pos0[b], window, first) + chunk - 1) / chunk;
+}
+
+// The sequence whose chunks hold block g (counted over all kv heads), or -1 past the last chunk.
+__device__ __forceinline__ int attn_locate(const int* __restrict__ seq_pos0, int n_seqs, int n_kv, int window,
+                                           int chunk, int g, int& before, int& mine) {
+  const int lane = threadIdx.x & 63;
+  int run = 0, first;
+  for (int i0 = 0; i0 < n_seqs; i0 += 64) {
+    const int i = i0 + lane;
+    const int c = (i < n_seqs) ? (attn_pages_of(seq_pos0[i], window, first) + chunk - 1) / chunk : 0;
+    int incl = c;                                      // inclusive sums along the wave
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int up = __shfl_up(incl, off, 64);
+      if (lane >= off) incl += up;
+    }
+    const bool here = c > 0 && g >= n_kv * (run + incl - c) && g < n_kv * (run + incl);
+    const unsigned long long votes = __ballot(here);
+    if (votes) {
+      const int src = __ffsll((long long)votes) - 1;
+      before = run + __shfl(incl - c, src, 64);
+      mine = __shfl(c, src, 64);
+      return i0 + src;
+    }
+    run += __shfl(incl, 63, 64);
+  }
+  return -1;
+}
+
 template <int HD, int WAVES, bool AHEAD>
 __global__ __launch_bounds__(WAVES * 64, (HD <= 128) ? 2 : ((HD <= 192) ? 3 : 1)) void attn_decode_kernel(
     const bf16_t* __restrict__ q, int q_stride, const bf16_t* __restrict__ k_pages,
     const bf16_t* __restrict__ v_pages, const int* __restrict__ table, int table_stride,
     const int* __restrict__ seq_slot, const int* __restrict__ seq_pos0, float* __restrict__ part_o,
     float* __restrict__ part_ml, bf16_t* __restrict__ out, int n_heads, int n_kv, float scale_log2,
-    int window) {
+    int window, int budget, int n_seqs) {
   __shared__ float s_o[WAVES][HD][16];
   __shared__ float s_m[WAVES][16], s_l[WAVES][16];
-  const int blk = blockIdx.x, n_blk = gridDim.x, kvh = blockIdx.y, b = blockIdx.z;
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 15, g = lane >> 4;
   const int group = n_heads / n_kv;
+  // uniform: grid (blocks, n_kv, sequences), every pair cut into as many blocks;
+  // by length (budget > 0): a flat grid, see above
+  int blk = blockIdx.x, n_blk = gridDim.x, kvh = blockIdx.y, b = blockIdx.z;
+  int chunk = 0, chunk_id = 0;
+  if (budget > 0) {
+    chunk = attn_chunk_pages(seq_pos0, n_seqs, n_kv, window, budget, WAVES);
+    int before, mine;
+    b = attn_locate(seq_pos0, n_seqs, n_kv, window, chunk, blockIdx.x, before, mine);
+    if (b < 0) return;                               // past the last chunk (the whole block)
+    const int rest = blockIdx.x - n_kv * before;
+    kvh = rest / mine;
+    blk = rest % mine;
+    n_blk = mine;
+    chunk_id = blockIdx.x;
+  }
   const int pos = seq_pos0[b], slot = seq_slot[b];
   const int kmin = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
   const int pg_first = kmin / PAGE, pg_last = pos / PAGE;
-  const int n_waves = n_blk * WAVES;
-  const int per = (pg_last - pg_first + 1 + n_waves - 1) / n_waves;
-  const int p0 = pg_first + (blk * WAVES + wave) * per;
-  const int p1 = (p0 + per < pg_last + 1) ? p0 + per : pg_last + 1;
+  int p0, p1;
+  if (budget > 0) {
+    const int c0 = pg_first + blk * chunk;
+    const int c1 = (c0 + chunk < pg_last + 1) ? c0 + chunk : pg_last + 1;
+    const int per = (c1 - c0 + WAVES - 1) / WAVES;
+    p0 = c0 + wave * per;
+    p1 = (p0 + per < c1) ? p0 + per : c1;
+  } else {
+    const int n_waves = n_blk * WAVES;
+    const int per = (pg_last - pg_first + 1 + n_waves - 1) / n_waves;
+    p0 = pg_first + (blk * WAVES + wave) * per;
+    p1 = (p0 + per < pg_last + 1) ? p0 + per : pg_last + 1;
+  }
   const int* trow = table + (size_t)slot * table_stride;
 
   for (int hb = 0; hb < group; hb += 16) {
@@ -571,7 +664,8 @@ __global__ __launch_bounds__(WAVES * 64, (HD <= 128) ? 2 : ((HD <= 192) ? 3 : 1)
       if (n_blk == 1) {
         out[((size_t)b * n_heads + hh) * HD + d] = f32_to_bf16(o / l);
       } else {
-        const size_t idx = ((size_t)b * n_heads + hh) * n_blk + blk;
+        const size_t idx = (budget > 0) ? (size_t)chunk_id * group + hb + j
+                                        : ((size_t)b * n_heads + hh) * n_blk + blk;
         part_o[idx * HD + d] = o;
         if (d == 0) {
           part_ml[idx * 2] = m;
@@ -660,6 +754,58 @@ __global__ void attn_decode_combine_loop_kernel(const float* __restrict__ part_o
   out[((size_t)b * n_heads + h) * hd + d] = f32_to_bf16(ot / lt);
 }
 
+// The same where the work was dealt out by length: block (dims, G groups) for (head, sequence)
+// finds the pair's chunks by the sums that the attention kernel used; a pair of one chunk has
+// written its output already.
+template <int G>
+__global__ void attn_decode_combine_by_length_kernel(const float* __restrict__ part_o,
+                                                     const float* __restrict__ part_ml,
+                                                     const int* __restrict__ seq_pos0, bf16_t* __restrict__ out,
+                                                     int n_heads, int n_kv, int hd, int window, int budget,
+                                                     int waves, int n_seqs) {
+  __shared__ float s_m[G], s_l[G], s_o[G][256];
+  const int h = blockIdx.x, b = blockIdx.y, d = threadIdx.x, grp = threadIdx.y;
+  const int group = n_heads / n_kv, kvh = h / group;
+  const int chunk = attn_chunk_pages(seq_pos0, n_seqs, n_kv, window, budget, waves);
+  int before, mine;
+  attn_chunks_before(seq_pos0, n_seqs, window, chunk, b, before, mine);
+  if (mine == 1) return;
+  const size_t first = (size_t)n_kv * before + (size_t)kvh * mine;       // the pair's first chunk
+  const bool live = d < hd;
+  float m = -INFINITY, l = 0.f, o = 0.f;
+#pragma unroll 4
+  for (int s = grp; s < mine; s += G) {
+    const size_t idx = (first + s) * group + (h - kvh * group);
+    const float2 ml = *reinterpret_cast<const float2*>(part_ml + idx * 2);
+    const float ov = live ? part_o[idx * hd + d] : 0.f;
+    if (ml.x > -INFINITY) {
+      const float m_new = fmaxf(m, ml.x);
+      const float c_old = exp2f(m - m_new), c_new = exp2f(ml.x - m_new);   // exp2(-inf) = 0 at first
+      l = l * c_old + ml.y * c_new;
+      o = o * c_old + ov * c_new;
+      m = m_new;
+    }
+  }
+  if (d == 0) {
+    s_m[grp] = m;
+    s_l[grp] = l;
+  }
+  s_o[grp][d] = o;
+  __syncthreads();
+  if (grp != 0 || !live) return;
+  float mm = s_m[0];
+#pragma unroll
+  for (int gg = 1; gg < G; ++gg) mm = fmaxf(mm, s_m[gg]);
+  float lt = 0.f, ot = 0.f;
+#pragma unroll
+  for (int gg = 0; gg < G; ++gg) {
+    const float w = (s_m[gg] > -INFINITY) ? exp2f(s_m[gg] - mm) : 0.f;
+    lt += s_l[gg] * w;
+    ot += s_o[gg][d] * w;
+  }
+  out[((size_t)b * n_heads + h) * hd + d] = f32_to_bf16(ot / lt);
+}
+
 // ---------------------------------------------------------------------------------- entry points
 #define FOR_HEAD_DIMS(X) X(16) X(32) X(48) X(64) X(80) X(96) X(112) X(128) X(144) X(160) X(176) X(192) X(208) X(224) X(240) X(256)
 
@@ -716,18 +862,48 @@ extern "C" int llm_attention_prefill_bf16(const void* q, int q_stride, const voi
 }
 
 // part_o: [n_seqs, n_heads, n_blocks, hd] float32; part_ml: [n_seqs, n_heads, n_blocks, 2].
+// With budget > 0 the work is dealt out by the sequences' lengths instead (see the kernel):
+// n_blocks is not used, and the partials are [budget + n_seqs * n_kv, n_heads / n_kv, hd] and
+// [..., 2].
 extern "C" int llm_attention_decode_bf16(const void* q, int q_stride, const void* k_pages,
                                          const void* v_pages, const int* table, int table_stride,
                                          int page_size, const int* seq_slot, const int* seq_pos0,
                                          float* part_o, float* part_ml, void* out,
                                          int n_seqs, int n_heads, int n_kv, int hd, float scale,
-                                         int window, int n_blocks, hipStream_t stream) {
+                                         int window, int n_blocks, int budget, hipStream_t stream) {
   if (n_seqs <= 0) return LLM_OK;
   if (page_size != PAGE || !attn_args_ok(q, q_stride, k_pages, v_pages, n_heads, n_kv, hd, window) ||
-      n_blocks <= 0 || n_blocks > 1024 || n_kv > 65535 || n_seqs > 65535 || n_heads > 65535 || hd > 256)
+      n_blocks <= 0 || n_blocks > 1024 || n_kv > 65535 || n_seqs > 65535 || n_heads > 65535 || hd > 256 ||
+      budget < 0 || budget > (1 << 20))
     return LLM_ERR_ARG;
-  if (n_blocks > 1 && (!part_o || !part_ml)) return LLM_ERR_ARG;
+  if ((n_blocks > 1 || budget > 0) && (!part_o || !part_ml)) return LLM_ERR_ARG;
   const float scale_log2 = scale * 1.4426950408889634f;
+  if (budget > 0) {
+    const dim3 flat((unsigned)(budget + n_seqs * n_kv));
+    const dim3 cgrid(n_heads, n_seqs);
+    const int cthreads = ((hd + 63) / 64) * 64;
+#define CASE(D)                                                                                   \
+  if (hd == D) {                                                                                  \
+    constexpr int WAVES = (D > 192) ? 2 : 4;                                                      \
+    attn_decode_kernel<D, WAVES, false><<<flat, WAVES * 64, 0, stream>>>(                         \
+        (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, table,        \
+        table_stride, seq_slot, seq_pos0, part_o, part_ml, (bf16_t*)out, n_heads, n_kv,           \
+        scale_log2, window, budget, n_seqs);                                                      \
+    if (hipGetLastError() != hipSuccess) return LLM_ERR_LAUNCH;                                   \
+    if (cthreads <= 128)                                                                          \
+      attn_decode_combine_by_length_kernel<8><<<cgrid, dim3(cthreads, 8), 0, stream>>>(           \
+          part_o, part_ml, seq_pos0, (bf16_t*)out, n_heads, n_kv, hd, window, budget, WAVES,      \
+          n_seqs);                                                                                \
+    else                                                                                          \
+      attn_decode_combine_by_length_kernel<4><<<cgrid, dim3(cthreads, 4), 0, stream>>>(           \
+          part_o, part_ml, seq_pos0, (bf16_t*)out, n_heads, n_kv, hd, window, budget, WAVES,      \
+          n_seqs);                                                                                \
+    return llm_launch_status();                                                                   \
+  }
+    FOR_HEAD_DIMS(CASE)
+#undef CASE
+    return LLM_ERR_ARG;
+  }
   dim3 grid(n_blocks, n_kv, n_seqs);
   // pages overlapped within a wave where all blocks are resident at two a compute unit
   const bool ahead = hd <= 128 && (long long)n_blocks * n_kv * n_seqs <= 2LL * llm_compute_units();
@@ -738,12 +914,12 @@ extern "C" int llm_attention_decode_bf16(const void* q, int q_stride, const void
       attn_decode_kernel<D, WAVES, true><<<grid, WAVES * 64, 0, stream>>>(                        \
           (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, table,      \
           table_stride, seq_slot, seq_pos0, part_o, part_ml, (bf16_t*)out, n_heads, n_kv,         \
-          scale_log2, window);                                                                    \
+          scale_log2, window, 0, n_seqs);                                                         \
     else                                                                                          \
       attn_decode_kernel<D, WAVES, false><<<grid, WAVES * 64, 0, stream>>>(                       \
           (const bf16_t*)q, q_stride, (const bf16_t*)k_pages, (const bf16_t*)v_pages, table,      \
           table_stride, seq_slot, seq_pos0, part_o, part_ml, (bf16_t*)out, n_heads, n_kv,         \
-          scale_log2, window);                                                                    \
+          scale_log2, window, 0, n_seqs);                                                         \
     if (n_blocks > 1) {                                                                           \
       if (hipGetLastError() != hipSuccess) return LLM_ERR_LAUNCH;                                 \
       const dim3 cgrid(n_heads, n_seqs);                                                          \

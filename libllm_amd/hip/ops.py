@@ -53,7 +53,7 @@ _SIGNATURES = {
     "llm_attention_prefill_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _i, _i,
                                    _i, _i, _f, _i, _i, _vp],
     "llm_attention_decode_bf16": [_vp, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i,
-                                  _i, _i, _i, _f, _i, _i, _vp],
+                                  _i, _i, _i, _f, _i, _i, _i, _vp],
     "llm_attention_decode_waves": [_i],
     "llm_argmax": [_vp, _vp, _vp, _vp, _i, _i, _vp],
     "llm_argmax_parts": [_i],
@@ -853,13 +853,22 @@ class HipOps:
                 n_blocks = max(1, min(-(-pages // waves), max(1, budget // (m * n_kv))))
                 per_wave = -(-pages // (n_blocks * waves))
                 n_blocks = -(-pages // (per_wave * waves))
-                part_o = torch.empty((m, n_heads, n_blocks, hd), dtype=torch.float32, device=self.device)
-                part_ml = torch.empty((m, n_heads, n_blocks, 2), dtype=torch.float32, device=self.device)
+                by_length = 0
+                if getattr(ctx, "unequal", False) and m > 1:
+                    # lengths that differ widely: the kernel deals the pages out by the lengths it
+                    # finds in device memory, within so many blocks (and one more a pair at most)
+                    by_length, n_blocks = self.DECODE_BLOCKS, 1
+                    chunks = by_length + m * n_kv
+                    part_o = torch.empty((chunks, n_heads // n_kv, hd), dtype=torch.float32, device=self.device)
+                    part_ml = torch.empty((chunks, n_heads // n_kv, 2), dtype=torch.float32, device=self.device)
+                else:
+                    part_o = torch.empty((m, n_heads, n_blocks, hd), dtype=torch.float32, device=self.device)
+                    part_ml = torch.empty((m, n_heads, n_blocks, 2), dtype=torch.float32, device=self.device)
                 self._check(self.lib.llm_attention_decode_bf16(
                     qkv.data_ptr(), width, k_pages.data_ptr(), v_pages.data_ptr(),
                     table.data_ptr(), table.shape[1], 64, ctx.seq_slot.data_ptr(),
                     ctx.seq_pos0.data_ptr(), part_o.data_ptr(), part_ml.data_ptr(), out.data_ptr(), m, n_heads, n_kv, hd, float(scale),
-                    int(window), n_blocks, self._stream()), "attention_decode_bf16")
+                    int(window), n_blocks, by_length, self._stream()), "attention_decode_bf16")
             else:
                 tiles = self.prompt_tiles
                 if not tiles:

@@ -157,6 +157,7 @@ class StepContext:
         self.max_new = 0
         self.max_ctx = 0
         self.decode = False        # every sequence brings exactly one token
+        self.unequal = False       # a decode step whose sequences' cached lengths differ widely: work is then best dealt out by length, not by sequence
         # (stream tensor, weight, eps) while the next thing to read that stream is an RMS norm
         # with these, nothing else touching it in between: a product that adds into the stream
         # may then prepare that norm (``ops.linear(..., then_norm=)``).  Set by blocks.

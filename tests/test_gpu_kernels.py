@@ -1035,11 +1035,12 @@ def test_rope_pairing_and_sign(ops):
 
 # ------------------------------------------------------------------------------- attention
 def run_attention(ops, dtype, n_heads, n_kv, hd, seqs, window=0, seed=0, boost=None, fast=True, tiles=0,
-                  checked=None):
+                  checked=None, unequal=False):
     """seqs: (slot, past, new).  Returns (out, oracle) over all new tokens, or, with ``checked``,
     over that many rows of every sequence (its first and last, those next to every border of a
     block of 128 rows among them, the others drawn)."""
     ctx = make_ctx(ops, dtype, seqs)
+    ctx.unequal = unequal                              # decode attention deals its pages out by length
     pages = max((p + n + PAGE - 1) // PAGE for _, p, n in seqs)
     kv = make_kv("cuda", dtype, max(s for s, _, _ in seqs) + 1, pages, n_kv, hd, seed=seed)
     scale = hd ** -0.5
@@ -1050,7 +1051,8 @@ def run_attention(ops, dtype, n_heads, n_kv, hd, seqs, window=0, seed=0, boost=N
         vals = rnd((past + new, n_kv, hd), dtype, seed + 20 + slot)
         if boost is not None:                                       # one far key stands out
             key_pos, gain = boost
-            keys[key_pos] = keys[key_pos] * gain
+            if key_pos < past + new:                                # (a sequence too short for it has none)
+                keys[key_pos] = keys[key_pos] * gain
         fill_kv(kv, slot, keys, vals)
         which = range(new)
         if checked is not None and new > checked:
@@ -1206,6 +1208,43 @@ def test_a_build_whose_product_for_33_to_128_rows_spills_does_not_use_it(monkeyp
     assert not other.mid_gemm
     x, w = rnd((100, 256), torch.bfloat16, 1).cuda(), rnd((3200, 256), torch.bfloat16, 2).cuda()
     assert not other._mid_ok(x, other.prepare_weight(w), 100, 256)
+
+
+BY_LENGTH = {
+    "one long among short": [(0, 9000, 1), (1, 3, 1), (2, 70, 1), (3, 0, 1), (4, 64, 1)],
+    "two long": [(0, 5000, 1), (1, 63, 1), (2, 4999, 1)],
+    "all equal": [(i, 700, 1) for i in range(6)],
+    "all short": [(i, i, 1) for i in range(9)],
+    "seventy sequences": [(i, (37 * i) % 300 if i != 50 else 6000, 1) for i in range(70)],
+    "two hundred sequences": [(i, (53 * i) % 200 if i % 67 else 3000 + i, 1) for i in range(200)],
+}
+
+
+@pytest.mark.parametrize("case", list(BY_LENGTH))
+@pytest.mark.parametrize("shape", [(8, 2, 64), (4, 4, 128), (20, 1, 32), (2, 1, 256), (6, 3, 176)])
+def test_attention_decode_by_length(ops, case, shape):
+    """Decode attention with its pages dealt out by the sequences' lengths (a flat grid, every
+    block finding its share from the lengths in device memory): one long sequence among short
+    ones, equal ones, more sequences than a wave has lanes; groups of 4, 1 and 20 heads, heads of
+    32 to 256 dims; against the per-query oracle, and the same bits as the uniform grid gives
+    where a pair is one chunk in both."""
+    n_heads, n_kv, hd = shape
+    seqs = BY_LENGTH[case]
+    if hd >= 176:
+        seqs = seqs[:40]                                  # (the oracle is slow)
+    out, ref = run_attention(ops, torch.bfloat16, n_heads, n_kv, hd, seqs, seed=len(seqs) + hd, unequal=True)
+    assert max_err(out, ref) < BF16_2ULP
+    far = max(range(len(seqs)), key=lambda i: seqs[i][1])
+    out, ref = run_attention(ops, torch.bfloat16, n_heads, n_kv, hd, seqs, seed=hd, unequal=True,
+                             boost=(seqs[far][1] // 2, 12.0))
+    assert max_err(out, ref) < BF16_2ULP
+
+
+@pytest.mark.parametrize("window", [0, 100, 4096])
+def test_attention_decode_by_length_with_a_window(ops, window):
+    seqs = [(0, 9000, 1), (1, 3, 1), (2, 70, 1), (3, 5000, 1), (4, 64, 1)]
+    out, ref = run_attention(ops, torch.bfloat16, 8, 2, 64, seqs, window=window, seed=5, unequal=True)
+    assert max_err(out, ref) < BF16_2ULP
 
 
 @pytest.mark.parametrize("hd", [144, 160, 176, 192, 208, 224, 240, 256])

@@ -297,6 +297,30 @@ def test_batches_of_more_than_128_requests(long_models, tmp_path, case):
     check("long" + name, cfg, weights, group, traces.collect(steps, str(tmp_path), cfg.vocab), dtype)
 
 
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("use_graphs", [True, False])
+def test_a_long_request_among_short_ones(long_models, tmp_path, monkeypatch, dtype, use_graphs):
+    """One request of two thousand tokens decodes beside nine of a few dozen: such a step is run
+    with its decode attention dealt out by length (a graph of its own kind), and when the long
+    request has ended the others go on in the uniform kind; every position against the plain
+    implementation."""
+    from libllm_amd.engine import Engine
+    monkeypatch.setattr(Engine, "UNEQUAL_MIN", 512)          # (the tiny configurations stop far below 4,096 tokens)
+    path, cfg, weights = long_models["B"]
+    rng = np.random.default_rng(77)
+    group = {"long": rng.integers(0, cfg.vocab, size=2050).tolist()}
+    group.update({"s%d" % i: rng.integers(0, cfg.vocab, size=int(n)).tolist() for i, n in enumerate(rng.integers(20, 70, size=9))})
+    tails = {r: 18 for r in group}
+    tails["long"] = 6                                           # it ends first; the short ones decode on
+    steps = traces.batches([group], tails)
+    for i, s in enumerate(steps):
+        s["step"] = i
+    engine = run_replay(path, dtype, steps, tmp_path, max_tokens=traces.max_tokens_needed(steps), use_graphs=use_graphs)
+    if use_graphs:
+        assert {k[2] for k in engine._graphs} == {True, False}      # graphs of both kinds were made
+    check("long" + "B", cfg, weights, group, traces.collect(steps, str(tmp_path), cfg.vocab), dtype)
+
+
 BENCH_SHAPES = {
     "1b": dict(hidden_size=2048, num_attention_heads=32, num_key_value_heads=8, head_dim=64,
                intermediate_size=8192, tie_word_embeddings=True, factor=32.0),
@@ -601,7 +625,7 @@ def test_a_captured_step_whose_replay_differs_is_not_used(models, monkeypatch):
     with pytest.warns(UserWarning, match="run without a captured graph"):
         got = _decode_rows(engine, requests, 4)
     assert len(calls) == 1 and not engine._graphs
-    assert engine._no_graph == {("decode", 3, 128)}         # (the position limit of this configuration is 128)
+    assert engine._no_graph == {("decode", 3, 128, False)}  # (the position limit of this configuration is 128; lengths not far apart)
     assert np.array_equal(got, want)
 
 
