@@ -5,6 +5,7 @@ decoding at batch 1, 64 and 256.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--layers L] [--batch B] [--context C]
     python bench.py --sweep            # decode at batch 1..256 x context 4,096..131,072, as a table
+    python bench.py --unequal          # decode steps of batches whose contexts differ widely
 
 A step is one decode step inside the generation loop (``Generator.stream``, the loop that serves
 requests): the step function over the cache as a captured graph, arg-max sampling on the device,
@@ -295,6 +296,65 @@ def run_sweep(args, torch):
     return 0
 
 
+UNEQUAL_CASES = (
+    ("8x16384", [16384] * 8), ("1x131072", [131072]), ("1x131072_7x128", [131072] + [128] * 7),
+    ("64x4096", [4096] * 64), ("1x131072_63x2048", [131072] + [2048] * 63), ("8x32768_56x256", [32768] * 8 + [256] * 56),
+    ("64x64to8128", [64 + 128 * i for i in range(64)]),
+)
+
+
+def run_unequal(args, torch):
+    """Decode steps of batches whose sequences hold very different numbers of tokens, beside
+    batches of like lengths with about as many bytes, each with its bytes / time against 8 TB/s
+    (the cache's books are filled as in the sweep).  Decode attention sizes its grid by the
+    longest sequence of a step unless the lengths differ widely; then it deals the pages out by
+    length."""
+    from libllm_amd.config import config_from_dict
+    from libllm_amd.engine import StepEntry
+    from libllm_amd.runtime import random_engine
+    d = dict(FULL)
+    d.update(SHAPES[args.shape])
+    cfg = config_from_dict(d)
+    itemsize = 2 if args.dtype == "bfloat16" else 4
+    per_token = kv_bytes_per_token(cfg, itemsize)
+    max_tokens = max(sum(c + 64 for c in ctxs) for _, ctxs in UNEQUAL_CASES)
+    engine = random_engine(cfg, seed=0, dtype=args.dtype, max_tokens=max_tokens, max_slots=64)
+    for g in engine.cache.groups:
+        for plane in g.planes.values():
+            plane.normal_()
+    steps, warmup = min(args.steps, 32), min(args.warmup, 8)        # (the shortest sequences end at 128 tokens)
+    points = {}
+    for name, ctxs in UNEQUAL_CASES:
+        ids = [("unequal", name, i) for i in range(len(ctxs))]
+        for r, c in zip(ids, ctxs):                           # the books only: pages and lengths, no prompt step
+            slot = engine.cache.admit(r)
+            engine.cache.reserve(slot, c - steps - warmup - 1)
+            engine.cache.commit(slot, c - steps - warmup - 1)
+        engine.cache.flush()
+        tokens = torch.zeros((len(ids),), dtype=torch.int32, device=engine.device)
+        entries = [StepEntry(r, [0], [0]) for r in ids]
+        for k in range(warmup + steps):
+            if k == warmup:
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+            tokens = engine.ops.argmax(engine.step(entries, tokens_device=tokens))
+        torch.cuda.synchronize()
+        dt = (time.perf_counter() - t0) / steps
+        engine.end(ids)
+        frac = (weight_bytes(cfg, itemsize) + (sum(ctxs) - len(ctxs) * steps / 2.0) * per_token) / dt / HBM_BYTES_PER_S
+        points[name + "_ms"] = round(dt * 1e3, 3)
+        points[name + "_hbm_frac"] = round(frac, 4)
+        log("%-20s %.3f ms a step, %.2f of 8 TB/s" % (name, dt * 1e3, frac))
+    print(json.dumps({
+        "metric": "decode ms a step over batches of unequal contexts (%s)" % NAMES[args.shape],
+        "value": points["1x131072_63x2048_ms"], "unit": "ms", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": points["1x131072_63x2048_ms"], "higher_is_better": False, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if itemsize == 2 else "fp32", "data": "synthetic: random cache contents, random weights N(0, 0.02)",
+        "config": {"model": NAMES[args.shape], "layers": cfg.num_hidden_layers, "sampling": "greedy"},
+        "points": points}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -313,6 +373,8 @@ def main() -> int:
                     help="run a generation workload through the generation loop instead")
     ap.add_argument("--sweep", action="store_true",
                     help="decode steps at batch 1 to 256 and contexts of 4,096 to 131,072 tokens, as a table")
+    ap.add_argument("--unequal", action="store_true",
+                    help="decode steps of batches whose sequences hold very different numbers of tokens")
     ap.add_argument("--no-workloads", action="store_true",
                     help="skip the generation workloads of the 3B and 8B shapes")
     args = ap.parse_args()
@@ -326,6 +388,8 @@ def main() -> int:
         return run_workload(args, torch)
     if args.sweep:
         return run_sweep(args, torch)
+    if args.unequal:
+        return run_unequal(args, torch)
 
     from libllm_amd.cache import PAGE
     from libllm_amd.config import config_from_dict
