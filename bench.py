@@ -303,6 +303,30 @@ UNEQUAL_CASES = (
 )
 
 
+def time_contexts(engine, torch, name, ctxs, steps, warmup):
+    """Seconds a decode step of sequences that end at ``ctxs`` tokens takes: the cache's books are
+    filled without prompt steps (pages and lengths only), then the step function decodes, arg-max
+    on the device and the tokens fed back without the host reading them."""
+    from libllm_amd.engine import StepEntry
+    ids = [("contexts", name, i) for i in range(len(ctxs))]
+    for r, c in zip(ids, ctxs):
+        slot = engine.cache.admit(r)
+        engine.cache.reserve(slot, c - steps - warmup - 1)
+        engine.cache.commit(slot, c - steps - warmup - 1)
+    engine.cache.flush()
+    tokens = torch.zeros((len(ids),), dtype=torch.int32, device=engine.device)
+    entries = [StepEntry(r, [0], [0]) for r in ids]
+    for k in range(warmup + steps):
+        if k == warmup:
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+        tokens = engine.ops.argmax(engine.step(entries, tokens_device=tokens))
+    torch.cuda.synchronize()
+    dt = (time.perf_counter() - t0) / steps
+    engine.end(ids)
+    return dt
+
+
 def run_unequal(args, torch):
     """Decode steps of batches whose sequences hold very different numbers of tokens, beside
     batches of like lengths with about as many bytes, each with its bytes / time against 8 TB/s
@@ -325,22 +349,7 @@ def run_unequal(args, torch):
     steps, warmup = min(args.steps, 32), min(args.warmup, 8)        # (the shortest sequences end at 128 tokens)
     points = {}
     for name, ctxs in UNEQUAL_CASES:
-        ids = [("unequal", name, i) for i in range(len(ctxs))]
-        for r, c in zip(ids, ctxs):                           # the books only: pages and lengths, no prompt step
-            slot = engine.cache.admit(r)
-            engine.cache.reserve(slot, c - steps - warmup - 1)
-            engine.cache.commit(slot, c - steps - warmup - 1)
-        engine.cache.flush()
-        tokens = torch.zeros((len(ids),), dtype=torch.int32, device=engine.device)
-        entries = [StepEntry(r, [0], [0]) for r in ids]
-        for k in range(warmup + steps):
-            if k == warmup:
-                torch.cuda.synchronize()
-                t0 = time.perf_counter()
-            tokens = engine.ops.argmax(engine.step(entries, tokens_device=tokens))
-        torch.cuda.synchronize()
-        dt = (time.perf_counter() - t0) / steps
-        engine.end(ids)
+        dt = time_contexts(engine, torch, name, ctxs, steps, warmup)
         frac = (weight_bytes(cfg, itemsize) + (sum(ctxs) - len(ctxs) * steps / 2.0) * per_token) / dt / HBM_BYTES_PER_S
         points[name + "_ms"] = round(dt * 1e3, 3)
         points[name + "_hbm_frac"] = round(frac, 4)
@@ -443,6 +452,15 @@ def main() -> int:
             bytes_b = weight_bytes(cfg, itemsize) + b * mean_ctx * kv_bytes_per_token(cfg, itemsize)
             points["decode_b%d_hbm_frac" % b] = round(bytes_b / (dtb / args.steps) / HBM_BYTES_PER_S, 4)
             log("decode at batch %d: %.3f ms a step, %.0f tokens/s" % (b, dtb / args.steps * 1e3, b * args.steps / dtb))
+    if 256 in point_batches:
+        # one sequence of 131,072 tokens among 63 of 2,048 (the cache for batch 256 holds them): decode
+        # attention deals such a step's pages out by length
+        ctxs = [131072] + [2048] * 63
+        dtu = time_contexts(engine, torch, "unequal64", ctxs, 32, 8)
+        points["decode_1x131072_63x2048_ms_per_step"] = round(dtu * 1e3, 3)
+        points["decode_1x131072_63x2048_hbm_frac"] = round(
+            (weight_bytes(cfg, itemsize) + (sum(ctxs) - 64 * 16) * kv_bytes_per_token(cfg, itemsize)) / dtu / HBM_BYTES_PER_S, 4)
+        log("decode of 1 x 131,072 + 63 x 2,048 tokens: %.3f ms a step" % (dtu * 1e3))
     if not (args.no_points or args.no_workloads) and args.shape == "1b" and args.layers == layers_full:
         # the family's other two shapes with the workloads named for them, each on an engine of its own
         del gen, engine
