@@ -364,6 +364,55 @@ def run_unequal(args, torch):
     return 0
 
 
+def run_requests(args, torch):
+    """Many requests of mixed lengths through the generation loop, more than a batch holds: prompt
+    lengths log-normal (median about 240 tokens, clipped to [4, 6000]) with four long ones of
+    12,000 to 50,000, greedy, at most 256 new tokens, and stop tokens drawn so that a reply ends
+    after about 200 tokens on average (random weights give a near-uniform next token).  The loop
+    forms batch after batch, shorter replies end earlier, slots and pages are used again.  The
+    second of two runs counts (the first captures the graphs of the shapes that come up)."""
+    import numpy as np
+    from libllm_amd.cache import PAGE
+    from libllm_amd.config import config_from_dict
+    from libllm_amd.engine import Generator
+    from libllm_amd.runtime import random_engine
+    from libllm_amd.sampling import Sampler, SamplingParams
+    d = dict(FULL)
+    d.update(SHAPES[args.shape])
+    d["eos_token_id"] = None
+    cfg = config_from_dict(d)
+    rng = np.random.default_rng(0)
+    n, new = args.requests, 256
+    lens = np.clip(np.exp(rng.normal(5.5, 1.2, size=n)).astype(int), 4, 6000)
+    lens[rng.integers(0, n, size=4)] = [30000, 50000, 12000, 20000]
+    prompts = [rng.integers(0, cfg.vocab_size, size=int(l)).tolist() for l in lens]
+    stop = tuple(int(t) for t in rng.integers(0, cfg.vocab_size, size=cfg.vocab_size // 200))
+    engine = random_engine(cfg, seed=0, dtype=args.dtype, max_tokens=2_000_000, max_slots=args.max_batch)
+    gen = Generator(engine, Sampler(engine.ops, cfg.vocab_size), stop, cfg.max_position_embeddings,
+                    engine.cache.n_pages, PAGE, max_batch=args.max_batch)
+    log("%d requests, %d prompt tokens (median %d, longest %d), batches of at most %d"
+        % (n, lens.sum(), np.median(lens), lens.max(), args.max_batch))
+    for rep in range(2):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        out = gen.generate(prompts, SamplingParams(temperature=0.0), max_new_tokens=new)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        n_out = sum(len(o) for o in out)
+        log("run %d: %.2f s, %d new tokens, %.0f generated tok/s, %.0f tok/s with the prompts' tokens"
+            % (rep, dt, n_out, n_out / dt, (n_out + lens.sum()) / dt))
+    print(json.dumps({
+        "metric": "generated tok/s over %d requests of mixed lengths (%s)" % (n, NAMES[args.shape]),
+        "value": round(n_out / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": None, "warmup": None,
+        "ms_per_step": None, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+        "data": "synthetic: uniform random token ids, random weights N(0, 0.02)",
+        "config": {"model": NAMES[args.shape], "layers": cfg.num_hidden_layers, "requests": n, "max_batch": args.max_batch,
+                   "prompt_tokens": int(lens.sum()), "new_tokens": n_out, "max_new_tokens": new, "sampling": "greedy"},
+        "points": {"seconds": round(dt, 3), "tok_s_with_prompts": round((n_out + lens.sum()) / dt, 1)}}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -384,6 +433,9 @@ def main() -> int:
                     help="decode steps at batch 1 to 256 and contexts of 4,096 to 131,072 tokens, as a table")
     ap.add_argument("--unequal", action="store_true",
                     help="decode steps of batches whose sequences hold very different numbers of tokens")
+    ap.add_argument("--requests", type=int, default=0,
+                    help="run so many requests of mixed lengths through the generation loop instead")
+    ap.add_argument("--max-batch", type=int, default=256, help="the largest batch of --requests")
     ap.add_argument("--no-workloads", action="store_true",
                     help="skip the generation workloads of the 3B and 8B shapes")
     args = ap.parse_args()
@@ -399,6 +451,8 @@ def main() -> int:
         return run_sweep(args, torch)
     if args.unequal:
         return run_unequal(args, torch)
+    if args.requests:
+        return run_requests(args, torch)
 
     from libllm_amd.cache import PAGE
     from libllm_amd.config import config_from_dict
