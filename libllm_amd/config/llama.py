@@ -8,8 +8,8 @@ hidden_act == "silu" (tools/llama_exporter.py:87-88).  Keys the reference bakes 
 exported rotary table are read here directly: rope_theta, rope_scaling, head_dim,
 tie_word_embeddings.
 """
-from dataclasses import dataclass, field
-from typing import Any, Dict, List, Optional, Tuple
+from dataclasses import dataclass
+from typing import Any, Dict, Optional, Tuple
 
 from ..errors import ConfigError
 from ..parts.attention import AttentionSpec

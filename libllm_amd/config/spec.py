@@ -8,7 +8,7 @@ sees the configuration class or the architecture's name.
 Each kind of part defines its own record type next to its implementation (for instance
 ``AttentionSpec`` beside the attention mixer); the records here are the ones every model has.
 """
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, List, Optional, Tuple
 
 from ..errors import ConfigError

@@ -12,7 +12,7 @@ from typing import Callable, Iterable, List, Optional, Sequence
 import torch
 
 from ..errors import RequestError
-from ..sampling import Sampler, SamplingParams
+from ..sampling import SamplingParams
 from .step import StepEntry
 
 

@@ -4,7 +4,7 @@ This class is the same for every architecture; what differs between architecture
 ModelSpec their configuration produces (src/libllm/llama.cc:273-312 is the reference's fixed
 counterpart for Llama).
 """
-from typing import Dict, List, Optional
+from typing import Dict, Optional
 
 import torch
 

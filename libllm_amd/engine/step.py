@@ -7,7 +7,7 @@ points for one sequence, prefill and decode (src/libllm/llama.cc:349-368); this 
 generalisation to unequal batches.
 """
 import warnings
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Dict, Hashable, List, Optional, Sequence
 
 import numpy as np

@@ -6,7 +6,7 @@ head h reading kv head h // (n_heads / n_kv_heads) (src/flint/operators.cc:43-56
 heads, output product.  Here the rotation and the cache write are one kernel, and attention reads
 keys and values from the cache for whole prompts and single tokens alike.
 """
-from dataclasses import dataclass, field
+from dataclasses import dataclass
 from typing import Optional
 
 import torch

@@ -8,7 +8,7 @@ large file is never held in host memory whole.
 import json
 import os
 import struct
-from typing import Dict, List, Optional, Tuple
+from typing import Dict, Optional
 
 import numpy as np
 import torch

@@ -14,7 +14,7 @@ from libllm_amd.config import ScheduleEntry, config_from_dict
 from libllm_amd.engine import DecoderModel, Engine, StepEntry
 from libllm_amd.engine.trace import replay
 from libllm_amd.runtime import load_engine
-from libllm_amd.weights import load_tensors, random_tensors
+from libllm_amd.weights import random_tensors
 from plain import files, llama, sampling
 from tiny import TINY_A, TINY_B, TINY_C, make_model
 

@@ -10,8 +10,7 @@ import torch
 from libllm_amd import WeightError
 from libllm_amd.config import config_from_dict
 from libllm_amd.engine import DecoderModel
-from libllm_amd.weights import (SafetensorsFile, load_tensors, open_model_files, write_random_model,
-                                write_safetensors)
+from libllm_amd.weights import SafetensorsFile, load_tensors, open_model_files, write_safetensors
 from plain import files
 from tiny import TINY_A, TINY_B, TINY_C, make_model
 
