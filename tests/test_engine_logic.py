@@ -90,6 +90,32 @@ def test_generation_matches_plain(models):
     assert [c.token_id for c in chunks if c.token_id is not None] == sampling.generate(cfg, weights, prompts[1], 3)
 
 
+@pytest.mark.parametrize("seed", range(6))
+def test_generation_of_drawn_requests_matches_plain(models, seed):
+    """Requests, batch size, cache size, the bound on a prompt step's rows and stop tokens drawn at
+    random: every reply is what the plain implementation gives for that prompt alone, and the
+    cache's books are whole afterwards."""
+    path, cfg, weights = models["ABC"[seed % 3]]
+    rng = np.random.default_rng(100 + seed)
+    n = int(rng.integers(1, 10))
+    new = int(rng.integers(1, 7))
+    prompts = [rng.integers(0, cfg.vocab, size=int(l)).tolist() for l in rng.integers(1, 90, size=n)]
+    longest = max(len(p) for p in prompts) + new
+    max_tokens = int(rng.integers(1, 4)) * (-(-longest // 64) * 64)              # room for one to three of the longest
+    stop = rng.integers(0, cfg.vocab, size=cfg.vocab // 6).tolist()               # ends about every sixth token
+    model = Model(path, dtype="float32", max_tokens=max_tokens, ops=CpuOps(), max_batch=int(rng.integers(1, 6)),
+                  max_prompt_rows=int(rng.integers(16, 120)))
+    for temperature in (0.0, 0.9):
+        got = model.generate(prompts, max_new_tokens=new, temperature=temperature, top_k=40, top_p=0.9, seed=seed,
+                             stop_tokens=stop)
+        want = [sampling.generate(cfg, weights, p, new, temperature, 40, 0.9, seed=seed, stream=i, stop=stop)
+                for i, p in enumerate(prompts)]
+        assert got == want
+        model.engine.cache.check()
+        assert model.engine.cache.slots.n_free == model.engine.cache.slots.n_slots
+        assert not model.engine.live_requests()
+
+
 def test_messages_become_the_architectures_chat_format(models, tmp_path):
     """The messages of a chat, block by block as the reference's model class appends them
     (src/libllm/llama.cc:406-442), where the tokenizer beside the model knows the control tokens;
