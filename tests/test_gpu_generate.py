@@ -96,6 +96,33 @@ def test_greedy_generation_of_two_hundred_requests_with_stop_tokens(model_b):
     assert model.engine.cache.slots.n_free == model.engine.cache.slots.n_slots
 
 
+@pytest.mark.parametrize("seed", range(4))
+def test_greedy_generation_of_drawn_requests(model_b, seed):
+    """Requests, batch size, cache size, the bound on a prompt step's rows and stop tokens drawn at
+    random, in 32-bit: every reply is what the plain implementation gives for that prompt alone
+    (but for a tie closer than 1e-4), and the cache's books are whole afterwards."""
+    from libllm_amd import Model
+    path, cfg, weights = model_b
+    rng = np.random.default_rng(200 + seed)
+    n, new = int(rng.integers(2, 12)), int(rng.integers(2, 10))
+    prompts = [rng.integers(0, cfg.vocab, size=int(l)).tolist() for l in rng.integers(1, 100, size=n)]
+    longest = max(len(p) for p in prompts) + new
+    stop = rng.integers(0, cfg.vocab, size=cfg.vocab // 8).tolist()
+    model = Model(path, dtype="float32", max_tokens=int(rng.integers(1, 4)) * (-(-longest // 64) * 64),
+                  max_batch=int(rng.integers(1, 6)), max_prompt_rows=int(rng.integers(16, 120)))
+    for rep in range(2):                                # the second time through captured graphs of the same shapes
+        got = model.generate(prompts, max_new_tokens=new, temperature=0.0, stop_tokens=stop)
+        want = [sampling.generate(cfg, weights, p, new, stop=stop) for p in prompts]
+        for p, g, w in zip(prompts, got, want):
+            if g != w:
+                k = next(k for k in range(max(len(g), len(w))) if k >= len(g) or k >= len(w) or g[k] != w[k])
+                top = np.sort(llama.logits_all(cfg, weights, list(p) + w[:k])[-1])
+                assert top[-1] - top[-2] < 1e-4
+        model.engine.cache.check()
+        assert model.engine.cache.slots.n_free == model.engine.cache.slots.n_slots
+        assert not model.engine.live_requests()
+
+
 def test_sampled_generation_and_stop_tokens(model_b):
     from libllm_amd import Model
     path, cfg, weights = model_b
