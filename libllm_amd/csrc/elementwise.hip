@@ -362,17 +362,24 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride, const 
 // and their four angles at a time).  v is transposed through LDS, so that consecutive lanes write
 // consecutive positions of a page: rows of a prompt lie in order, and a wave's 64 stores of two
 // bytes then fall into two half lines instead of 64 lines.  Needs hd and rot_dim in multiples of 8.
+// Rows of a decode step lie in as many pages, so their values' stores are a line each whatever the
+// order: for few rows a v head is dealt to v_split blocks, each with hd / v_split of its dims
+// (grid: row tiles x (q heads + k heads + v heads * v_split)).
 template <int PAGE>
 __global__ __launch_bounds__(256) void rope_kv_write_tile_kernel(
     bf16_t* __restrict__ qkv, int row_stride, const float* __restrict__ bias, int n_heads, int n_kv, int hd,
     const float* __restrict__ cos_t, const float* __restrict__ sin_t, int rot_dim,
     const int* __restrict__ tok_pos, const int* __restrict__ tok_seq, const int* __restrict__ seq_slot,
     const int* __restrict__ table, int table_stride, bf16_t* __restrict__ k_pages,
-    bf16_t* __restrict__ v_pages, int M) {
+    bf16_t* __restrict__ v_pages, int M, int v_split) {
   extern __shared__ __attribute__((aligned(16))) unsigned char tile_raw[];
   __shared__ int s_pos[64], s_page[64];
-  const int tid = threadIdx.x, m0 = blockIdx.x * 64, h = blockIdx.y;
-  const bool is_q = h < n_heads, is_k = !is_q && h < n_heads + n_kv;
+  const int tid = threadIdx.x, m0 = blockIdx.x * 64;
+  const bool is_q = (int)blockIdx.y < n_heads, is_k = !is_q && (int)blockIdx.y < n_heads + n_kv;
+  // the head whose columns of a row this block takes, and for a v head which of its dims
+  const int v_block = (int)blockIdx.y - n_heads - n_kv;
+  const int h = (is_q || is_k) ? (int)blockIdx.y : n_heads + n_kv + v_block / v_split;
+  const int dims = (is_q || is_k) ? hd : hd / v_split, d0 = (is_q || is_k) ? 0 : (v_block % v_split) * dims;
   if (tid < 64) {
     const int m = m0 + tid;
     int pos = 0, page = 0;
@@ -431,17 +438,18 @@ __global__ __launch_bounds__(256) void rope_kv_write_tile_kernel(
   // a column is read without bank conflicts), then one dim a wave at a time, a row a lane
   const int kvh = h - n_heads - n_kv;
   uint32_t* tile = reinterpret_cast<uint32_t*>(tile_raw);
-  const int row_w = hd / 2 + 1;                                    // words per row of the tile
-  for (int it = tid; it < 64 * vecs; it += 256) {
-    const int r = it / vecs, d = (it % vecs) * 8, m = m0 + r;
+  const int row_w = dims / 2 + 1;                                  // words per row of the tile
+  const int vecs_v = dims / 8;
+  for (int it = tid; it < 64 * vecs_v; it += 256) {
+    const int r = it / vecs_v, d = (it % vecs_v) * 8, m = m0 + r;
     uint4 raw = make_uint4(0u, 0u, 0u, 0u);
-    if (m < M) raw = *reinterpret_cast<const uint4*>(qkv + (size_t)m * row_stride + (size_t)h * hd + d);
+    if (m < M) raw = *reinterpret_cast<const uint4*>(qkv + (size_t)m * row_stride + (size_t)h * hd + d0 + d);
     uint32_t w[4] = {raw.x, raw.y, raw.z, raw.w};
     if (b) {
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
-        const float lo = bf16_to_f32((bf16_t)(w[e] & 0xffffu)) + b[d + 2 * e];
-        const float hi = bf16_to_f32((bf16_t)(w[e] >> 16)) + b[d + 2 * e + 1];
+        const float lo = bf16_to_f32((bf16_t)(w[e] & 0xffffu)) + b[d0 + d + 2 * e];
+        const float hi = bf16_to_f32((bf16_t)(w[e] >> 16)) + b[d0 + d + 2 * e + 1];
         w[e] = (uint32_t)f32_to_bf16(lo) | ((uint32_t)f32_to_bf16(hi) << 16);
       }
     }
@@ -453,9 +461,9 @@ __global__ __launch_bounds__(256) void rope_kv_write_tile_kernel(
   if (m0 + lane < M) {
     const int pos = s_pos[lane];
     bf16_t* dst = v_pages + ((size_t)s_page[lane] * n_kv + kvh) * llm_value_block(hd);
-    for (int d = wave; d < hd; d += 4) {
+    for (int d = wave; d < dims; d += 4) {
       const uint32_t w = tile[lane * row_w + d / 2];
-      dst[llm_value_offset(hd, d, pos % PAGE)] = (bf16_t)((d & 1) ? (w >> 16) : (w & 0xffffu));
+      dst[llm_value_offset(hd, d0 + d, pos % PAGE)] = (bf16_t)((d & 1) ? (w >> 16) : (w & 0xffffu));
     }
   }
 }
@@ -479,11 +487,13 @@ extern "C" int llm_rope_kv_write(void* qkv, int dtype, int row_stride, const flo
                       ((uintptr_t)cos_t & 15) == 0 && ((uintptr_t)sin_t & 15) == 0 &&
                       (!write_kv || ((uintptr_t)k_pages & 15) == 0) && M >= 64;
   if (vec_ok) {
-    const dim3 grid((M + 63) / 64, n_heads + (write_kv ? 2 * n_kv : 0));
-    const size_t lds = write_kv ? (size_t)64 * (hd / 2 + 1) * 4 : 0;
+    // few rows (a decode step's, a short prompt's): more blocks for the values, see the kernel
+    const int v_split = (M > 256) ? 1 : (hd % 32 == 0) ? 4 : (hd % 16 == 0) ? 2 : 1;
+    const dim3 grid((M + 63) / 64, n_heads + (write_kv ? n_kv + n_kv * v_split : 0));
+    const size_t lds = write_kv ? (size_t)64 * (hd / v_split / 2 + 1) * 4 : 0;
     rope_kv_write_tile_kernel<64><<<grid, 256, lds, stream>>>(
         (bf16_t*)qkv, row_stride, bias, n_heads, n_kv, hd, cos_t, sin_t, rot_dim, tok_pos, tok_seq, seq_slot,
-        table, table_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, M);
+        table, table_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, M, v_split);
     return llm_launch_status();
   }
   if (dtype == LLM_DTYPE_F32)

@@ -967,13 +967,19 @@ def test_projection_with_rotation_and_cache_write(ops, dtype, shape, bias, seqs)
 @pytest.mark.parametrize("shape", [(4, 2, 16, 16), (6, 3, 48, 24), (5, 1, 64, 64), (8, 2, 128, 128), (2, 2, 256, 64),
                                    (3, 1, 32, 0)])
 @pytest.mark.parametrize("bias", [False, True])
-def test_rope_kv_write_on_many_rows(ops, shape, bias):
-    """Prompts of many rows in bfloat16 with neighbouring pairs take a kernel of their own (tiles
-    of 64 rows, v transposed through LDS): several sequences that cross page borders, a last tile
-    that is not full, partial rotation; and nothing beside the new positions is written."""
+@pytest.mark.parametrize("seqs", [
+    [(2, 0, 70), (0, 61, 9), (1, 130, 50), (3, 5, 31)],            # 160 rows: two tiles and a half
+    [(2, 0, 200), (0, 61, 90), (1, 130, 60)],                      # 350 rows: a v head is one block's again
+    [(i, (37 * i) % 250, 1) for i in range(70)],                   # a decode step: every row in a page of its own
+], ids=["160rows", "350rows", "70decode"])
+def test_rope_kv_write_on_many_rows(ops, shape, bias, seqs):
+    """Steps of 64 rows and more in bfloat16 with neighbouring pairs take a kernel of their own (tiles
+    of 64 rows, v transposed through LDS, a v head dealt to several blocks where the rows are few):
+    several sequences that cross page borders, a last tile that is not full, partial rotation, rows of
+    as many sequences; and nothing beside the new positions is written."""
     n_heads, n_kv, hd, rot = shape
     dtype = torch.bfloat16
-    seqs = [(2, 0, 70), (0, 61, 9), (1, 130, 50), (3, 5, 31)]      # 160 rows: two tiles and a half
+    n_slots = max(slot for slot, _, _ in seqs) + 1
     ctx = make_ctx(ops, dtype, seqs)
     m = ctx.n_tokens
     width = (n_heads + 2 * n_kv) * hd
@@ -995,7 +1001,7 @@ def test_rope_kv_write_on_many_rows(ops, shape, bias):
         heads[..., half:rot] = x2 * c + x1 * s_
     v_ref = x[:, (n_heads + n_kv) * hd:].reshape(m, n_kv, hd)
     for write in (True, False):
-        kv = make_kv("cuda", dtype, 4, 4, n_kv, hd, seed=1)
+        kv = make_kv("cuda", dtype, n_slots, 4, n_kv, hd, seed=1)
         cols = width if write else n_heads * hd                     # queries alone when nothing is written
         qkv = nat[:, order][:, :cols].contiguous().cuda()
         bd = b_nat[order][:cols].contiguous().cuda() if bias else None
