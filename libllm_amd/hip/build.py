@@ -6,6 +6,7 @@ decides whether what is built is current.  Nothing here falls back to another im
 the library cannot be loaded or built, KernelError says why.
 """
 import ctypes
+import fcntl
 import hashlib
 import json
 import os
@@ -129,6 +130,20 @@ def build(force: bool = True, verbose: bool = True) -> str:
     target = next((d for d in _lib_dirs() if _writable(d)), None)
     if target is None:
         raise KernelError("no writable folder for the kernel library (tried %s)" % ", ".join(_lib_dirs()))
+    # one build at a time in a folder: a second process waits, and takes what the first has built
+    with open(os.path.join(target, ".build.lock"), "w") as lock:
+        try:
+            fcntl.flock(lock, fcntl.LOCK_EX | fcntl.LOCK_NB)
+        except OSError:
+            if verbose:
+                _say("another process is building the kernels in %s: waiting for it" % target)
+            fcntl.flock(lock, fcntl.LOCK_EX)
+        if not force and _current(target, want):
+            return os.path.join(target, LIB_NAME)
+        return _build_into(target, hipcc, want, verbose)
+
+
+def _build_into(target: str, hipcc: str, want: str, verbose: bool) -> str:
     objdir = os.path.join(target, "obj")
     os.makedirs(objdir, exist_ok=True)
     srcs = sources()

@@ -63,3 +63,36 @@ def test_the_build_records_that_the_product_for_33_to_128_rows_spills_no_registe
     found["no_spill"] = {}
     (other / build.INFO_NAME).write_text(json.dumps(found))
     assert not build.trusted("gemm_mid.hip", str(other / build.LIB_NAME))
+
+
+def test_two_processes_that_find_nothing_built_build_once(tmp_path, monkeypatch):
+    """Two callers that find no library at the same moment (two programs started together in a
+    fresh checkout): one compiles, the other waits for it and takes what it built, instead of
+    both writing the same object files."""
+    import json
+    import threading
+    import time
+    from libllm_amd.hip import build
+    target = str(tmp_path / "lib")
+    calls = []
+
+    def slow_build(folder, hipcc, want, verbose):
+        calls.append(folder)
+        time.sleep(0.4)
+        for name, text in ((build.LIB_NAME, ""), (build.INFO_NAME, json.dumps({"hash": want})),
+                           (build.LIB_NAME + ".hash", want)):
+            with open(os.path.join(folder, name), "w") as f:
+                f.write(text)
+        return os.path.join(folder, build.LIB_NAME)
+
+    monkeypatch.setattr(build, "_lib_dirs", lambda: [target])
+    monkeypatch.setattr(build, "_hipcc", lambda: "/bin/true")
+    monkeypatch.setattr(build, "_build_into", slow_build)
+    got = []
+    threads = [threading.Thread(target=lambda: got.append(build.build(force=False, verbose=False))) for _ in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert got == [os.path.join(target, build.LIB_NAME)] * 2 and len(calls) == 1
+    assert build.build(force=False, verbose=False) == got[0] and len(calls) == 1      # and it stays built
