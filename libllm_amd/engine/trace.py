@@ -13,7 +13,6 @@ import json
 import os
 import sys
 
-
 from ..errors import RequestError
 from .step import StepEntry
 
