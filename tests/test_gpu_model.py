@@ -278,6 +278,47 @@ def test_random_traces(long_models, tmp_path, case):
     check("long" + name, cfg, weights, requests, traces.collect(steps, str(tmp_path), cfg.vocab), dtype)
 
 
+def drawn_config(rng):
+    """A tiny configuration with every size and option drawn: 1 to 5 kv heads with 1 to 8 query
+    heads each, head sizes of 16 to 128, widths and feed-forwards in multiples of 8, any
+    vocabulary, the three rotary scalings, biases, tied or untied output, either eps."""
+    n_kv = int(rng.choice([1, 2, 3, 4, 5]))
+    scaling = [None, {"rope_type": "linear", "factor": float(rng.choice([2.0, 4.0]))},
+               {"rope_type": "llama3", "factor": float(rng.choice([8.0, 32.0])), "low_freq_factor": 1.0,
+                "high_freq_factor": 4.0,
+                "original_max_position_embeddings": int(rng.choice([32, 64, 128]))}][int(rng.integers(0, 3))]
+    return {"model_type": "llama", "num_hidden_layers": int(rng.integers(1, 4)),
+            "hidden_size": 8 * int(rng.integers(4, 48)), "num_attention_heads": n_kv * int(rng.choice([1, 2, 3, 4, 8])),
+            "num_key_value_heads": n_kv, "head_dim": int(rng.choice([16, 32, 48, 64, 80, 96, 112, 128])),
+            "intermediate_size": 8 * int(rng.integers(6, 90)), "vocab_size": int(rng.integers(64, 3000)),
+            "rope_theta": float(rng.choice([10000.0, 500000.0])), "rope_scaling": scaling,
+            "rms_norm_eps": float(rng.choice([1e-5, 1e-6])), "tie_word_embeddings": bool(rng.integers(0, 2)),
+            "max_position_embeddings": 256, "attention_bias": bool(rng.integers(0, 2)), "hidden_act": "silu",
+            "eos_token_id": 2}
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_drawn_configurations(tmp_path, seed):
+    """Configurations drawn at random (see drawn_config) with requests of drawn lengths: whole,
+    with the last tokens one by one, and in two batches, in both dtypes, every position against
+    the plain implementation."""
+    rng = np.random.default_rng(7000 + seed)
+    name = "drawn%d" % seed
+    path = make_model(tmp_path, drawn_config(rng), seed=seed, name=name)
+    cfg_json, weights = files.read_model_dir(path)
+    cfg = llama.PlainConfig(cfg_json)
+    requests = make_requests(cfg, [int(n) for n in rng.integers(1, 150, size=int(rng.integers(3, 8)))], seed=seed)
+    ids = list(requests)
+    half = max(1, len(ids) // 2)
+    groups = [{r: requests[r] for r in ids[:half]}, {r: requests[r] for r in ids[half:]}]
+    for dtype in DTYPES:
+        for mode, steps in (("whole", traces.whole(requests)), ("tail", traces.tail_one_by_one(requests)),
+                            ("batches", traces.batches(groups))):
+            out_dir = tmp_path / (dtype + mode)
+            run_replay(path, dtype, steps, out_dir)
+            check(name, cfg, weights, requests, traces.collect(steps, str(out_dir), cfg.vocab), dtype)
+
+
 @pytest.mark.parametrize("case", range(6))
 def test_batches_of_more_than_128_requests(long_models, tmp_path, case):
     """160 to 250 short requests start together and decode a few tokens each, the shorter ones
