@@ -12,7 +12,8 @@
 #include "no_alloc.h"
 
 __device__ __forceinline__ uint32_t order_key(float x) {
-  const uint32_t u = __float_as_uint(x);
+  uint32_t u = __float_as_uint(x);
+  if (u == 0x80000000u) u = 0u;                          // -0 and +0 are one value: ties go by index
   return (u & 0x80000000u) ? ~u : (u | 0x80000000u);     // larger float -> larger key
 }
 

@@ -1350,6 +1350,24 @@ def test_sampling_with_many_equal_logits(ops):
         assert bad <= 2, (vocab, bad)
 
 
+def test_sampling_takes_both_zeros_for_one_value(ops):
+    """Logits of -0.0 and +0.0 are equal: among equal logits the lower index comes first, whatever
+    the sign of a zero (a kernel that orders by the bits of the float puts every +0 before every -0)."""
+    from plain import sampling
+    g = torch.Generator().manual_seed(11)
+    for vocab, top_k, top_p, temp in [(300, 50, 0.95, 1.6), (188, 0, 0.8, 0.7), (2007, 1000, 0.8, 0.7), (260, 200, 0.95, 0.3),
+                                      (5000, 0, 1.0, 1.0)]:
+        logits = torch.round(torch.randn((32, vocab), generator=g) * 0.5)       # -1, -0.0, 0.0, 1 for the most part
+        assert (logits == 0).sum() > vocab and torch.signbit(logits[logits == 0]).any() and not torch.signbit(logits[logits == 0]).all()
+        streams, counters = list(range(32)), list(range(200, 232))
+        got = ops.sample(logits.cuda(), temp, top_k, top_p, 21, streams, counters).tolist()
+        for r in range(32):
+            u = sampling.uniform(21, streams[r], counters[r])
+            want = sampling.sample(logits[r].double().numpy(), temp, top_k, top_p, u)
+            if got[r] != want:
+                assert sampling.margin(logits[r].double().numpy(), temp, top_k, top_p, u) < 1e-5, (vocab, r, got[r], want)
+
+
 @pytest.mark.parametrize("vocab", [5003, 128256])
 def test_nucleus_without_a_limit_on_the_candidates(ops, vocab):
     """top_k 0 with top_p below 1 (the reference's sampler takes any top_k up to the vocabulary,
