@@ -116,6 +116,31 @@ def test_generation_of_drawn_requests_matches_plain(models, seed):
         assert not model.engine.live_requests()
 
 
+def test_completions_taken_in_turns_and_one_left_unfinished(models):
+    """Two completions of one model whose chunks are taken in turns give what each gives alone
+    (each holds a slot of the cache of its own), and one that is dropped half way gives its slot
+    and pages back."""
+    import gc
+    path, cfg, weights = models["B"]
+    model = Model(path, dtype="float32", max_tokens=1024, ops=CpuOps())
+    prompts = ([21, 500, 13, 640, 15, 77], [100, 200, 300])
+    alone = [sampling.generate(cfg, weights, p, 8) for p in prompts]
+    assert all(len(a) > 2 for a in alone)
+    turns = [iter(model.complete(p, temperature=0.0, max_new_tokens=8)) for p in prompts]
+    got = [[], []]
+    for _ in range(10):
+        for it, out in zip(turns, got):
+            out.extend(c.token_id for c in [next(it, None)] if c is not None and c.token_id is not None)
+    assert got == alone
+    dropped = iter(model.complete(prompts[0], temperature=0.0, max_new_tokens=8))
+    next(dropped)
+    assert model.engine.live_requests()
+    del dropped
+    gc.collect()
+    model.engine.cache.check()
+    assert not model.engine.live_requests() and model.engine.cache.slots.n_free == model.engine.cache.slots.n_slots
+
+
 def test_messages_become_the_architectures_chat_format(models, tmp_path):
     """The messages of a chat, block by block as the reference's model class appends them
     (src/libllm/llama.cc:406-442), where the tokenizer beside the model knows the control tokens;
