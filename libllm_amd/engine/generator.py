@@ -11,7 +11,7 @@ from typing import Callable, Iterable, List, Optional, Sequence
 
 import torch
 
-from ..errors import RequestError
+from ..errors import CacheError, RequestError
 from ..sampling import SamplingParams
 from .step import StepEntry
 
@@ -145,7 +145,23 @@ class Generator:
         lens = [len(p) for p in prompts]
         batches = plan_batches(lens, max_new_tokens, self.max_batch, self.page_budget, self.page,
                                self.max_position)
-        for batch in batches:
+        room = getattr(self.engine, "room", None)
+        todo = [i for batch in batches for i in batch]
+        while todo:
+            # The plan above holds where the whole cache is free (and refuses what can never fit).
+            # Other requests may hold a part of it (a completion that its caller has not
+            # finished): each batch is cut, by the same rule, to what is free when it starts.
+            slots, pages = room() if room is not None else (self.max_batch, self.page_budget)
+            if slots <= 0:
+                raise CacheError("no free slot: other requests hold every slot of the cache")
+            head = todo[:self.max_batch]
+            try:
+                first = plan_batches([lens[i] for i in head], max_new_tokens, min(self.max_batch, slots),
+                                     min(self.page_budget, pages), self.page, self.max_position)[0]
+            except RequestError:
+                raise CacheError("the cache is full: request %d needs more pages than the %d that other "
+                                 "requests leave free" % (todo[0], pages)) from None
+            batch, todo = head[:len(first)], todo[len(first):]
             yield from self._run_batch(batch, prompts, params, max_new_tokens, stop)
 
     def _run_batch(self, batch, prompts, params, max_new_tokens, stop):

@@ -81,6 +81,11 @@ class Engine:
     def live_requests(self):
         return self.cache.slots.live()
 
+    def room(self):
+        """(free slots, free pages): what requests that start now can take; the pages of the
+        group of layers that has the fewest left."""
+        return self.cache.slots.n_free, min(g.pool.n_free for g in self.cache.groups)
+
     def end(self, requests) -> None:
         for r in requests:
             self.cache.release(r)

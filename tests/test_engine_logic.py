@@ -141,6 +141,37 @@ def test_completions_taken_in_turns_and_one_left_unfinished(models):
     assert not model.engine.live_requests() and model.engine.cache.slots.n_free == model.engine.cache.slots.n_slots
 
 
+def test_generation_beside_an_unfinished_completion(models):
+    """A completion that its caller has not finished holds a slot and pages of the cache: the
+    generation loop cuts its batches to what is free when each starts (here one batch of four
+    becomes two), and the completion goes on afterwards as if nothing had happened."""
+    path, cfg, weights = models["B"]
+    model = Model(path, dtype="float32", max_tokens=256, ops=CpuOps())
+    rng = np.random.default_rng(0)
+    prompts = [rng.integers(10, cfg.vocab, size=n).tolist() for n in (60, 50, 40, 30)]
+    want = [sampling.generate(cfg, weights, p, 4) for p in prompts]
+    assert model.generate(prompts, max_new_tokens=4, temperature=0.0) == want
+    first = model._generator._serial
+    long_prompt = [21, 500, 13, 640, 15, 77] * 10
+    reply = sampling.generate(cfg, weights, long_prompt, 6)
+    assert len(reply) == 6
+    held = iter(model.complete(long_prompt, temperature=0.0, max_new_tokens=6))
+    got = [next(held).token_id]
+    assert model.generate(prompts, max_new_tokens=4, temperature=0.0) == want
+    assert model._generator._serial - first > 2            # the completion's batch, and more than one for the four
+    got += [c.token_id for c in held if c.token_id is not None]
+    assert got == reply
+    model.engine.cache.check()
+    assert model.engine.cache.slots.n_free == model.engine.cache.slots.n_slots
+    # nothing free at all is an error that says so
+    from libllm_amd.engine import StepEntry
+    for i in range(model.engine.cache.slots.n_slots):
+        model.engine.step([StepEntry(("held", i), [1], [])])
+    with pytest.raises(CacheError, match="other requests hold"):
+        model.generate(prompts[:1], max_new_tokens=2, temperature=0.0)
+    model.engine.end([("held", i) for i in range(model.engine.cache.slots.n_slots)])
+
+
 def test_messages_become_the_architectures_chat_format(models, tmp_path):
     """The messages of a chat, block by block as the reference's model class appends them
     (src/libllm/llama.cc:406-442), where the tokenizer beside the model knows the control tokens;
