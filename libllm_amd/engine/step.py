@@ -126,7 +126,13 @@ class Engine:
             seen.add(e.request)
             if len(e.tokens) == 0:
                 raise RequestError("request %r brings no tokens" % (e.request,))
-            lo, hi = min(e.tokens), max(e.tokens)
+            if len(e.tokens) == 1 and type(e.tokens[0]) is int:          # a decode step's entry
+                lo = hi = e.tokens[0]
+            else:
+                ids = np.asarray(e.tokens)
+                if ids.ndim != 1 or ids.dtype.kind not in "iu":
+                    raise RequestError("request %r: token ids are a flat list of integers" % (e.request,))
+                lo, hi = int(ids.min()), int(ids.max())
             if tokens_device is None and (lo < 0 or hi >= self.vocab):
                 raise RequestError("request %r has a token id outside [0, %d)" % (e.request, self.vocab))
             for w in e.want:

@@ -58,7 +58,8 @@ def test_step_refuses_bad_requests(models):
     path, cfg, _ = models["A"]
     engine = load_engine(path, dtype="float32", max_tokens=128, ops=CpuOps())
     for bad in ([], [StepEntry("a", [], [])], [StepEntry("a", [1], [1])], [StepEntry("a", [cfg.vocab], [])],
-                [StepEntry("a", [-1], [])], [StepEntry("a", [1], []), StepEntry("a", [2], [])]):
+                [StepEntry("a", [-1], [])], [StepEntry("a", [1], []), StepEntry("a", [2], [])],
+                [StepEntry("a", [1, 2.5], [])], [StepEntry("a", [[1, 2]], [])], [StepEntry("a", ["1"], [])]):
         with pytest.raises(RequestError):
             engine.step(bad)
     assert not engine.live_requests()
